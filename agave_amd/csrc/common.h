@@ -1,0 +1,103 @@
+// Shared device helpers for the gfx950 kernels: element types, wave64 reductions,
+// error reporting to the host.  Everything is compiled for MI355X only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define AGAVE_WAVE 64
+#define AGAVE_PAGE 64          // positions per cache page
+
+// dtype codes shared with the Python side
+#define AGAVE_F32 0
+#define AGAVE_BF16 1
+
+// ---------------------------------------------------------------- error reporting
+// Every entry point returns 0 or a negative code and leaves a message here.
+extern "C" const char* agave_last_error();
+void agave_set_error(const char* fmt, ...);
+
+#define AGAVE_CHECK(cond, ...)                      \
+    do {                                            \
+        if (!(cond)) {                              \
+            agave_set_error(__VA_ARGS__);           \
+            return -1;                              \
+        }                                           \
+    } while (0)
+
+#define AGAVE_LAUNCH_CHECK(name)                                                   \
+    do {                                                                           \
+        hipError_t e__ = hipGetLastError();                                        \
+        if (e__ != hipSuccess) {                                                   \
+            agave_set_error("%s: launch failed: %s", name, hipGetErrorString(e__)); \
+            return -2;                                                             \
+        }                                                                          \
+    } while (0)
+
+// ---------------------------------------------------------------- bfloat16
+struct bf16 {
+    uint16_t x;
+};
+
+__host__ __device__ __forceinline__ float bf16_to_f32(bf16 v) {
+    union { uint32_t u; float f; } c;
+    c.u = ((uint32_t)v.x) << 16;
+    return c.f;
+}
+
+// round to nearest, ties to even; NaN stays NaN
+__host__ __device__ __forceinline__ bf16 f32_to_bf16(float f) {
+    union { uint32_t u; float f; } c;
+    c.f = f;
+    bf16 r;
+    if ((c.u & 0x7fffffffu) > 0x7f800000u) {
+        r.x = 0x7fc0;
+        return r;
+    }
+    c.u += 0x7fffu + ((c.u >> 16) & 1u);
+    r.x = (uint16_t)(c.u >> 16);
+    return r;
+}
+
+template <typename T> __device__ __forceinline__ float ld(const T* p);
+template <> __device__ __forceinline__ float ld<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float ld<bf16>(const bf16* p) { return bf16_to_f32(*p); }
+
+template <typename T> __device__ __forceinline__ void st(T* p, float v);
+template <> __device__ __forceinline__ void st<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void st<bf16>(bf16* p, float v) { *p = f32_to_bf16(v); }
+
+// ---------------------------------------------------------------- wave64 reductions
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Block-wide reductions for blocks of up to 1024 threads; `red` is 16 floats of LDS.
+// Every thread gets the result.  Contains barriers: call from all threads.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_sum(v);
+    __syncthreads();
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float r = 0.f;
+    for (int i = 0; i < nw; ++i) r += red[i];
+    return r;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    v = wave_max(v);
+    __syncthreads();
+    if (lane == 0) red[w] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int i = 1; i < nw; ++i) r = fmaxf(r, red[i]);
+    return r;
+}

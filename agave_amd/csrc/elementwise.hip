@@ -1,0 +1,275 @@
+// Row-wise kernels of the decoder for gfx950: embedding with scale, RMSNorm with the
+// residual sum, per-head q/k norm + rotation + cache write, GeGLU, casts.
+//
+// The residual stream is always 32-bit; activations (T) are float or bf16.  Norm sums,
+// rotation angles and the residual sum are computed in 32-bit in both cases.
+// Reference formulas: src/backend/kernels/cpu/norm.zig:7-40 (x * 1/sqrt(mean x^2 + eps) * g),
+// src/backend/kernels/cpu/rope.zig:11-48 (split-half pairs), src/models/gemma3.zig:884-902
+// (position scaled before the angle), src/backend/kernels/cpu/activation.zig:69-113 (tanh GELU).
+#include "common_impl.h"
+
+// ------------------------------------------------------------------ embedding
+template <typename T>
+__global__ void embed_scale_kernel(const int* __restrict__ tokens, const T* __restrict__ table,
+                                   float scale, float* __restrict__ out, int e, int vocab) {
+    const int t = blockIdx.x;
+    int tok = tokens[t];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);   // the host rejects such ids; never read outside
+    const T* row = table + (size_t)tok * e;
+    float* o = out + (size_t)t * e;
+    for (int i = threadIdx.x; i < e; i += blockDim.x) o[i] = ld(row + i) * scale;
+}
+
+extern "C" int agave_embed_scale(int dtype, const int* tokens, const void* table, float scale,
+                                 float* out, int n_tokens, int e, int vocab, hipStream_t stream) {
+    AGAVE_CHECK(n_tokens >= 0 && e > 0 && vocab > 0, "embed_scale: bad sizes N=%d e=%d vocab=%d", n_tokens, e, vocab);
+    if (n_tokens == 0) return 0;
+    const int threads = e >= 1024 ? 256 : (e >= 256 ? 128 : 64);
+    if (dtype == AGAVE_F32)
+        embed_scale_kernel<float><<<n_tokens, threads, 0, stream>>>(tokens, (const float*)table, scale, out, e, vocab);
+    else if (dtype == AGAVE_BF16)
+        embed_scale_kernel<bf16><<<n_tokens, threads, 0, stream>>>(tokens, (const bf16*)table, scale, out, e, vocab);
+    else
+        AGAVE_CHECK(false, "embed_scale: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("embed_scale");
+    return 0;
+}
+
+// ------------------------------------------------------------------ residual + norms
+//   r = rows ? rows[i] : i                       (row of h and of branch)
+//   if branch: h[r] += post_gain ? rmsnorm(branch[r]) * post_gain : branch[r]
+//   if out:    out[i] = rmsnorm(h[r]) * pre_gain
+// Gains are 32-bit and already hold the "+1" where the architecture has it.
+template <typename T>
+__global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb,
+                                     const float* __restrict__ post_gain, float post_eps,
+                                     T* __restrict__ out, long ldo, const float* __restrict__ pre_gain,
+                                     float pre_eps, const int* __restrict__ rows, int e) {
+    __shared__ float red[16];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    float* hr = h + (size_t)r * e;
+    float ss_h = 0.f;
+    if (branch) {
+        const T* br = branch + (size_t)r * ldb;
+        float inv = 1.0f;
+        if (post_gain) {
+            float ss = 0.f;
+            for (int c = threadIdx.x; c < e; c += blockDim.x) {
+                const float v = ld(br + c);
+                ss += v * v;
+            }
+            ss = block_sum(ss, red);
+            inv = 1.0f / sqrtf(ss / (float)e + post_eps);
+        }
+        for (int c = threadIdx.x; c < e; c += blockDim.x) {
+            const float y = post_gain ? ld(br + c) * inv * post_gain[c] : ld(br + c);
+            const float hv = hr[c] + y;
+            hr[c] = hv;
+            ss_h += hv * hv;
+        }
+    } else if (out) {
+        for (int c = threadIdx.x; c < e; c += blockDim.x) {
+            const float hv = hr[c];
+            ss_h += hv * hv;
+        }
+    }
+    if (out) {
+        ss_h = block_sum(ss_h, red);
+        const float inv = 1.0f / sqrtf(ss_h / (float)e + pre_eps);
+        T* o = out + (size_t)i * ldo;
+        for (int c = threadIdx.x; c < e; c += blockDim.x) st(o + c, hr[c] * inv * pre_gain[c]);
+    }
+}
+
+extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long ldb, const float* post_gain,
+                                   float post_eps, void* out, long ldo, const float* pre_gain, float pre_eps,
+                                   const int* rows, int n_rows, int e, hipStream_t stream) {
+    AGAVE_CHECK(n_rows >= 0 && e > 0, "residual_norm: bad sizes rows=%d e=%d", n_rows, e);
+    AGAVE_CHECK(h != nullptr, "residual_norm: residual stream is null");
+    AGAVE_CHECK(!out || pre_gain, "residual_norm: output without its gain");
+    AGAVE_CHECK(!branch || ldb >= e, "residual_norm: branch row stride %ld < %d", ldb, e);
+    AGAVE_CHECK(!out || ldo >= e, "residual_norm: output row stride %ld < %d", ldo, e);
+    AGAVE_CHECK(!(rows && branch), "residual_norm: row gather with a branch is not supported");
+    if (n_rows == 0 || (!branch && !out)) return 0;
+    const int threads = e >= 2048 ? 512 : (e >= 512 ? 256 : 64);
+    if (dtype == AGAVE_F32)
+        residual_norm_kernel<float><<<n_rows, threads, 0, stream>>>(h, (const float*)branch, ldb, post_gain, post_eps,
+                                                                    (float*)out, ldo, pre_gain, pre_eps, rows, e);
+    else if (dtype == AGAVE_BF16)
+        residual_norm_kernel<bf16><<<n_rows, threads, 0, stream>>>(h, (const bf16*)branch, ldb, post_gain, post_eps,
+                                                                   (bf16*)out, ldo, pre_gain, pre_eps, rows, e);
+    else
+        AGAVE_CHECK(false, "residual_norm: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("residual_norm");
+    return 0;
+}
+
+// ------------------------------------------------------------------ q/k head norm + rotation + cache write
+// One wave per (token, head); q heads first, then k heads.  A k-head wave also stores the
+// matching v head.  Cache pages: K [page][kv head][64 rows][hd], V transposed
+// [page][kv head][hd][64 rows]; position p of sequence b lies in page
+// table[b][p/64 - base[b]], row p % 64.
+#define QK_HD_MAX 512
+template <typename T>
+__global__ void qk_norm_rope_kv_kernel(const T* q, long ldq, const T* __restrict__ k, long ldk,
+                                       const T* __restrict__ v, long ldv, T* q_out, long ldqo,
+                                       const float* __restrict__ q_gain, const float* __restrict__ k_gain,
+                                       float eps_q, float eps_k, const float* __restrict__ inv_freq,
+                                       int rot_half, float pos_scale, const int* __restrict__ tok_seq,
+                                       const int* __restrict__ tok_pos, T* __restrict__ k_pages,
+                                       T* __restrict__ v_pages, const int* __restrict__ table, int width,
+                                       const int* __restrict__ base, int n_pages, int N, int nh, int nkv, int hd) {
+    __shared__ float buf[4][QK_HD_MAX];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int heads = nh + nkv;
+    const long unit = (long)blockIdx.x * 4 + wave;
+    const bool active = unit < (long)N * heads;
+    const int t = active ? (int)(unit / heads) : 0;
+    const int hh = active ? (int)(unit % heads) : 0;
+    const bool is_q = hh < nh;
+    const int head = is_q ? hh : hh - nh;
+    const T* src = is_q ? q + (size_t)t * ldq + (size_t)head * hd : k + (size_t)t * ldk + (size_t)head * hd;
+    const float* gain = is_q ? q_gain : k_gain;
+    const float eps = is_q ? eps_q : eps_k;
+    float* y = buf[wave];
+
+    float ss = 0.f;
+    if (active)
+        for (int d = lane; d < hd; d += 64) {
+            const float x = ld(src + d);
+            y[d] = x;
+            ss += x * x;
+        }
+    if (active && gain) {
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+        for (int d = lane; d < hd; d += 64) y[d] = y[d] * inv * gain[d];
+    }
+    __syncthreads();
+    if (!active) return;
+
+    const int p = tok_pos[t];
+    T* dst;
+    long pg = -1;
+    int row = 0;
+    if (is_q) {
+        dst = q_out + (size_t)t * ldqo + (size_t)head * hd;
+    } else {
+        const int b = tok_seq[t];
+        const int col = p / AGAVE_PAGE - base[b];
+        row = p % AGAVE_PAGE;
+        if (col >= 0 && col < width) pg = table[(size_t)b * width + col];
+        if (pg < 0 || pg >= n_pages) return;   // a table the host built wrongly: write nothing
+        dst = k_pages + (((size_t)pg * nkv + head) * AGAVE_PAGE + row) * hd;
+    }
+    const float pf = (float)p * pos_scale;
+    for (int i = lane; i < rot_half; i += 64) {
+        const float a = y[i], b2 = y[i + rot_half];
+        float s, c;
+        sincosf(pf * inv_freq[i], &s, &c);
+        st(dst + i, a * c - b2 * s);
+        st(dst + i + rot_half, a * s + b2 * c);
+    }
+    for (int d = 2 * rot_half + lane; d < hd; d += 64) st(dst + d, y[d]);
+    if (!is_q) {
+        const T* sv = v + (size_t)t * ldv + (size_t)head * hd;
+        T* dv = v_pages + ((size_t)pg * nkv + head) * hd * AGAVE_PAGE + row;
+        for (int d = lane; d < hd; d += 64) dv[(size_t)d * AGAVE_PAGE] = sv[d];
+    }
+}
+
+extern "C" int agave_qk_norm_rope_kv(int dtype, const void* q, long ldq, const void* k, long ldk, const void* v,
+                                     long ldv, void* q_out, long ldqo, const float* q_gain, const float* k_gain,
+                                     float eps_q, float eps_k, const float* inv_freq, int rot_half, float pos_scale,
+                                     const int* tok_seq, const int* tok_pos, void* k_pages, void* v_pages,
+                                     const int* table, int width, const int* base, int n_pages, int N, int nh,
+                                     int nkv, int hd, hipStream_t stream) {
+    AGAVE_CHECK(N >= 0 && nh >= 0 && nkv >= 0 && hd > 0, "qk_norm_rope_kv: bad sizes N=%d nh=%d nkv=%d hd=%d", N, nh, nkv, hd);
+    AGAVE_CHECK(hd <= QK_HD_MAX, "qk_norm_rope_kv: head_dim %d exceeds the supported maximum %d", hd, QK_HD_MAX);
+    AGAVE_CHECK(rot_half >= 0 && 2 * rot_half <= hd, "qk_norm_rope_kv: rotary_dim %d exceeds head_dim %d", 2 * rot_half, hd);
+    AGAVE_CHECK(rot_half == 0 || inv_freq, "qk_norm_rope_kv: rotation without a frequency table");
+    AGAVE_CHECK(nh == 0 || (q && q_out && ldq >= (long)nh * hd && ldqo >= (long)nh * hd), "qk_norm_rope_kv: bad q buffers");
+    AGAVE_CHECK(nkv == 0 || (k && v && k_pages && v_pages && table && base && tok_seq && width > 0 && n_pages > 0 &&
+                             ldk >= (long)nkv * hd && ldv >= (long)nkv * hd),
+                "qk_norm_rope_kv: bad k/v buffers or cache table");
+    AGAVE_CHECK(tok_pos != nullptr, "qk_norm_rope_kv: positions are null");
+    const long units = (long)N * (nh + nkv);
+    if (units == 0) return 0;
+    const int blocks = (int)((units + 3) / 4);
+    if (dtype == AGAVE_F32)
+        qk_norm_rope_kv_kernel<float><<<blocks, 256, 0, stream>>>(
+            (const float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv, (float*)q_out, ldqo, q_gain, k_gain,
+            eps_q, eps_k, inv_freq, rot_half, pos_scale, tok_seq, tok_pos, (float*)k_pages, (float*)v_pages, table,
+            width, base, n_pages, N, nh, nkv, hd);
+    else if (dtype == AGAVE_BF16)
+        qk_norm_rope_kv_kernel<bf16><<<blocks, 256, 0, stream>>>(
+            (const bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv, (bf16*)q_out, ldqo, q_gain, k_gain, eps_q,
+            eps_k, inv_freq, rot_half, pos_scale, tok_seq, tok_pos, (bf16*)k_pages, (bf16*)v_pages, table, width,
+            base, n_pages, N, nh, nkv, hd);
+    else
+        AGAVE_CHECK(false, "qk_norm_rope_kv: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("qk_norm_rope_kv");
+    return 0;
+}
+
+// ------------------------------------------------------------------ GeGLU
+__device__ __forceinline__ float gelu_tanh(float x) {
+    const float c = 0.7978845608028654f;
+    return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
+}
+
+template <typename T>
+__global__ void geglu_kernel(const T* __restrict__ gate, long ldg, const T* __restrict__ up, long ldu,
+                             T* __restrict__ out, long ldo, long total, int ff) {
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / ff;
+        const int c = (int)(idx % ff);
+        const float g = ld(gate + r * ldg + c), u = ld(up + r * ldu + c);
+        st(out + r * ldo + c, gelu_tanh(g) * u);
+    }
+}
+
+extern "C" int agave_geglu(int dtype, const void* gate, long ldg, const void* up, long ldu, void* out, long ldo,
+                           int n_rows, int ff, hipStream_t stream) {
+    AGAVE_CHECK(n_rows >= 0 && ff > 0, "geglu: bad sizes rows=%d ff=%d", n_rows, ff);
+    AGAVE_CHECK(ldg >= ff && ldu >= ff && ldo >= ff, "geglu: a row stride is below %d", ff);
+    if (n_rows == 0) return 0;
+    const long total = (long)n_rows * ff;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == AGAVE_F32)
+        geglu_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)gate, ldg, (const float*)up, ldu, (float*)out, ldo, total, ff);
+    else if (dtype == AGAVE_BF16)
+        geglu_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)gate, ldg, (const bf16*)up, ldu, (bf16*)out, ldo, total, ff);
+    else
+        AGAVE_CHECK(false, "geglu: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("geglu");
+    return 0;
+}
+
+// ------------------------------------------------------------------ casts
+template <typename TI, typename TO>
+__global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, long n) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x)
+        st(out + i, ld(in + i));
+}
+
+extern "C" int agave_cast(int dtype_in, const void* in, int dtype_out, void* out, long n, hipStream_t stream) {
+    AGAVE_CHECK(n >= 0, "cast: negative count");
+    if (n == 0) return 0;
+    long blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype_in == AGAVE_F32 && dtype_out == AGAVE_BF16)
+        cast_kernel<float, bf16><<<(int)blocks, 256, 0, stream>>>((const float*)in, (bf16*)out, n);
+    else if (dtype_in == AGAVE_BF16 && dtype_out == AGAVE_F32)
+        cast_kernel<bf16, float><<<(int)blocks, 256, 0, stream>>>((const bf16*)in, (float*)out, n);
+    else if (dtype_in == AGAVE_F32 && dtype_out == AGAVE_F32)
+        cast_kernel<float, float><<<(int)blocks, 256, 0, stream>>>((const float*)in, (float*)out, n);
+    else if (dtype_in == AGAVE_BF16 && dtype_out == AGAVE_BF16)
+        cast_kernel<bf16, bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)in, (bf16*)out, n);
+    else
+        AGAVE_CHECK(false, "cast: unknown dtypes %d -> %d", dtype_in, dtype_out);
+    AGAVE_LAUNCH_CHECK("cast");
+    return 0;
+}

@@ -1,0 +1,130 @@
+"""The engine: a model on one GPU with its cache, its step function and generation.
+
+Programmatic surface in the manner of the reference's ``Model`` interface
+(``src/models/model.zig:205-307``: ``forward``, ``prefill``, ``getLogits``, ``resetCache``,
+``eosId``, ``vocabSize``, ``nLayers``, ``kvSeqLen``), for a batch of sequences in slots:
+
+    engine = Engine.from_folder(model_dir, dtype="bfloat16", max_slots=8, max_context=4096)
+    slot = engine.alloc_slot()
+    logits = engine.step([slot], [[2, 17, 5]], want="last")      # float32 [1, vocab] on the GPU
+    engine.free_slot(slot)
+    results = engine.generate(prompts, SamplingParams(temperature=0.8, seed=1))
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..cache import PAGE, GroupKey, KVCache
+from ..config import find_architecture, read_config_json
+from ..config.spec import ModelSpec
+from ..parts import BuildEnv, Workspace
+from ..weights import Checkpoint, DictWeightSource, WeightSource
+from .model import Model, tensor_needs
+from .step import Step, StepPlanner, Want
+
+_DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
+           "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+           torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+def parse_dtype(dtype) -> torch.dtype:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype must be bfloat16 or float32, got {dtype!r}") from None
+
+
+def require_gpu(device=None) -> torch.device:
+    """The MI355X the engine runs on.  There is no CPU path."""
+    if not torch.cuda.is_available():
+        raise RuntimeError("agave_amd needs a GPU: no HIP device is visible (there is no CPU fallback)")
+    dev = torch.device(device if device is not None else "cuda:0")
+    if dev.type != "cuda":
+        raise RuntimeError(f"agave_amd runs on the GPU only, got device {dev}")
+    return dev
+
+
+class Engine:
+    def __init__(self, spec: ModelSpec, weights, *, dtype="bfloat16", max_slots: int = 8,
+                 max_context: Optional[int] = None, cache_tokens: Optional[int] = None,
+                 device=None, config=None):
+        """``max_context``: longest sequence a slot may hold (default: the model's).
+        ``cache_tokens``: positions the cache holds over all live sequences, each counted
+        rounded up to a multiple of 64 (default: ``max_slots * max_context``)."""
+        self.device = require_gpu(device)
+        self.dtype = parse_dtype(dtype)
+        self.spec = spec
+        self.config = config
+        torch.cuda.set_device(self.device)
+        self.workspace = Workspace(self.device)
+        self.env = BuildEnv(self.dtype, self.device, self.workspace)
+        self.model = Model(spec, weights, self.env)
+        self.max_context = int(max_context) if max_context else int(spec.max_context)
+        if self.max_context < 1:
+            raise ValueError("max_context must be positive")
+        per_seq = (self.max_context + PAGE - 1) // PAGE
+        if cache_tokens is None:
+            n_pages = max_slots * per_seq
+        else:
+            n_pages = max(1, (int(cache_tokens) + PAGE - 1) // PAGE)
+        kv_needs = self.model.kv_needs()
+        pages: Dict[GroupKey, int] = {key: n_pages for key in set(kv_needs.values())}
+        self.cache = KVCache(kv_needs, self.model.state_needs(), max_slots, pages, self.dtype, self.device,
+                             self.max_context)
+        self.planner = StepPlanner(self.cache, spec.vocab_size, self.device)
+
+    # ------------------------------------------------------------------ construction
+    @classmethod
+    def from_folder(cls, model_dir: str, **kw) -> "Engine":
+        """A folder with config.json and safetensors; the model class is chosen by config.json."""
+        raw = read_config_json(model_dir)
+        arch = find_architecture(raw)
+        cfg = arch.parse(raw)
+        ckpt = Checkpoint(model_dir)
+        spec = arch.spec(cfg, ckpt.names())
+        weights = WeightSource(ckpt, tensor_needs(spec))
+        return cls(spec, weights, config=cfg, **kw)
+
+    @classmethod
+    def from_tensors(cls, raw_config: dict, tensors: Dict[str, torch.Tensor], **kw) -> "Engine":
+        arch = find_architecture(raw_config)
+        cfg = arch.parse(raw_config)
+        spec = arch.spec(cfg, tensors.keys())
+        return cls(spec, DictWeightSource(tensors, tensor_needs(spec)), config=cfg, **kw)
+
+    # ------------------------------------------------------------------ the reference's accessors
+    @property
+    def vocab_size(self) -> int:
+        return self.spec.vocab_size
+
+    @property
+    def n_layers(self) -> int:
+        return len(self.spec.layers)
+
+    @property
+    def eos_ids(self):
+        return tuple(self.spec.eos_token_ids)
+
+    def kv_seq_len(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ------------------------------------------------------------------ slots and steps
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def step(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want = "last") -> Optional[torch.Tensor]:
+        """Run ``tokens[i]`` as the next tokens of the sequence in ``slots[i]``.  Returns the
+        float32 logits [wanted, vocab] on the GPU in the order of the sequences and of their
+        wanted places (valid until the next step), or None if nothing is wanted."""
+        step = self.planner.plan(slots, tokens, want)
+        logits = self.model.forward(step)
+        self.planner.commit(step)
+        return logits
+
+    def synchronize(self) -> None:
+        torch.cuda.synchronize(self.device)

@@ -1,0 +1,129 @@
+"""The model: embedding, the layers in their run order, final norm, output matrix.
+
+It is built from a :class:`ModelSpec` alone, out of registered parts; the same class serves
+every architecture.  Reference for the overall order: embedding scaled by ``embed_scale``
+(``src/models/gemma3.zig:338, 1017-1046``), ``for i in 0..L: attention(i); feedForward(i)``
+(``:341-348``), final norm and output product on the rows whose logits are wanted
+(``:352-359``), the output matrix being the embedding table when none is stored (``:357-358``).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..cache import GroupKey, StateNeed
+from ..config.spec import ModelSpec
+from ..ops import kernels
+from ..parts import BuildEnv, Linear, add_pending_and_norm, lookup
+from ..weights.loader import TensorNeed
+
+
+def tensor_needs(spec: ModelSpec) -> List[TensorNeed]:
+    """Every tensor the model reads, in a fixed order (embedding, layers, final norm, head)."""
+    needs = [TensorNeed(spec.embed_weight, (spec.vocab_size, spec.hidden))]
+    for layer in spec.layers:
+        needs += lookup("block", layer.kind).tensor_needs(layer)
+    if spec.final_norm is not None:
+        needs += lookup("norm", spec.final_norm.kind).tensor_needs(spec.final_norm)
+    if spec.head_weight is not None:
+        needs.append(TensorNeed(spec.head_weight, (spec.vocab_size, spec.hidden)))
+    return needs
+
+
+class Model:
+    def __init__(self, spec: ModelSpec, weights, env: BuildEnv):
+        self.spec = spec
+        self.env = env
+        table = weights.get(spec.embed_weight)
+        if env.dtype == torch.float32 and table.dtype != torch.float32:
+            table = table.to(torch.float32)
+        if table.dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError(f"embedding table has unsupported element type {table.dtype}")
+        self.embed_table = table.to(env.device).contiguous()
+        self.blocks = [lookup("block", layer.kind)(layer, weights, env) for layer in spec.layers]
+        self.final_norm = (lookup("norm", spec.final_norm.kind)(spec.final_norm, weights, env)
+                           if spec.final_norm is not None else None)
+        if spec.head_weight is not None:
+            self.head = Linear([weights.get(spec.head_weight)], env, "lm_head")
+        else:
+            self.head = Linear([self.embed_table], env, "lm_head")      # tied: the same device tensor
+        for entry in spec.order:
+            if not (0 <= entry.layer < len(self.blocks)):
+                raise ValueError(f"run order names layer {entry.layer}, the model has {len(self.blocks)}")
+        writers = {e.memory for e in spec.order if e.writes}
+        for e in spec.order:
+            if not e.writes and e.memory not in writers:
+                raise ValueError(f"run order: memory {e.memory} is read but never written")
+
+    # ------------------------------------------------------------------ what the cache must hold
+    def kv_needs(self) -> Dict[int, GroupKey]:
+        needs: Dict[int, GroupKey] = {}
+        for e in self.spec.order:
+            need = self.blocks[e.layer].mixer.kv_need()
+            if need is None:
+                continue
+            if e.memory in needs and needs[e.memory] != need:
+                raise ValueError(f"memory {e.memory} is shared by mixers with different needs: "
+                                 f"{needs[e.memory]} and {need}")
+            needs[e.memory] = need
+        return needs
+
+    def state_needs(self) -> Dict[int, StateNeed]:
+        needs: Dict[int, StateNeed] = {}
+        for e in self.spec.order:
+            need = self.blocks[e.layer].mixer.state_need()
+            if need is None:
+                continue
+            if e.memory in needs and needs[e.memory] != need:
+                raise ValueError(f"memory {e.memory} is shared by mixers with different state")
+            needs[e.memory] = need
+        return needs
+
+    def weight_bytes(self) -> int:
+        seen, total = set(), 0
+
+        def add(t):
+            nonlocal total
+            if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
+                seen.add(t.data_ptr())
+                total += t.numel() * t.element_size()
+
+        def walk(obj, depth=0):
+            if isinstance(obj, torch.Tensor):
+                add(obj)
+            elif depth < 4 and hasattr(obj, "__dict__"):
+                for v in vars(obj).values():
+                    if isinstance(v, (list, tuple)):
+                        for x in v:
+                            walk(x, depth + 1)
+                    elif isinstance(v, torch.Tensor) or hasattr(v, "__dict__"):
+                        if v is not self.env and not isinstance(v, (BuildEnv,)):
+                            walk(v, depth + 1)
+        add(self.embed_table)
+        for b in self.blocks:
+            walk(b)
+        walk(self.final_norm)
+        walk(self.head)
+        return total
+
+    # ------------------------------------------------------------------ one step
+    def forward(self, step) -> Optional[torch.Tensor]:
+        """Run the step's tokens through the model; float32 logits [wanted, vocab] or None."""
+        ws = self.env.workspace
+        n = step.n_tokens
+        h = ws.get("residual", n, self.spec.hidden, torch.float32)
+        kernels.embed_scale(step.tokens, self.embed_table, self.spec.embed_scale, h)
+        pending = None
+        for entry in self.spec.order:
+            pending = self.blocks[entry.layer].forward(h, pending, step, entry.memory, entry.writes)
+        if step.n_want == 0:
+            return None
+        x = ws.get("final_normed", step.n_want, self.spec.hidden, self.env.dtype)
+        if self.final_norm is not None:
+            add_pending_and_norm(h, pending, self.final_norm, x, rows=step.want_rows)
+        else:
+            raise NotImplementedError("a model without a final norm is not supported")
+        logits = ws.get("logits", step.n_want, self.spec.vocab_size, torch.float32)
+        self.head.forward(x, out=logits)
+        return logits

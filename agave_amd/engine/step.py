@@ -1,0 +1,173 @@
+"""One step: a batch of sequences that start together, with unequal lengths.
+
+The first step of a batch brings every prompt whole, later steps one token per sequence.
+A step runs only the tokens it is given, as one ragged batch (no padding token enters the
+model), from the cache that earlier steps left, and returns the logits at the wanted places.
+
+Reference: the reference has ``forward(one token)`` and ``prefill(one sequence)`` on a single
+sequence (``src/models/gemma3.zig:331-368, 373-411``); positions of a chunk are
+``base + t`` (``:430-432``), and only the last row's logits are computed (``:393-403``).
+The batch, the slots and the choice of wanted rows are this engine's own.
+
+Everything the kernels need to know about the step travels to the device as one block of
+int32: the tokens, for every token its sequence and its position, the wanted rows, and for
+every cache group one row of page ids per sequence with the page index its first column
+stands for.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence, Tuple, Union
+
+import numpy as np
+import torch
+
+from ..cache import KVCache
+
+Want = Union[str, Sequence[Sequence[int]]]
+
+
+class StepError(ValueError):
+    pass
+
+
+@dataclass
+class Step:
+    n_tokens: int
+    n_seqs: int
+    n_want: int
+    slots: List[int]
+    pos0: List[int]                 # length of each sequence before the step
+    n_new: List[int]                # tokens each sequence brings
+    cu: List[int]                   # prefix sums of n_new (host)
+    max_new: int
+    max_len: int                    # longest sequence after the step
+    tokens: torch.Tensor            # int32 [N] (device)
+    tok_seq: torch.Tensor           # int32 [N]: index of the token's sequence in this step
+    tok_pos: torch.Tensor           # int32 [N]: absolute position
+    slots_dev: torch.Tensor         # int32 [B]
+    pos0_dev: torch.Tensor          # int32 [B]
+    cu_dev: torch.Tensor            # int32 [B + 1]
+    want_rows: torch.Tensor         # int32 [n_want]: rows of the step whose logits are wanted
+    tables: List[Tuple[torch.Tensor, torch.Tensor]]   # per cache group: (pages [B, width], base [B])
+    cache: KVCache
+
+    @property
+    def is_decode(self) -> bool:
+        return self.max_new == 1
+
+
+def resolve_want(want: Want, n_new: Sequence[int]) -> List[List[int]]:
+    if isinstance(want, str):
+        if want == "last":
+            return [[n - 1] for n in n_new]
+        if want == "all":
+            return [list(range(n)) for n in n_new]
+        if want == "none":
+            return [[] for _ in n_new]
+        raise StepError(f"want must be 'last', 'all', 'none' or lists of places, got {want!r}")
+    if len(want) != len(n_new):
+        raise StepError(f"want lists {len(want)} sequences, the step has {len(n_new)}")
+    out = []
+    for i, (w, n) in enumerate(zip(want, n_new)):
+        w = [int(x) for x in w]
+        for x in w:
+            if not (0 <= x < n):
+                raise StepError(f"sequence {i}: wanted place {x} is outside its {n} tokens")
+        out.append(w)
+    return out
+
+
+class StepPlanner:
+    """Turns (slots, tokens, want) into a :class:`Step`: checks the request, takes cache
+    pages, and uploads the step's description in one copy."""
+
+    def __init__(self, cache: KVCache, vocab_size: int, device: torch.device):
+        self.cache = cache
+        self.vocab_size = vocab_size
+        self.device = device
+        self._host: Optional[torch.Tensor] = None
+        self._dev: Optional[torch.Tensor] = None
+        self._copied = None          # event: the last upload has left the host buffer
+        self.fixed_width: Optional[List[int]] = None   # table widths pinned for graph capture
+
+    def _buffers(self, n: int) -> None:
+        if self._host is None or self._host.numel() < n:
+            cap = max(n, 4096) if self._host is None else max(n, 2 * self._host.numel())
+            if self._copied is not None:
+                self._copied.synchronize()
+            self._host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+            self._dev = torch.empty(cap, dtype=torch.int32, device=self.device)
+
+    def plan(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want = "last") -> Step:
+        if len(slots) != len(tokens) or len(slots) == 0:
+            raise StepError("a step needs as many token lists as slots, and at least one")
+        n_new = [len(t) for t in tokens]
+        if min(n_new) < 1:
+            raise StepError("every sequence of a step brings at least one token")
+        flat = np.fromiter((int(x) for t in tokens for x in t), dtype=np.int64, count=sum(n_new))
+        if flat.size and (flat.min() < 0 or flat.max() >= self.vocab_size):
+            bad = int(flat[(flat < 0) | (flat >= self.vocab_size)][0])
+            raise StepError(f"token id {bad} is outside the vocabulary of {self.vocab_size}")
+        wanted = resolve_want(want, n_new)
+        pos0, plans = self.cache.plan_step(list(slots), n_new)
+
+        b, n = len(slots), int(flat.size)
+        cu = [0]
+        for x in n_new:
+            cu.append(cu[-1] + x)
+        want_rows = [cu[i] + x for i, w in enumerate(wanted) for x in w]
+        widths = []
+        for gi, p in enumerate(plans):
+            w = max(len(r) for r in p.rows)
+            if self.fixed_width is not None:
+                if w > self.fixed_width[gi]:
+                    raise StepError(f"step needs {w} table columns, the captured width is {self.fixed_width[gi]}")
+                w = self.fixed_width[gi]
+            widths.append(w)
+        total = 3 * n + 3 * b + 1 + len(want_rows) + sum(b + b * w for w in widths)
+        self._buffers(total)
+        if self._copied is not None:
+            self._copied.synchronize()
+        host = self._host.numpy()
+        off = 0
+
+        def put(values, count) -> Tuple[int, int]:
+            nonlocal off
+            host[off:off + count] = values
+            span = (off, off + count)
+            off += count
+            return span
+
+        s_tok = put(flat, n)
+        s_seq = put(np.repeat(np.arange(b, dtype=np.int32), n_new), n)
+        s_pos = put(np.concatenate([np.arange(p, p + k, dtype=np.int32) for p, k in zip(pos0, n_new)]), n)
+        s_slots = put(np.asarray(slots, dtype=np.int32), b)
+        s_pos0 = put(np.asarray(pos0, dtype=np.int32), b)
+        s_cu = put(np.asarray(cu, dtype=np.int32), b + 1)
+        s_want = put(np.asarray(want_rows, dtype=np.int32), len(want_rows))
+        s_tables = []
+        for p, w in zip(plans, widths):
+            s_base = put(np.asarray(p.base, dtype=np.int32), b)
+            tab = np.full((b, w), -1, dtype=np.int32)
+            for i, r in enumerate(p.rows):
+                tab[i, :len(r)] = r
+            s_tables.append((put(tab.reshape(-1), b * w), s_base, w))
+        assert off == total
+        self._dev[:total].copy_(self._host[:total], non_blocking=True)
+        self._copied = torch.cuda.Event()
+        self._copied.record()
+        d = self._dev
+
+        def view(span):
+            return d[span[0]:span[1]]
+
+        return Step(
+            n_tokens=n, n_seqs=b, n_want=len(want_rows), slots=list(slots), pos0=pos0, n_new=n_new, cu=cu,
+            max_new=max(n_new), max_len=max(p + k for p, k in zip(pos0, n_new)),
+            tokens=view(s_tok), tok_seq=view(s_seq), tok_pos=view(s_pos), slots_dev=view(s_slots),
+            pos0_dev=view(s_pos0), cu_dev=view(s_cu), want_rows=view(s_want),
+            tables=[(view(t).view(b, w), view(sb)) for t, sb, w in s_tables], cache=self.cache)
+
+    def commit(self, step: Step) -> None:
+        self.cache.commit_step(step.slots, step.n_new)

@@ -1,0 +1,19 @@
+"""Choosing the matrix-product kernel for a linear layer."""
+from __future__ import annotations
+
+import torch
+
+from . import kernels
+
+
+def linear(x: torch.Tensor, lin, out: torch.Tensor) -> None:
+    """out[N, out_features] = x[N, in_features] @ lin.weight^T."""
+    if x.dim() != 2 or x.shape[1] != lin.in_features:
+        raise ValueError(f"{lin.name}: input is {tuple(x.shape)}, weight takes {lin.in_features} columns")
+    if out.shape != (x.shape[0], lin.out_features):
+        raise ValueError(f"{lin.name}: output is {tuple(out.shape)}, needs {(x.shape[0], lin.out_features)}")
+    if x.dtype == torch.bfloat16 and lin.weight.dtype == torch.bfloat16:
+        from . import gemm_mfma
+        if gemm_mfma.try_linear(x, lin, out):
+            return
+    kernels.gemm_plain(x, lin.weight, out)

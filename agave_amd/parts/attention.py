@@ -1,0 +1,88 @@
+"""Attention as a mixer: grouped-query attention over the paged cache, with optional per-head
+q/k norm, a position encoding, and an optional sliding window.
+
+Order of operations as the reference (``src/models/gemma3.zig:701-828``): q, k, v projections;
+RMSNorm of every q and k head with one gain vector per tensor, before the rotation
+(``:722-729``); rotation (``:732-749``); k and v appended to the cache, then attention over it
+with ``scale`` on the scores (``:795-813``); output projection (``:819-820``).  A query at
+position p sees keys ``max(0, p-W+1) .. p`` on a windowed layer, ``0 .. p`` otherwise.
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from ..cache import GroupKey, StateNeed
+from ..config.spec import AttentionSpec
+from ..ops import attention as attn_ops
+from ..ops import kernels
+from ..weights.loader import TensorNeed
+from .base import BuildEnv, lookup, register
+from .linear import Linear
+
+
+class Attention:
+    def __init__(self, spec: AttentionSpec, weights, env: BuildEnv):
+        if spec.n_heads % spec.n_kv_heads:
+            raise ValueError("query heads must be a multiple of kv heads")
+        self.spec = spec
+        self.env = env
+        self.qd = spec.n_heads * spec.head_dim
+        self.kvd = spec.n_kv_heads * spec.head_dim
+        # q, k and v in one product: rows of the three matrices stacked
+        self.qkv = Linear([weights.get(spec.q_proj), weights.get(spec.k_proj), weights.get(spec.v_proj)], env, "qkv")
+        self.q_only: Optional[Linear] = None       # built on demand for runs that only read a cache
+        self.o = Linear([weights.get(spec.o_proj)], env, "attn_o")
+        self.q_norm = lookup("norm", spec.q_norm.kind)(spec.q_norm, weights, env) if spec.q_norm else None
+        self.k_norm = lookup("norm", spec.k_norm.kind)(spec.k_norm, weights, env) if spec.k_norm else None
+        self.position = lookup("position", spec.position.kind)(spec.position, env)
+
+    @staticmethod
+    def tensor_needs(spec: AttentionSpec) -> List[TensorNeed]:
+        qd, kvd = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim
+        needs = [TensorNeed(spec.q_proj, (qd, spec.hidden)), TensorNeed(spec.k_proj, (kvd, spec.hidden)),
+                 TensorNeed(spec.v_proj, (kvd, spec.hidden)), TensorNeed(spec.o_proj, (spec.hidden, qd))]
+        for n in (spec.q_norm, spec.k_norm):
+            if n is not None:
+                needs += lookup("norm", n.kind).tensor_needs(n)
+        return needs
+
+    def kv_need(self) -> Optional[GroupKey]:
+        return GroupKey(self.spec.window, self.spec.n_kv_heads, self.spec.head_dim)
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, x: torch.Tensor, step, memory: int, writes: bool = True) -> torch.Tensor:
+        s, ws = self.spec, self.env.workspace
+        n = x.shape[0]
+        k_pages, v_pages = step.cache.pages_of(memory)
+        table, base = step.tables[step.cache.group_of_memory[memory]]
+        inv_freq, pos_scale = (None, 1.0)
+        fused = getattr(self.position, "fused_rotation", None)
+        if writes:
+            qkv = self.qkv.forward(x, tag="qkv")
+            q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
+        else:
+            if self.q_only is None:
+                self.q_only = Linear([self.qkv.weight[:self.qd]], self.env, "q_only")
+            q, k, v = self.q_only.forward(x, tag="q_only"), None, None
+        if fused is not None:
+            inv_freq, pos_scale = fused()
+        else:
+            self.position.apply(q, k, step)
+        q_out = ws.get("q_rot", n, self.qd, x.dtype)
+        kernels.qk_norm_rope_kv(
+            q, k, v, q_out,
+            self.q_norm.gain if self.q_norm else None, self.k_norm.gain if self.k_norm else None,
+            self.q_norm.eps if self.q_norm else 0.0, self.k_norm.eps if self.k_norm else 0.0,
+            inv_freq, pos_scale, step.tok_seq, step.tok_pos, k_pages, v_pages, table, base,
+            s.n_heads, s.n_kv_heads, s.head_dim)
+        ctx_out = ws.get("attn_ctx", n, self.qd, x.dtype)
+        attn_ops.attention(q_out, ctx_out, k_pages, v_pages, table, base, step, s.n_heads, s.n_kv_heads,
+                           s.head_dim, s.scale, s.window)
+        return self.o.forward(ctx_out, tag="attn_o")
+
+
+register("mixer", "attention", Attention)

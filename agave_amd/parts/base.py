@@ -1,0 +1,83 @@
+"""What every part of a layer looks like to the model builder, and the part registries.
+
+A part is built from its spec (sizes and constants as plain data) and a weight source; it
+states the tensors it needs before anything is loaded; and it runs on the tokens of one
+step.  No part knows which model it is in: the block arrangement asks the registries for
+the kinds that the layer's spec names.
+
+Interfaces (duck-typed; the classes below document them):
+
+* norm:        ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, fields ``gain`` (float32
+               on the device, any "+1" folded in) and ``eps``; the residual kernels take those.
+* position:    ``__init__(spec, env)``, ``fused_rotation() -> (inv_freq | None, pos_scale)`` when the
+               q/k kernel can apply it, else ``apply(q, k, step)`` on the projected rows.
+* mixer:       ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, ``kv_need() -> GroupKey | None``,
+               ``state_need() -> StateNeed | None``,
+               ``forward(x[N, hidden], step, memory, writes) -> [N, hidden]``.
+* feed-forward: ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, ``forward(x[N, hidden], step) -> [N, hidden]``.
+* block:       ``tensor_needs(spec)``, ``__init__(spec, weights, env)``,
+               ``forward(h, pending, step, memory, writes) -> pending`` (see ``block.py``).
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional
+
+import torch
+
+
+@dataclass
+class BuildEnv:
+    """Where and in which element type the parts are built."""
+    dtype: torch.dtype                 # torch.float32 or torch.bfloat16: activations and cache
+    device: torch.device
+    workspace: "Workspace"
+
+
+class Workspace:
+    """Named device buffers that are reused from step to step, so a step allocates nothing
+    once its sizes have been seen.  ``generation`` changes whenever a buffer had to grow,
+    which tells a captured graph that its addresses are stale."""
+
+    def __init__(self, device: torch.device):
+        self.device = device
+        self._buffers: Dict[str, torch.Tensor] = {}
+        self.generation = 0
+
+    def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
+        key = f"{name}:{cols}:{dtype}"
+        buf = self._buffers.get(key)
+        if buf is None or buf.shape[0] < rows:
+            cap = max(rows, 1)
+            if buf is not None:
+                cap = max(cap, buf.shape[0] * 2)
+            buf = torch.empty((cap, cols), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+            self.generation += 1
+        return buf[:rows]
+
+    def reserve(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> None:
+        self.get(name, rows, cols, dtype)
+
+
+_REGISTRIES: Dict[str, Dict[str, Callable]] = {"norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}}
+
+
+def register(category: str, kind: str, cls: Callable) -> None:
+    """Make ``cls`` the implementation of ``kind`` in ``category`` (norm, position, mixer, ffn,
+    block).  A later registration of the same kind replaces the earlier one."""
+    if category not in _REGISTRIES:
+        raise KeyError(f"unknown part category {category!r}; known: {sorted(_REGISTRIES)}")
+    _REGISTRIES[category][kind] = cls
+
+
+def lookup(category: str, kind: str) -> Callable:
+    try:
+        return _REGISTRIES[category][kind]
+    except KeyError:
+        raise KeyError(f"no {category} part of kind {kind!r} is registered; known: "
+                       f"{sorted(_REGISTRIES.get(category, {}))}") from None
+
+
+def registered(category: str) -> List[str]:
+    return sorted(_REGISTRIES[category])

@@ -1,0 +1,89 @@
+"""Arrangements of a layer's parts around the 32-bit residual stream ``h``.
+
+``sandwich`` (``src/models/gemma3.zig:341-348, 708-709, 823-826, 835-836, 872-878``):
+
+    h += post_mixer_norm(mixer(pre_mixer_norm(h)));  h += post_ffn_norm(ffn(pre_ffn_norm(h)))
+
+``prenorm`` is the same without the two post norms.  A block never adds its last branch
+itself: it returns it as *pending* ``(branch, norm | None)``, and whoever runs next (the
+next block's first norm, or the model's end) adds it in the same kernel that computes the
+next norm, so the residual stream is read and written once per sublayer.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Tuple
+
+import torch
+
+from ..config.spec import LayerSpec
+from ..ops import kernels
+from ..weights.loader import TensorNeed
+from .base import BuildEnv, lookup, register
+
+Pending = Optional[Tuple[torch.Tensor, Optional[object]]]
+
+
+def add_pending_and_norm(h: torch.Tensor, pending: Pending, norm, out: Optional[torch.Tensor],
+                         rows: Optional[torch.Tensor] = None) -> None:
+    """h += post(branch) for a pending branch, then out = norm(h) if asked."""
+    branch, post = pending if pending is not None else (None, None)
+    if rows is not None and branch is not None:
+        kernels.residual_norm(h, branch, post.gain if post else None, post.eps if post else 0.0, None, None, 0.0)
+        branch = None
+    kernels.residual_norm(h, branch, post.gain if (branch is not None and post) else None,
+                          post.eps if (branch is not None and post) else 0.0,
+                          out, norm.gain if out is not None else None, norm.eps if out is not None else 0.0, rows)
+
+
+class SandwichBlock:
+    post_norms = True
+
+    def __init__(self, spec: LayerSpec, weights, env: BuildEnv):
+        self.spec = spec
+        self.env = env
+
+        def norm(ns):
+            return lookup("norm", ns.kind)(ns, weights, env) if ns is not None else None
+        self.pre_mixer = norm(spec.pre_mixer_norm)
+        self.post_mixer = norm(spec.post_mixer_norm) if self.post_norms else None
+        self.pre_ffn = norm(spec.pre_ffn_norm)
+        self.post_ffn = norm(spec.post_ffn_norm) if self.post_norms else None
+        if self.pre_mixer is None or (spec.ffn is not None and self.pre_ffn is None):
+            raise ValueError("a block needs a norm before its mixer and before its feed-forward")
+        self.mixer = lookup("mixer", spec.mixer.kind)(spec.mixer, weights, env)
+        self.ffn = lookup("ffn", spec.ffn.kind)(spec.ffn, weights, env) if spec.ffn is not None else None
+        self.hidden = self.pre_mixer.size
+
+    @classmethod
+    def tensor_needs(cls, spec: LayerSpec) -> List[TensorNeed]:
+        needs: List[TensorNeed] = []
+        norms = [spec.pre_mixer_norm, spec.pre_ffn_norm]
+        if cls.post_norms:
+            norms += [spec.post_mixer_norm, spec.post_ffn_norm]
+        for ns in norms:
+            if ns is not None:
+                needs += lookup("norm", ns.kind).tensor_needs(ns)
+        needs += lookup("mixer", spec.mixer.kind).tensor_needs(spec.mixer)
+        if spec.ffn is not None:
+            needs += lookup("ffn", spec.ffn.kind).tensor_needs(spec.ffn)
+        return needs
+
+    def forward(self, h: torch.Tensor, pending: Pending, step, memory: int, writes: bool) -> Pending:
+        n = h.shape[0]
+        x = self.env.workspace.get("normed", n, self.hidden, self.env.dtype)
+        add_pending_and_norm(h, pending, self.pre_mixer, x)
+        a = self.mixer.forward(x, step, memory, writes)
+        pending = (a, self.post_mixer)
+        if self.ffn is None:
+            return pending
+        add_pending_and_norm(h, pending, self.pre_ffn, x)
+        f = self.ffn.forward(x, step)
+        return (f, self.post_ffn)
+
+
+class PreNormBlock(SandwichBlock):
+    post_norms = False
+
+
+register("block", "sandwich", SandwichBlock)
+register("block", "prenorm", PreNormBlock)

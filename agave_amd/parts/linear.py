@@ -1,0 +1,45 @@
+"""A linear map y = W x with W stored row-major [out, in] (``src/backend/backend.zig:474, 481``).
+
+The weight stays in the element type it was stored in, unless the engine runs in 32-bit, in
+which case bfloat16 weights are widened (exactly).  The kernel is chosen by the types: 32-bit
+anything goes through the plain multiply-add kernel; bfloat16 activations with bfloat16
+weights go through the matrix-core kernels, which fall back to the plain kernel for shapes
+they refuse.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import torch
+
+from ..ops import kernels
+from .base import BuildEnv
+
+
+class Linear:
+    def __init__(self, weights: Sequence[torch.Tensor], env: BuildEnv, name: str = "linear"):
+        """``weights``: one or more [out_i, in] matrices that are stacked along ``out``."""
+        ws = []
+        for w in weights:
+            if w.dim() != 2:
+                raise ValueError(f"{name}: weight must be a matrix, got {tuple(w.shape)}")
+            if env.dtype == torch.float32 and w.dtype != torch.float32:
+                w = w.to(torch.float32)
+            ws.append(w)
+        if len({w.dtype for w in ws}) != 1 or len({w.shape[1] for w in ws}) != 1:
+            raise ValueError(f"{name}: stacked weights must agree in element type and input size")
+        dev = [w.to(env.device) for w in ws]
+        self.weight = dev[0].contiguous() if len(dev) == 1 else torch.cat(dev, dim=0).contiguous()
+        self.out_features, self.in_features = self.weight.shape
+        self.env = env
+        self.name = name
+        self.packed = None          # set by the matrix-core module when it repacks the weight
+
+    def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
+                out_dtype: Optional[torch.dtype] = None, tag: Optional[str] = None) -> torch.Tensor:
+        n = x.shape[0]
+        if out is None:
+            out = self.env.workspace.get(tag or self.name, n, self.out_features, out_dtype or x.dtype)
+        from ..ops import gemm
+        gemm.linear(x, self, out)
+        return out

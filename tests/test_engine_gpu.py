@@ -1,0 +1,106 @@
+"""The engine against the plain implementation on the GPU: each request alone and whole, with
+the last 32 tokens one by one, and in batches of unequal lengths whose shorter requests end
+earlier, one batch after another so that slots and pages are used again; in 32-bit and in
+bfloat16."""
+import pytest
+import torch
+
+import engine_utils as U
+import plain_gemma3 as P
+
+pytestmark = pytest.mark.gpu
+
+# 32-bit: rounding only.  The logits are O(1); a fault in any formula shows as >= 1e-3.
+F32_ATOL, F32_RTOL = 2e-5, 1e-5
+
+
+def bf16_close(got: torch.Tensor, ref: torch.Tensor, what: str):
+    """bfloat16 keeps 8 bits: activations are rounded at ~2^-9 relative at each of a few dozen
+    places, so a logit row may differ by a few percent of its largest entry."""
+    scale = ref.abs().max(dim=-1, keepdim=True).values
+    err = ((got.double() - ref) .abs() / scale).max(dim=-1).values
+    worst = int(err.argmax())
+    assert float(err.max()) < 0.04, f"{what}: relative error {float(err.max()):.4f} at position {worst}"
+
+
+def f32_close(got: torch.Tensor, ref: torch.Tensor, what: str):
+    diff = (got.double() - ref).abs()
+    tol = F32_ATOL + F32_RTOL * ref.abs()
+    bad = (diff > tol).any(dim=-1)
+    if bad.any():
+        first = int(torch.nonzero(bad)[0])
+        raise AssertionError(f"{what}: first wrong position {first} of {got.shape[0]}, "
+                             f"max error there {float(diff[first].max()):.3e}, overall {float(diff.max()):.3e}")
+
+
+def close(dtype):
+    return f32_close if dtype == "float32" else bf16_close
+
+
+@pytest.fixture(scope="module", params=["A", "B", "C"])
+def tiny(request, tmp_path_factory):
+    which = request.param
+    cfg = P.tiny_config(which)
+    weights = P.random_weights(cfg, {"A": 0, "B": 1, "C": 2}[which])
+    folder = U.write_model(str(tmp_path_factory.mktemp(f"tiny{which}")), cfg, weights)
+    return which, cfg, weights, folder
+
+
+@pytest.fixture(scope="module", params=["float32", "bfloat16"])
+def engine_of(request, tiny):
+    from agave_amd.engine import Engine
+    which, cfg, weights, folder = tiny
+    eng = Engine.from_folder(folder, dtype=request.param, max_slots=6, max_context=192)
+    return eng, request.param, cfg, weights
+
+
+def test_whole_prompt(engine_of):
+    eng, dtype, cfg, weights = engine_of
+    for n, seed in ((1, 10), (5, 11), (40, 12), (150, 13)):
+        toks = U.random_tokens(n, cfg["vocab_size"], seed)
+        close(dtype)(U.run_whole(eng, toks), U.plain_logits(cfg, weights, toks), f"whole n={n}")
+
+
+def test_tail_one_by_one(engine_of):
+    eng, dtype, cfg, weights = engine_of
+    for n, seed in ((33, 20), (100, 21), (160, 22)):
+        toks = U.random_tokens(n, cfg["vocab_size"], seed)
+        ref = U.plain_logits(cfg, weights, toks)
+        close(dtype)(U.run_tail(eng, toks, 32), ref, f"tail n={n}")
+
+
+def test_first_tokens_one_by_one(engine_of):
+    eng, dtype, cfg, weights = engine_of
+    toks = U.random_tokens(20, cfg["vocab_size"], 30)
+    close(dtype)(U.run_tail(eng, toks, 19), U.plain_logits(cfg, weights, toks), "from the first token")
+
+
+def test_batches_of_unequal_lengths_reuse_slots(engine_of):
+    eng, dtype, cfg, weights = engine_of
+    v = cfg["vocab_size"]
+    batches = [
+        ([U.random_tokens(n, v, 40 + i) for i, n in enumerate((13, 48, 27))], (5, 40, 19)),
+        ([U.random_tokens(n, v, 50 + i) for i, n in enumerate((9, 70, 31, 69, 100))], (1, 57, 13, 30, 7)),
+        ([U.random_tokens(n, v, 60 + i) for i, n in enumerate((66, 3))], (64, 3)),
+    ]
+    for bi, (reqs, plens) in enumerate(batches):
+        outs = U.run_batched(eng, reqs, plens)
+        for i, (r, o) in enumerate(zip(reqs, outs)):
+            close(dtype)(o, U.plain_logits(cfg, weights, r), f"batch {bi} request {i}")
+    assert eng.cache.slots.n_free == eng.cache.max_slots
+    for g in eng.cache.groups:
+        assert g.pool.n_free == g.pool.n_pages
+
+
+def test_cutting_gives_the_same_numbers(engine_of):
+    """With the plain kernels a position's arithmetic does not depend on the cutting at all;
+    with the matrix-core kernels it may differ by rounding."""
+    eng, dtype, cfg, weights = engine_of
+    toks = U.random_tokens(90, cfg["vocab_size"], 70)
+    whole, tail = U.run_whole(eng, toks), U.run_tail(eng, toks, 32)
+    other = U.random_tokens(50, cfg["vocab_size"], 71)
+    batched = U.run_batched(eng, [other, toks], (20, 58))[1]
+    tol = 1e-5 if dtype == "float32" else 0.03
+    scale = float(whole.abs().max())
+    assert float((whole - tail).abs().max()) <= tol * scale
+    assert float((whole - batched).abs().max()) <= tol * scale
