@@ -74,6 +74,7 @@ class Engine:
         self.cache = KVCache(kv_needs, self.model.state_needs(), max_slots, pages, self.dtype, self.device,
                              self.max_context)
         self.planner = StepPlanner(self.cache, spec.vocab_size, self.device)
+        self.prefill_chunk = 0          # > 0: prompts enter in pieces of at most this many tokens
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -128,3 +129,49 @@ class Engine:
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.device)
+
+    # ------------------------------------------------------------------ sampling and generation
+    @property
+    def max_slots(self) -> int:
+        return self.cache.max_slots
+
+    def step_sample(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], rows) -> List[int]:
+        """One step, then one token per sequence drawn from its last logits on the GPU.
+        ``rows``: one :class:`RowSampling` per sequence."""
+        from ..ops import sampling as sample_ops
+        chunk = int(self.prefill_chunk or 0)
+        if chunk > 0 and max(len(t) for t in tokens) > chunk:
+            # the reference feeds a prompt in chunks (src/models/gemma3.zig:385-391); only the
+            # last piece of each sequence needs logits
+            tokens = [list(t) for t in tokens]
+            while max(len(t) for t in tokens) > chunk:
+                idx = [i for i, t in enumerate(tokens) if len(t) > chunk]
+                self.step([slots[i] for i in idx], [tokens[i][:chunk] for i in idx], "none")
+                for i in idx:
+                    tokens[i] = tokens[i][chunk:]
+        logits = self.step(slots, tokens, "last")
+        b = len(slots)
+        if any(r.repeat_penalty != 1.0 and r.generated for r in rows):
+            cu = [0]
+            flat: List[int] = []
+            for r in rows:
+                if r.repeat_penalty != 1.0:
+                    flat.extend(r.generated)
+                cu.append(len(flat))
+            ids = torch.tensor(flat or [0], dtype=torch.int32, device=self.device)
+            cu_t = torch.tensor(cu, dtype=torch.int32, device=self.device)
+            pen = torch.tensor([r.repeat_penalty for r in rows], dtype=torch.float32, device=self.device)
+            sample_ops.repeat_penalty(logits, ids, cu_t, pen)
+        params = torch.tensor([[r.temperature, float(min(r.top_k, 1 << 20)), r.top_p, r.u] for r in rows],
+                              dtype=torch.float32, device=self.device)
+        work = self.workspace.get("sample_work", b, self.spec.vocab_size, torch.float32)
+        out = self.workspace.get("sampled", b, 1, torch.int32).view(-1)
+        sample_ops.sample(logits, work, params, out)
+        return out.cpu().tolist()
+
+    def generate(self, prompts, params=None, max_batch: Optional[int] = None, stats=None):
+        """Generate for every prompt (lists of token ids); see :func:`agave_amd.engine.generate.generate`."""
+        from ..sampling import SamplingParams
+        from .generate import generate
+        return generate(self, prompts, params if params is not None else SamplingParams(),
+                        eos_ids=self.spec.eos_token_ids, max_batch=max_batch, stats=stats)

@@ -1,0 +1,131 @@
+"""The generation loop above the step function: batches of unequal prompts, stop tokens,
+sequences that end earlier, and as many batches one after another as there are requests.
+
+Reference (one sequence): ``generateAndPrintInner`` (``src/main.zig:2118-2461``): the first
+token comes from the prompt's last logits (``:2290-2294``), then up to ``max_tokens - 1``
+further steps (``:2342``); the repeat penalty covers every id generated so far (``:2350-2352``);
+an end-of-generation id stops the sequence and is not emitted (``:2366-2369``); a full cache
+ends it too (``KVCacheFull``, ``src/models/gemma3.zig:332``).  The reference's "halt after six
+equal tokens" (``src/main.zig:2400-2407``) changes outputs and is not taken over.
+
+The loop's decisions need no GPU: it talks to a *backend* with ``max_context``, ``max_slots``,
+``alloc_slot()``, ``free_slot(slot)`` and ``step_sample(slots, tokens, rows) -> token ids``;
+the engine is one, the tests use a fake.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence, Union
+
+import numpy as np
+
+from ..sampling import GenerationResult, SamplingParams
+
+
+@dataclass
+class RowSampling:
+    """What the sampler needs for one sequence of a step."""
+    temperature: float
+    top_k: int
+    top_p: float
+    repeat_penalty: float
+    u: float                     # uniform draw in [0, 1) of this request's own stream
+    generated: List[int]         # ids generated so far (for the repeat penalty)
+
+
+@dataclass
+class GenerationStats:
+    """Counters in the reference's terms (``src/display.zig:143-163, 702-744``)."""
+    prefill_tokens: int = 0
+    prefill_ms: float = 0.0
+    tokens: int = 0              # generated tokens of all requests
+    gen_ms: float = 0.0          # decode steps only
+    decode_tokens: int = 0       # tokens produced by decode steps
+    batches: int = 0
+
+    @property
+    def tok_per_sec(self) -> float:
+        return self.decode_tokens / (self.gen_ms / 1e3) if self.gen_ms > 0 else 0.0
+
+    @property
+    def prefill_tok_per_sec(self) -> float:
+        return self.prefill_tokens / (self.prefill_ms / 1e3) if self.prefill_ms > 0 else 0.0
+
+
+def generate(backend, prompts: Sequence[Sequence[int]],
+             params: Union[SamplingParams, Sequence[SamplingParams]] = SamplingParams(),
+             eos_ids: Sequence[int] = (), max_batch: Optional[int] = None,
+             stats: Optional[GenerationStats] = None) -> List[GenerationResult]:
+    """Generate for every prompt (lists of token ids).  Requests run in batches of at most
+    ``max_batch`` (default: the backend's slots), in the order given, one batch after another;
+    a request's result does not depend on the others."""
+    n = len(prompts)
+    plist = [params] * n if isinstance(params, SamplingParams) else list(params)
+    if len(plist) != n:
+        raise ValueError(f"{len(plist)} sampling parameter sets for {n} prompts")
+    max_batch = int(max_batch or backend.max_slots)
+    if max_batch < 1 or max_batch > backend.max_slots:
+        raise ValueError(f"max_batch must be in 1..{backend.max_slots}")
+    stats = stats if stats is not None else GenerationStats()
+    clock_seed = time.time_ns() & 0x7FFFFFFF
+    results = [GenerationResult(i, len(p)) for i, p in enumerate(prompts)]
+    rngs = [np.random.default_rng([p.seed if p.seed is not None else clock_seed, i]) for i, p in enumerate(plist)]
+    stops = [set() if p.ignore_eos else (set(int(x) for x in eos_ids) | set(p.stop_ids)) for p in plist]
+
+    queue = []
+    for i, p in enumerate(prompts):
+        if len(p) == 0:
+            raise ValueError(f"prompt {i} is empty (give at least the begin-of-sequence id)")
+        if len(p) > backend.max_context:
+            results[i].finish_reason = "context"        # the prompt alone does not fit a slot
+        else:
+            queue.append(i)
+
+    def row(i: int) -> RowSampling:
+        p = plist[i]
+        u = float(rngs[i].random(dtype=np.float32)) if p.temperature > 0 else 0.0
+        return RowSampling(p.temperature, p.top_k, p.top_p, p.repeat_penalty, u, results[i].tokens)
+
+    while queue:
+        batch, queue = queue[:max_batch], queue[max_batch:]
+        stats.batches += 1
+        slots = {i: backend.alloc_slot() for i in batch}
+        live = list(batch)
+        feed = [list(prompts[i]) for i in live]
+        first = True
+        try:
+            while live:
+                t0 = time.perf_counter()
+                sampled = backend.step_sample([slots[i] for i in live], feed, [row(i) for i in live])
+                ms = (time.perf_counter() - t0) * 1e3
+                if first:
+                    stats.prefill_tokens += sum(len(f) for f in feed)
+                    stats.prefill_ms += ms
+                else:
+                    stats.gen_ms += ms
+                    stats.decode_tokens += len(live)
+                first = False
+                nxt = []
+                for i, tok in zip(live, sampled):
+                    tok = int(tok)
+                    r = results[i]
+                    if tok in stops[i]:
+                        r.finish_reason = "stop"                      # the end token is not emitted
+                    else:
+                        r.tokens.append(tok)
+                        stats.tokens += 1
+                        if len(r.tokens) >= plist[i].max_tokens:
+                            r.finish_reason = "length"
+                        elif r.prompt_tokens + len(r.tokens) > backend.max_context:
+                            r.finish_reason = "context"               # no room to feed this token
+                    if r.finish_reason:
+                        backend.free_slot(slots.pop(i))               # given back at once
+                    else:
+                        nxt.append(i)
+                live = nxt
+                feed = [[results[i].tokens[-1]] for i in live]
+        finally:
+            for s in slots.values():
+                backend.free_slot(s)
+    return results

@@ -1,0 +1,50 @@
+"""Faces of the sampling kernels."""
+from __future__ import annotations
+
+import torch
+
+from . import kernels, library
+from .kernels import _I, _L, _P
+
+kernels.register_signatures("sampling", {
+    "agave_sample": [_P, _L, _P, _L, _P, _P, _I, _I, _P],
+    "agave_repeat_penalty": [_P, _L, _P, _P, _P, _I, _I, _P],
+})
+
+
+def _logits(logits: torch.Tensor) -> int:
+    if not logits.is_cuda:
+        raise RuntimeError("sampling runs on the GPU only; got CPU logits")
+    if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+        raise TypeError("logits must be float32 [rows, vocab] with contiguous rows")
+    return logits.stride(0)
+
+
+def sample(logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor) -> None:
+    """out[b] = a token drawn from row b.  ``params`` float32 [rows, 4] = temperature, top_k,
+    top_p, u; temperature 0 takes the argmax (first index on ties).  ``work``: float32 scratch
+    of the logits' shape."""
+    ld = _logits(logits)
+    b, v = logits.shape
+    if work.dtype != torch.float32 or work.shape != logits.shape or work.stride(1) != 1 or not work.is_cuda:
+        raise TypeError("sample: work must be a float32 GPU tensor of the logits' shape")
+    if params.dtype != torch.float32 or params.shape != (b, 4) or not params.is_contiguous() or not params.is_cuda:
+        raise TypeError(f"sample: params must be contiguous float32 [{b}, 4] on the GPU")
+    if out.dtype != torch.int32 or out.numel() != b or not out.is_contiguous() or not out.is_cuda:
+        raise TypeError(f"sample: out must be {b} contiguous int32 on the GPU")
+    library.call(kernels.lib("sampling"), "agave_sample", logits.data_ptr(), ld, work.data_ptr(), work.stride(0),
+                 params.data_ptr(), out.data_ptr(), b, v, kernels.stream())
+
+
+def repeat_penalty(logits: torch.Tensor, ids: torch.Tensor, cu: torch.Tensor, penalty: torch.Tensor) -> None:
+    """In place: for every id in ids[cu[b]:cu[b+1]], once per occurrence, row b's logit is divided
+    by penalty[b] if positive, else multiplied."""
+    ld = _logits(logits)
+    b, v = logits.shape
+    for t, n, what in ((ids, 0, "ids"), (cu, b + 1, "cu")):
+        if t.dtype != torch.int32 or not t.is_contiguous() or not t.is_cuda or t.numel() < n:
+            raise TypeError(f"repeat_penalty: {what} must be contiguous int32 on the GPU")
+    if penalty.dtype != torch.float32 or penalty.numel() != b or not penalty.is_cuda:
+        raise TypeError(f"repeat_penalty: penalty must be {b} float32 on the GPU")
+    library.call(kernels.lib("sampling"), "agave_repeat_penalty", logits.data_ptr(), ld, ids.data_ptr(),
+                 cu.data_ptr(), penalty.data_ptr(), b, v, kernels.stream())

@@ -1,0 +1,156 @@
+"""The cache's bookkeeping: no slot or page lost, held twice or freed twice; windowed groups
+give pages back; a step that does not fit changes nothing."""
+import random
+
+import pytest
+import torch
+
+from agave_amd.cache import (PAGE, CacheError, GroupKey, GroupPages, KVCache, OutOfPages, OutOfSlots, PagePool,
+                             SlotTable, StateNeed)
+
+
+def test_page_pool_alloc_free():
+    pool = PagePool(4)
+    got = [pool.alloc() for _ in range(4)]
+    assert sorted(got) == [0, 1, 2, 3] and pool.n_free == 0
+    with pytest.raises(OutOfPages):
+        pool.alloc()
+    pool.free(2)
+    with pytest.raises(CacheError):
+        pool.free(2)                        # freed twice
+    with pytest.raises(CacheError):
+        pool.free(9)
+    assert pool.alloc() == 2                # used again
+    for p in got:
+        pool.free(p)
+    assert pool.n_free == 4
+
+
+def test_slot_table():
+    st = SlotTable(2)
+    a, b = st.alloc(), st.alloc()
+    assert {a, b} == {0, 1}
+    with pytest.raises(OutOfSlots):
+        st.alloc()
+    st.free(a)
+    with pytest.raises(CacheError):
+        st.free(a)
+    assert st.alloc() == a and st.length[a] == 0
+
+
+def _cache(window=None, n_pages=8, slots=3, ctx=512):
+    full, win = GroupKey(None, 1, 8), GroupKey(window, 1, 8)
+    needs = {0: win, 1: full, 2: win} if window else {0: full, 1: full}
+    return KVCache(needs, {}, slots, {k: n_pages for k in set(needs.values())}, torch.float32, None, ctx)
+
+
+def test_full_group_tables_and_release():
+    c = _cache()
+    s = c.alloc_slot()
+    pos0, plans = c.plan_step([s], [70])
+    assert pos0 == [0] and plans[0].base == [0] and len(plans[0].rows[0]) == 2
+    c.commit_step([s], [70])
+    assert c.length(s) == 70
+    pos0, plans = c.plan_step([s], [1])
+    assert pos0 == [70] and len(plans[0].rows[0]) == 2          # position 70 is in page 1: nothing new
+    c.commit_step([s], [1])
+    for _ in range(57):
+        c.plan_step([s], [1]); c.commit_step([s], [1])
+    assert c.length(s) == 128
+    _, plans = c.plan_step([s], [1])
+    assert len(plans[0].rows[0]) == 3
+    c.commit_step([s], [1])
+    c.free_slot(s)
+    assert c.groups[0].pool.n_free == 8 and c.slots.n_free == 3
+    with pytest.raises(CacheError):
+        c.free_slot(s)
+
+
+def test_window_group_gives_pages_back_and_keeps_reach():
+    W = 100
+    c = _cache(window=W, n_pages=16, ctx=1024)
+    gi = [i for i, k in enumerate(c.group_keys) if k.window == W][0]
+    g = c.groups[gi]
+    s = c.alloc_slot()
+    c.plan_step([s], [500]); c.commit_step([s], [500])
+    held = g.held(s)
+    # a query at position >= 500 reaches back to 500 - W + 1 = 401 -> page 6
+    assert min(held) == 401 // PAGE and max(held) == 499 // PAGE
+    for step in range(200):
+        L = c.length(s)
+        _, plans = c.plan_step([s], [1])
+        base, row = plans[gi].base[0], plans[gi].rows[0]
+        assert base == max(0, L - W + 1) // PAGE
+        assert base + len(row) - 1 == L // PAGE
+        assert len(set(row)) == len(row)
+        c.commit_step([s], [1])
+        assert len(g.held(s)) <= W // PAGE + 2
+    c.free_slot(s)
+    assert all(x.pool.n_free == x.pool.n_pages for x in c.groups)
+
+
+def test_step_that_does_not_fit_changes_nothing():
+    c = _cache(n_pages=4)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    with pytest.raises(OutOfPages):
+        c.plan_step([a, b], [130, 130])            # 3 + 3 pages > 4
+    assert c.groups[0].pool.n_free == 4 and c.groups[0].held(a) == {}
+    c.plan_step([a, b], [64, 128]); c.commit_step([a, b], [64, 128])
+    with pytest.raises(CacheError, match="context"):
+        c.plan_step([a], [512])
+    with pytest.raises(CacheError, match="twice"):
+        c.plan_step([a, a], [1, 1])
+    with pytest.raises(CacheError):
+        c.plan_step([2], [1])                      # slot not held
+
+
+def test_random_traffic_never_loses_or_doubles_a_page():
+    rnd = random.Random(0)
+    c = _cache(window=70, n_pages=40, slots=5, ctx=600)
+    live = {}
+    for _ in range(400):
+        if live and rnd.random() < 0.15:
+            s = rnd.choice(list(live))
+            c.free_slot(s); del live[s]
+        elif len(live) < 5 and rnd.random() < 0.3:
+            s = c.alloc_slot()
+            assert s not in live
+            live[s] = 0
+        elif live:
+            s = rnd.choice(list(live))
+            n = rnd.choice([1, 1, 1, 5, 64, 130])
+            try:
+                c.plan_step([s], [n])
+            except (OutOfPages, CacheError):
+                continue
+            c.commit_step([s], [n]); live[s] += n
+            assert c.length(s) == live[s]
+        for g in c.groups:
+            held = [p for s in range(5) for p in g.held(s).values()]
+            assert len(held) == len(set(held))                       # no page held twice
+            assert len(held) + g.pool.n_free == g.pool.n_pages       # none lost
+    for s in list(live):
+        c.free_slot(s)
+    assert all(g.pool.n_free == g.pool.n_pages for g in c.groups) and c.slots.n_free == 5
+
+
+def test_groups_and_state():
+    full, win = GroupKey(None, 2, 16), GroupKey(8, 2, 16)
+    c = KVCache({0: win, 1: win, 2: full, 3: win}, {1: StateNeed((3, 4))}, 2, {full: 4, win: 6},
+                torch.float32, torch.device("cpu"), 256)
+    assert c.group_keys == [win, full]
+    assert c.k_store[0].shape == (3, 6, 2, PAGE, 16) and c.v_store[0].shape == (3, 6, 2, 16, PAGE)
+    assert c.k_store[1].shape == (1, 4, 2, PAGE, 16)
+    assert c.index_in_group == {0: 0, 1: 1, 2: 0, 3: 2}
+    k, v = c.pages_of(3)
+    assert k.data_ptr() == c.k_store[0][2].data_ptr()
+    s = c.alloc_slot()
+    c.state[1][s].fill_(5.0)
+    c.free_slot(s)
+    assert c.alloc_slot() == s and float(c.state[1][s].abs().sum()) == 0.0    # zeroed when taken again
+
+
+def test_table_width():
+    g = GroupPages(GroupKey(1024, 1, 8), 64, 2)
+    assert g.table_width(4096) == 17 and g.table_width(512) == 8
+    assert GroupPages(GroupKey(None, 1, 8), 64, 2).table_width(4096) == 64

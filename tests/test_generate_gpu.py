@@ -1,0 +1,156 @@
+"""Generation, the command line and the replay tool on the GPU, against the plain implementation."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import engine_utils as U
+import plain_gemma3 as P
+
+pytestmark = pytest.mark.gpu
+ROOT = U.ROOT
+
+
+@pytest.fixture(scope="module")
+def model_a(tmp_path_factory):
+    cfg = P.tiny_config("A")
+    w = P.random_weights(cfg, 0)
+    return cfg, w, U.write_model(str(tmp_path_factory.mktemp("genA")), cfg, w)
+
+
+@pytest.fixture(scope="module")
+def model_b(tmp_path_factory):
+    cfg = P.tiny_config("B")
+    w = P.random_weights(cfg, 1)
+    return cfg, w, U.write_model(str(tmp_path_factory.mktemp("genB")), cfg, w)
+
+
+def plain_greedy(cfg, w, prompt, n, stops=()):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        nxt = P.argmax_first(P.forward(cfg, w, toks)[-1])
+        if nxt in stops:
+            break
+        out.append(nxt)
+        toks.append(nxt)
+    return out
+
+
+def test_greedy_generation_through_the_entry_point(model_a):
+    """BASELINE's Tiny A run: prompts of 5 / 19 / 40 tokens, 8 greedy steps each, context 64."""
+    from agave_amd import Engine, SamplingParams
+    cfg, w, folder = model_a
+    eng = Engine.from_folder(folder, dtype="float32", max_slots=3, max_context=64)
+    prompts = [U.random_tokens(n, 512, 80 + i) for i, n in enumerate((5, 19, 40))]
+    res = eng.generate(prompts, SamplingParams(max_tokens=8, ignore_eos=True))
+    for r, p in zip(res, prompts):
+        assert r.tokens == plain_greedy(cfg, w, p, 8), f"request {r.request}"
+        assert r.finish_reason == "length"
+    # the same one request at a time, and with prompts entering in chunks of 7 tokens
+    eng.prefill_chunk = 7
+    alone = [eng.generate([p], SamplingParams(max_tokens=8, ignore_eos=True))[0].tokens for p in prompts]
+    assert alone == [r.tokens for r in res]
+    assert eng.cache.slots.n_free == 3
+
+
+def test_stop_ids_and_context_end_generation(model_a):
+    from agave_amd import Engine, SamplingParams
+    cfg, w, folder = model_a
+    eng = Engine.from_folder(folder, dtype="float32", max_slots=2, max_context=64)
+    prompt = U.random_tokens(9, 512, 90)
+    free = plain_greedy(cfg, w, prompt, 6)
+    stop = free[3]
+    res = eng.generate([prompt], SamplingParams(max_tokens=6, stop_ids=(stop,)))[0]
+    assert res.tokens == free[:free.index(stop)] and res.finish_reason == "stop"
+    long = U.random_tokens(60, 512, 91)
+    res = eng.generate([long], SamplingParams(max_tokens=50, ignore_eos=True))[0]
+    assert res.finish_reason == "context" and len(res.tokens) == 5       # 60 + 4 fed tokens fill the 64 positions
+    assert res.tokens == plain_greedy(cfg, w, long, 5)
+
+
+def test_temperature_sampling_is_seeded_and_independent_of_batch_mates(model_b):
+    """BASELINE's Tiny B run: prompts of 1 / 7 / 13 / 30 / 57 tokens, 12 steps at temperature 0.8."""
+    from agave_amd import Engine, SamplingParams
+    cfg, w, folder = model_b
+    eng = Engine.from_folder(folder, dtype="float32", max_slots=5, max_context=96)
+    prompts = [U.random_tokens(n, 1000, 100 + i) for i, n in enumerate((1, 7, 13, 30, 57))]
+    sp = SamplingParams(max_tokens=12, temperature=0.8, seed=1, ignore_eos=True)
+    a = [r.tokens for r in eng.generate(prompts, sp)]
+    b = [r.tokens for r in eng.generate(prompts, sp)]
+    assert a == b and all(len(t) == 12 for t in a)
+    c = [r.tokens for r in eng.generate(prompts, sp, max_batch=2)]       # other batch mates, other slots
+    assert c == a
+    d = [r.tokens for r in eng.generate(prompts, SamplingParams(max_tokens=12, temperature=0.8, seed=2, ignore_eos=True))]
+    assert d != a
+    # every drawn token follows the plain rule for the u of the request's own stream
+    rng = np.random.default_rng([1, 3])
+    toks = list(prompts[3])
+    for got in a[3]:
+        u = float(rng.random(dtype=np.float32))
+        want = P.sample_token(P.forward(cfg, w, toks)[-1].float(), 0.8, 0, 1.0, u)
+        assert got == want
+        toks.append(got)
+
+
+def test_command_line_json(model_a):
+    cfg, w, folder = model_a
+    prompt = [2] + U.random_tokens(6, 512, 110)
+    out = subprocess.run([sys.executable, "-m", "agave_amd", folder, " ".join(map(str, prompt)), "-n", "5",
+                          "--dtype", "float32", "--json", "--ignore-eos", "--ctx-size", "64", "--max-batch", "2"],
+                         capture_output=True, text=True, cwd=ROOT, timeout=600)
+    assert out.returncode == 0, out.stderr[-2000:]
+    rec = json.loads(out.stdout.strip().splitlines()[-1])
+    assert rec["outputs"][0]["tokens"] == plain_greedy(cfg, w, prompt, 5)
+    assert rec["tokens"] == 5 and rec["prefill_tokens"] == 7
+    for key in ("tok_per_sec", "prefill_ms", "prefill_tok_per_sec", "gen_ms"):      # src/display.zig:702-744
+        assert key in rec
+    info = subprocess.run([sys.executable, "-m", "agave_amd", folder, "--model-info", "--json", "--dtype", "float32"],
+                          capture_output=True, text=True, cwd=ROOT, timeout=600)
+    assert info.returncode == 0, info.stderr[-2000:]
+    meta = json.loads(info.stdout.strip().splitlines()[-1])
+    assert meta["architecture"] == "Gemma3ForCausalLM" and meta["n_layers"] == 4 and meta["vocab_size"] == 512
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_tool_whole_tail_and_batches(model_b, dtype, tmp_path):
+    """bin/trace_run as a user calls it: the same requests whole, with the last 32 tokens one by
+    one, and in batches of unequal lengths one after another."""
+    cfg, w, folder = model_b
+    v = cfg["vocab_size"]
+    reqs = [U.random_tokens(n, v, 120 + i) for i, n in enumerate((40, 75, 9, 64, 33))]
+    refs = [U.plain_logits(cfg, w, r) for r in reqs]
+
+    def check(got, ref, what):
+        if dtype == "float32":
+            assert float((got - ref).abs().max()) < 3e-5, what
+        else:
+            assert float(((got - ref).abs().max(-1).values / ref.abs().max(-1).values).max()) < 0.04, what
+
+    # whole, each alone; then tail32, each alone: one request after another in one process
+    whole = [[r] for r in reqs]
+    rec, where = U.trace_steps_batched(whole, [[len(r)] for r in reqs])
+    out = U.run_trace_tool(folder, dtype, rec, str(tmp_path / "whole"), 128, v)
+    for i, ref in enumerate(refs):
+        got = torch.from_numpy(np.stack([out[s][row] for s, row in where[(i, 0)]])).double()
+        check(got, ref, f"whole {i}")
+    rec, where = U.trace_steps_batched(whole, [[max(1, len(r) - 32)] for r in reqs])
+    out = U.run_trace_tool(folder, dtype, rec, str(tmp_path / "tail"), 128, v)
+    for i, ref in enumerate(refs):
+        got = torch.from_numpy(np.stack([out[s][row] for s, row in where[(i, 0)]])).double()
+        check(got, ref, f"tail {i}")
+    # batches of unequal lengths; the cache holds exactly what the live requests need
+    batches = [[reqs[0], reqs[1], reqs[2]], [reqs[3], reqs[4]], [reqs[1], reqs[0]]]
+    plens = [[30, 60, 2], [64, 1], [75, 8]]
+    rec, where = U.trace_steps_batched(batches, plens)
+    need = max(sum(-(-len(r) // 64) * 64 for r in b) for b in batches)
+    out = U.run_trace_tool(folder, dtype, rec, str(tmp_path / "batched"), need, v)
+    for bi, b in enumerate(batches):
+        for ri, r in enumerate(b):
+            got = torch.from_numpy(np.stack([out[s][row] for s, row in where[(bi, ri)]])).double()
+            check(got, U.plain_logits(cfg, w, r), f"batch {bi} request {ri}")
+    # a step that wants nothing writes no file
+    assert not os.path.exists(str(tmp_path / "none" / "0.f32"))

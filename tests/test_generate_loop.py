@@ -1,0 +1,101 @@
+"""The generation loop's decisions, against a fake backend (no GPU): stop tokens are not
+emitted, shorter sequences end earlier and give their slot back at once, batches follow one
+another, lengths and the context bound finish a request."""
+from typing import List
+
+import pytest
+
+from agave_amd.engine.generate import GenerationStats, generate
+from agave_amd.sampling import SamplingParams
+
+
+class FakeBackend:
+    """Next token = (last token fed + 1) % 50; records what it was asked."""
+
+    def __init__(self, max_slots=3, max_context=64):
+        self.max_slots, self.max_context = max_slots, max_context
+        self.free = list(range(max_slots))
+        self.length = {}
+        self.steps: List[dict] = []
+        self.max_live = 0
+
+    def alloc_slot(self):
+        s = self.free.pop(0)
+        self.length[s] = 0
+        self.max_live = max(self.max_live, len(self.length))
+        return s
+
+    def free_slot(self, s):
+        assert s in self.length, "slot freed twice"
+        del self.length[s]
+        self.free.append(s)
+
+    def step_sample(self, slots, tokens, rows):
+        assert len(slots) == len(tokens) == len(rows) and len(set(slots)) == len(slots)
+        for s, t in zip(slots, tokens):
+            assert s in self.length and len(t) >= 1
+            self.length[s] += len(t)
+            assert self.length[s] <= self.max_context
+        self.steps.append({"slots": list(slots), "n": [len(t) for t in tokens], "u": [r.u for r in rows],
+                           "gen": [list(r.generated) for r in rows]})
+        return [(t[-1] + 1) % 50 for t in tokens]
+
+
+def test_stop_token_is_not_emitted_and_short_sequences_leave():
+    be = FakeBackend()
+    prompts = [[10, 11], [40], [5]]
+    res = generate(be, prompts, SamplingParams(max_tokens=8), eos_ids=[13, 44])
+    assert [r.tokens for r in res] == [[12], [41, 42, 43], [6, 7, 8, 9, 10, 11, 12]]
+    assert [r.finish_reason for r in res] == ["stop", "stop", "stop"]
+    assert be.steps[0]["n"] == [2, 1, 1]                       # unequal prompts in one step
+    assert [len(s["slots"]) for s in be.steps] == [3, 3, 2, 2, 1, 1, 1, 1]   # the batch shrinks
+    assert be.length == {} and sorted(be.free) == [0, 1, 2]
+
+
+def test_max_tokens_and_context():
+    be = FakeBackend(max_context=6)
+    res = generate(be, [[1, 2, 3], [1, 2, 3, 4, 5, 6, 7]], SamplingParams(max_tokens=3, ignore_eos=True), eos_ids=[5])
+    assert res[0].tokens == [4, 5, 6] and res[0].finish_reason == "length"      # eos ignored
+    assert res[1].tokens == [] and res[1].finish_reason == "context"            # the prompt does not fit
+    res = generate(be, [[1, 2, 3, 4]], SamplingParams(max_tokens=50))
+    # 4 prompt positions + tokens fed back must stay within 6 positions
+    assert res[0].finish_reason == "context" and res[0].tokens == [5, 6, 7]
+    with pytest.raises(ValueError, match="empty"):
+        generate(be, [[]])
+
+
+def test_batches_follow_one_another_and_reuse_slots():
+    be = FakeBackend(max_slots=2)
+    stats = GenerationStats()
+    res = generate(be, [[i] for i in range(5)], SamplingParams(max_tokens=2), stats=stats)
+    assert [r.tokens for r in res] == [[i + 1, i + 2] for i in range(5)]
+    assert stats.batches == 3 and be.max_live == 2
+    assert stats.tokens == 10 and stats.prefill_tokens == 5 and stats.decode_tokens == 5
+    assert [r.request for r in res] == list(range(5))
+
+
+def test_per_request_streams_do_not_depend_on_batch_mates():
+    p = SamplingParams(max_tokens=4, temperature=0.8, seed=3)
+    a = FakeBackend(max_slots=3)
+    generate(a, [[1], [2], [3]], p)
+    b = FakeBackend(max_slots=1)
+    generate(b, [[1], [2], [3]], p)
+    ua = [[s["u"][s["slots"].index(sl)] for s in a.steps if sl in s["slots"]] for sl in (0, 1, 2)]
+    ub = [[s["u"][0] for s in b.steps[i * 4:(i + 1) * 4]] for i in range(3)]
+    assert ua == ub and len(set(ua[0])) == 4 and ua[0] != ua[1]
+    c = FakeBackend(max_slots=3)
+    generate(c, [[1], [2], [3]], SamplingParams(max_tokens=4, temperature=0.8, seed=4))
+    assert c.steps[0]["u"] != a.steps[0]["u"]
+
+
+def test_repeat_penalty_sees_generated_ids_only_after_the_first_token():
+    be = FakeBackend(max_slots=1)
+    generate(be, [[7, 8]], SamplingParams(max_tokens=3, repeat_penalty=1.3))
+    assert [s["gen"][0] for s in be.steps] == [[], [9], [9, 10]]
+
+
+def test_sampling_params_are_checked():
+    for bad in (dict(max_tokens=0), dict(temperature=-1), dict(top_p=0.0), dict(top_p=1.5), dict(top_k=-1),
+                dict(repeat_penalty=0)):
+        with pytest.raises(ValueError):
+            SamplingParams(**bad)

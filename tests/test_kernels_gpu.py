@@ -1,0 +1,336 @@
+"""Each HIP kernel alone against its plain reference, at other sizes than the engine's tiny
+models use, in 32-bit and in bfloat16, with inputs made so that a fault shows (a far key that
+must win, a window's edge, scattered page ids)."""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_gemma3 as P
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+DEV = "cuda:0"
+
+
+def _g(name):
+    path = os.path.join(GOLDEN, name + ".bin")
+    if not os.path.isfile(path):
+        pytest.skip("reference golden vectors not mounted")
+    return torch.from_numpy(np.fromfile(path, dtype="<f4").copy())
+
+
+def _i32(x):
+    return torch.tensor(x, dtype=torch.int32, device=DEV)
+
+
+def _tol(dtype):
+    return dict(atol=2e-6, rtol=2e-6) if dtype == torch.float32 else dict(atol=1e-2, rtol=1e-2)
+
+
+@pytest.fixture(scope="module")
+def K():
+    from agave_amd.ops import kernels
+    return kernels
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_scale(K, dtype):
+    table = (torch.randn(300, 72) * 0.05).to(dtype)
+    toks = [0, 299, 17, 17, 123]
+    out = torch.empty(5, 72, dtype=torch.float32, device=DEV)
+    K.embed_scale(_i32(toks), table.to(DEV), math.sqrt(72.0), out)
+    ref = P.embed(toks, table.double(), 72)
+    assert torch.allclose(out.cpu().double(), ref, atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("e", [100, 2560, 3136])
+def test_residual_norm(K, dtype, e):
+    n = 7
+    h = torch.randn(n, e) * 3
+    br = (torch.randn(n, e) * 0.3).to(dtype)
+    gp, gq = torch.randn(e) * 0.1 + 1, torch.randn(e) * 0.1 + 1
+    hd = h.clone().to(DEV)
+    out = torch.empty(n, e, dtype=dtype, device=DEV)
+    K.residual_norm(hd, br.to(DEV), gp.to(DEV), 1e-5, out, gq.to(DEV), 3e-6)
+    h_ref = h.double() + P.rms_norm(br.double(), gp.double(), 1e-5, add_one=False)
+    o_ref = P.rms_norm(h_ref, gq.double(), 3e-6, add_one=False)
+    assert torch.allclose(hd.cpu().double(), h_ref, atol=3e-6, rtol=1e-6)      # the sum is 32-bit in both types
+    assert torch.allclose(out.cpu().double(), o_ref, **_tol(dtype))
+    # norm only, on gathered rows; and a plain add without a norm on the branch
+    rows = _i32([5, 0, 5])
+    out2 = torch.empty(3, e, dtype=dtype, device=DEV)
+    K.residual_norm(hd, None, None, 0.0, out2, gq.to(DEV), 3e-6, rows)
+    assert torch.allclose(out2.cpu().double(), o_ref[[5, 0, 5]], **_tol(dtype))
+    h3 = h.clone().to(DEV)
+    K.residual_norm(h3, br.to(DEV), None, 0.0, None, None, 0.0)
+    assert torch.allclose(h3.cpu().double(), h.double() + br.double(), atol=1e-6)
+
+
+@pytest.mark.parametrize("n", [128, 1152, 2560, 3136])
+def test_residual_norm_golden(K, n):
+    # research/kernels/generate_golden.py:98-110 (eps 1e-5, plain weight)
+    x, w, want = _g(f"rms_norm_n{n}_x"), _g(f"rms_norm_n{n}_w"), _g(f"rms_norm_n{n}_out")
+    h = x.view(1, n).clone().to(DEV)
+    out = torch.empty(1, n, dtype=torch.float32, device=DEV)
+    K.residual_norm(h, None, None, 0.0, out, w.to(DEV), 1e-5)
+    assert torch.allclose(out.cpu().view(-1), want, atol=2e-5, rtol=1e-5)
+
+
+def _pages(n_pages, nkv, hd, dtype):
+    k = torch.zeros(n_pages, nkv, 64, hd, dtype=dtype, device=DEV)
+    v = torch.zeros(n_pages, nkv, hd, 64, dtype=dtype, device=DEV)
+    return k, v
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_qk_norm_rope_kv(K, dtype):
+    nh, nkv, hd, rot = 3, 1, 40, 24           # head size no multiple of 16, partial rotation
+    seqs = [(0, 5, 3), (1, 130, 4)]           # (sequence, first position, tokens)
+    tok_seq = [b for b, _, n in seqs for _ in range(n)]
+    tok_pos = [p + i for _, p, n in seqs for i in range(n)]
+    n = len(tok_pos)
+    q = (torch.randn(n, nh * hd)).to(dtype)
+    k = (torch.randn(n, nkv * hd)).to(dtype)
+    v = (torch.randn(n, nkv * hd)).to(dtype)
+    qg, kg = torch.randn(hd) * 0.1 + 1, torch.randn(hd) * 0.1 + 1
+    inv = torch.from_numpy(np.exp(-np.log(5e3) * 2.0 * np.arange(rot // 2) / rot).astype(np.float32))
+    kp, vp = _pages(6, nkv, hd, dtype)
+    table = _i32([[4, -1, -1], [-1, 5, 2]])   # sequence 1: base 1, so page index 2 is column 1 -> page 5
+    base = _i32([0, 1])
+    q_out = torch.empty(n, nh * hd, dtype=dtype, device=DEV)
+    K.qk_norm_rope_kv(q.to(DEV), k.to(DEV), v.to(DEV), q_out, qg.to(DEV), kg.to(DEV), 1e-6, 2e-6, inv.to(DEV), 0.25,
+                      _i32(tok_seq), _i32(tok_pos), kp, vp, table, base, nh, nkv, hd)
+    pos = torch.tensor(tok_pos, dtype=torch.float64)
+    ang = P.rope_angles(pos, rot, 5e3, 4.0)
+    q_ref = P.apply_rope(P.rms_norm(q.double().view(n, nh, hd), qg.double(), 1e-6, add_one=False), ang)
+    k_ref = P.apply_rope(P.rms_norm(k.double().view(n, nkv, hd), kg.double(), 2e-6, add_one=False), ang)
+    tol = dict(atol=3e-6, rtol=3e-6) if dtype == torch.float32 else dict(atol=2e-2, rtol=1e-2)
+    assert torch.allclose(q_out.cpu().double().view(n, nh, hd), q_ref, **tol)
+    page_of = {0: {0: 4}, 1: {2: 5}}
+    for t, (b, p) in enumerate(zip(tok_seq, tok_pos)):
+        pg, row = page_of[b][p // 64], p % 64
+        assert torch.allclose(kp[pg, :, row, :].cpu().double(), k_ref[t], **tol)
+        assert torch.equal(vp[pg, :, :, row].cpu().view(-1), v[t])            # v is stored as it is
+    # rows that no token wrote stay zero
+    written = {(page_of[b][p // 64], p % 64) for b, p in zip(tok_seq, tok_pos)}
+    mask = torch.ones(6, 64, dtype=torch.bool)
+    for pg, row in written:
+        mask[pg, row] = False
+    assert float(kp.cpu().float().abs().sum(dim=(1, 3))[mask].sum()) == 0.0
+
+
+@pytest.mark.parametrize("pos", [0, 1, 10, 100, 1000])
+def test_rope_golden(K, pos):
+    # research/kernels/generate_golden.py:140-155: nh 4, hd 256, theta 1e4, no norm
+    q, want = _g(f"rope_nh4_hd256_pos{pos}_q_in"), _g(f"rope_nh4_hd256_pos{pos}_q_out")
+    inv = torch.from_numpy(np.exp(-np.log(1e4) * 2.0 * np.arange(128) / 256).astype(np.float32))
+    q_out = torch.empty(1, 1024, dtype=torch.float32, device=DEV)
+    K.qk_norm_rope_kv(q.view(1, -1).to(DEV), None, None, q_out, None, None, 0.0, 0.0, inv.to(DEV), 1.0,
+                      _i32([0]), _i32([pos]), None, None, None, None, 4, 0, 256)
+    assert torch.allclose(q_out.cpu().view(-1), want, atol=3e-4 if pos >= 100 else 2e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_geglu(K, dtype):
+    n, ff = 5, 333
+    gu = (torch.randn(n, 2 * ff) * 2).to(dtype).to(DEV)
+    out = torch.empty(n, ff, dtype=dtype, device=DEV)
+    K.geglu(gu[:, :ff], gu[:, ff:], out)
+    ref = P.gelu_tanh(gu[:, :ff].cpu().double()) * gu[:, ff:].cpu().double()
+    assert torch.allclose(out.cpu().double(), ref, **_tol(dtype))
+    big = torch.tensor([[-100.0, 100.0, 1.0, 1.0]], device=DEV)
+    o = torch.empty(1, 2, device=DEV)
+    K.geglu(big[:, :2], big[:, 2:], o)
+    assert torch.isfinite(o).all() and float(o[0, 1]) == 100.0
+
+
+@pytest.mark.parametrize("n", [128, 1152, 6912])
+def test_gelu_golden(K, n):
+    x, want = _g(f"gelu_n{n}_x"), _g(f"gelu_n{n}_out")
+    out = torch.empty(1, n, device=DEV)
+    K.geglu(x.view(1, n).to(DEV), torch.ones(1, n, device=DEV), out)
+    assert torch.allclose(out.cpu().view(-1), want, atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("ta,tw,tc", [(torch.float32,) * 3, (torch.bfloat16,) * 3,
+                                      (torch.bfloat16, torch.bfloat16, torch.float32),
+                                      (torch.bfloat16, torch.float32, torch.bfloat16)])
+@pytest.mark.parametrize("m,n,k", [(1, 53, 29), (37, 130, 75), (65, 64, 16)])
+def test_gemm_plain(K, ta, tw, tc, m, n, k):
+    a, w = torch.randn(m, k).to(ta), torch.randn(n, k).to(tw)
+    c = torch.empty(m, n, dtype=tc, device=DEV)
+    K.gemm_plain(a.to(DEV), w.to(DEV), c)
+    ref = a.double() @ w.double().T
+    tol = dict(atol=1e-5, rtol=1e-5) if tc == torch.float32 else dict(atol=5e-2, rtol=1e-2)
+    assert torch.allclose(c.cpu().double(), ref, **tol)
+    # a strided input (a slice of a wider matrix)
+    wide = torch.randn(m, k + 11).to(ta).to(DEV)
+    K.gemm_plain(wide[:, 5:5 + k], w.to(DEV), c)
+    assert torch.allclose(c.cpu().double(), wide[:, 5:5 + k].cpu().double() @ w.double().T, **tol)
+
+
+def _attn_case(K, dtype, nh, nkv, hd, lens, window, scale, seed=0, boost=None):
+    """Sequences of the given lengths in scattered pages; every position is a query."""
+    g = torch.Generator().manual_seed(seed)
+    n_pages = sum((L + 63) // 64 for L in lens) + 3
+    kp, vp = _pages(n_pages, nkv, hd, dtype)
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    width = max((L + 63) // 64 for L in lens)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    ks, vs, qs, tok_seq, tok_pos = [], [], [], [], []
+    for b, L in enumerate(lens):
+        k = torch.randn(L, nkv, hd, generator=g).to(dtype)
+        v = torch.randn(L, nkv, hd, generator=g).to(dtype)
+        q = torch.randn(L, nh, hd, generator=g).to(dtype)
+        if boost is not None:                  # one far key must win for the last query:
+            k = k - k.mean(dim=-1, keepdim=True)   # every other key is orthogonal to that query (score 0),
+            k[boost] = 1.0                         # the far key scores 20
+            q[L - 1] = 20.0 / (hd * scale)
+        for i in range((L + 63) // 64):
+            pg = perm.pop()
+            table[b, i] = pg
+            rows = slice(i * 64, min(L, i * 64 + 64))
+            kp[pg, :, :rows.stop - rows.start, :] = k[rows].transpose(0, 1).to(DEV)
+            vp[pg, :, :, :rows.stop - rows.start] = v[rows].permute(1, 2, 0).to(DEV)
+        ks.append(k); vs.append(v); qs.append(q)
+        tok_seq += [b] * L
+        tok_pos += list(range(L))
+    q_all = torch.cat(qs).reshape(-1, nh * hd).to(DEV)
+    out = torch.empty_like(q_all)
+    K.attn_plain(q_all, out, kp, vp, table.to(DEV), _i32([0] * len(lens)), _i32(tok_seq), _i32(tok_pos),
+                 nh, nkv, hd, scale, window)
+    refs = [P.attention_core(q.double(), k.double(), v.double(), scale, window) for q, k, v in zip(qs, ks, vs)]
+    return out.cpu().double().view(-1, nh, hd), torch.cat(refs), vs
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 40, None), (6, 1, 16, 70), (5, 5, 72, 300), (2, 1, 256, 64)])
+def test_attn_plain(K, dtype, nh, nkv, hd, window):
+    got, ref, _ = _attn_case(K, dtype, nh, nkv, hd, [1, 77, 300, 64], window, 0.21)
+    # 32-bit: a score is a sum of hd products of N(0,1) values, so its rounding error, and with it
+    # the relative error of exp(score), grows with hd
+    tol = dict(atol=2e-6 + 1e-7 * hd, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    assert torch.allclose(got, ref, **tol)
+
+
+def test_attn_plain_far_key_wins(K):
+    # among 700 keys, key 3 is made to dominate the last query's softmax: the output must be its value
+    got, ref, vs = _attn_case(K, torch.float32, 2, 1, 32, [700], None, 0.5, seed=1, boost=3)
+    assert torch.allclose(got[-1], ref[-1], atol=1e-5)
+    assert torch.allclose(got[-1, 0], vs[0][3, 0].double(), atol=1e-2)
+    # with a window that ends before it, the same key must not be seen
+    got_w, ref_w, _ = _attn_case(K, torch.float32, 2, 1, 32, [700], 696, 0.5, seed=1, boost=3)
+    assert torch.allclose(got_w[-1], ref_w[-1], atol=1e-5)
+    assert not torch.allclose(got_w[-1, 0], vs[0][3, 0].double(), atol=1e-1)
+    got_e, ref_e, _ = _attn_case(K, torch.float32, 2, 1, 32, [700], 697, 0.5, seed=1, boost=3)   # edge: just inside
+    assert torch.allclose(got_e[-1, 0], vs[0][3, 0].double(), atol=1e-2)
+
+
+@pytest.mark.parametrize("tag,nh,nkv,hd,sl,suffix", [
+    ("sdpa_nh4_nkv1_hd256_sl256", 4, 1, 256, 256, "_naive"), ("sdpa_nh4_nkv1_hd256_sl64", 4, 1, 256, 64, "_online"),
+    ("sdpa_nh20_nkv5_hd128_sl32", 20, 5, 128, 32, ""), ("sdpa_nh4_nkv1_hd256_sl1", 4, 1, 256, 1, "_naive")])
+def test_attn_plain_golden(K, tag, nh, nkv, hd, sl, suffix):
+    # research/kernels/generate_golden.py:56-95; the reference's criterion is max error < 1e-3
+    # (tests/sdpa_harness.zig:124-136); 32-bit sums give far less
+    q, keys, values = _g(tag + "_q"), _g(tag + "_keys").view(sl, nkv, hd), _g(tag + "_values").view(sl, nkv, hd)
+    n_pages = (sl + 63) // 64
+    kp, vp = _pages(n_pages, nkv, hd, torch.float32)
+    for i in range(n_pages):
+        rows = slice(i * 64, min(sl, i * 64 + 64))
+        kp[i, :, :rows.stop - rows.start] = keys[rows].transpose(0, 1).to(DEV)
+        vp[i, :, :, :rows.stop - rows.start] = values[rows].permute(1, 2, 0).to(DEV)
+    out = torch.empty(1, nh * hd, device=DEV)
+    K.attn_plain(q.view(1, -1).to(DEV), out, kp, vp, _i32([list(range(n_pages))]), _i32([0]), _i32([0]), _i32([sl - 1]),
+                 nh, nkv, hd, 1.0 / math.sqrt(hd), None)
+    assert torch.allclose(out.cpu().view(-1), _g(tag + "_out" + suffix), atol=2e-5)
+
+
+# ---------------------------------------------------------------- sampling
+@pytest.fixture(scope="module")
+def S():
+    from agave_amd.ops import sampling
+    return sampling
+
+
+def _sample(S, logits, params):
+    lg = logits.to(DEV).float().contiguous()
+    work = torch.empty_like(lg)
+    out = torch.empty(lg.shape[0], dtype=torch.int32, device=DEV)
+    S.sample(lg, work, torch.tensor(params, dtype=torch.float32, device=DEV), out)
+    return out.cpu().tolist()
+
+
+def test_argmax_first_of_ties(S):
+    lg = torch.full((3, 5000), -1.0)
+    lg[0, [4000, 77, 3000]] = 2.0
+    lg[1, :] = float("-inf")
+    lg[2, 4999] = 0.5
+    assert _sample(S, lg, [[0, 0, 1, 0.9]] * 3) == [77, 0, 4999]
+
+
+@pytest.mark.parametrize("temperature,top_k,top_p", [(1.0, 0, 1.0), (0.7, 0, 1.0), (1.3, 5, 1.0), (1.0, 0, 0.6),
+                                                      (0.9, 50, 0.8), (1.0, 2000, 0.95), (2.0, 1, 1.0)])
+def test_sample_matches_plain_rule(S, temperature, top_k, top_p):
+    """For every token the plain rule can draw, a u in the middle of its interval of the running
+    sum must give exactly that token."""
+    g = torch.Generator().manual_seed(5)
+    vocab = 3001
+    logits = torch.randn(vocab, generator=g) * 2.5
+    w = P.sample_distribution(logits, temperature, top_k, top_p)
+    cdf = torch.cumsum(w, 0) / w.sum()
+    support = torch.nonzero(w > 0).view(-1).tolist()
+    if top_k:
+        assert len(support) <= min(top_k, 1024)
+    picks = support if len(support) <= 64 else [support[i] for i in range(0, len(support), len(support) // 64)]
+    us, want = [], []
+    for i in picks:
+        lo = float(cdf[i - 1]) if i > 0 else 0.0
+        hi = float(cdf[i])
+        if hi - lo < 1e-5:
+            continue
+        us.append((lo + hi) / 2)
+        want.append(i)
+    got = _sample(S, logits.view(1, -1).repeat(len(us), 1), [[temperature, top_k, top_p, u] for u in us])
+    assert got == want
+    assert all(P.sample_token(logits, temperature, top_k, top_p, u) == i for u, i in zip(us, want))
+
+
+def test_sample_rows_are_independent_and_mixed(S):
+    g = torch.Generator().manual_seed(6)
+    lg = torch.randn(4, 70001, generator=g)
+    params = [[0.0, 0, 1.0, 0.3], [0.8, 0, 1.0, 0.3], [0.8, 3, 1.0, 0.99], [1.0, 0, 0.5, 0.0]]
+    together = _sample(S, lg, params)
+    alone = [_sample(S, lg[i:i + 1], [params[i]])[0] for i in range(4)]
+    assert together == alone
+    assert together[0] == int(lg[0].argmax())
+    assert together[2] in torch.topk(lg[2], 3).indices.tolist()
+    assert together == [P.sample_token(lg[i], *params[i]) for i in range(4)]
+
+
+def test_sample_frequencies_follow_softmax(S):
+    lg = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]])
+    n = 4000
+    us = (torch.arange(n) + 0.5) / n                    # a stratified sweep of u
+    got = _sample(S, lg.repeat(n, 1), [[0.7, 0, 1.0, float(u)] for u in us])
+    freq = torch.bincount(torch.tensor(got), minlength=5).double() / n
+    assert torch.allclose(freq, torch.softmax(lg[0].double() / 0.7, 0), atol=2.0 / n)
+
+
+def test_repeat_penalty(S):
+    lg = torch.tensor([[2.0, -2.0, 1.0, 3.0], [2.0, -2.0, 1.0, 3.0], [1.0, 1.0, 1.0, 1.0]], device=DEV)
+    ids = _i32([0, 1, 0, 9, 3])
+    cu = _i32([0, 4, 5, 5])
+    S.repeat_penalty(lg, ids, cu, torch.tensor([2.0, 3.0, 1.5], device=DEV))
+    want = torch.stack([P.apply_repeat_penalty(torch.tensor([2.0, -2.0, 1.0, 3.0]), [0, 1, 0, 9], 2.0),
+                        P.apply_repeat_penalty(torch.tensor([2.0, -2.0, 1.0, 3.0]), [3], 3.0),
+                        torch.ones(4)])
+    assert torch.allclose(lg.cpu(), want, atol=1e-6)
+
+
+def test_cpu_tensors_are_refused(K):
+    with pytest.raises(RuntimeError, match="GPU"):
+        K.gemm_plain(torch.zeros(2, 2), torch.zeros(2, 2), torch.zeros(2, 2))

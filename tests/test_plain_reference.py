@@ -12,7 +12,7 @@ import torch.nn.functional as F
 
 import plain_gemma3 as P
 
-GOLDEN = "/root/reference/research/kernels/golden"
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 needs_golden = pytest.mark.skipif(not os.path.isdir(GOLDEN), reason="reference golden vectors not mounted")
 
 

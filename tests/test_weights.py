@@ -1,0 +1,144 @@
+"""Weights: the container's reader against another writer, the round trip of the random-weights
+mode, and the one error that lists everything wrong."""
+import json
+import os
+import struct
+
+import pytest
+import torch
+
+import plain_gemma3 as P
+from agave_amd.config import find_architecture
+from agave_amd.engine.model import tensor_needs
+from agave_amd.weights import (Checkpoint, DictWeightSource, SafetensorsError, TensorNeed, WeightError,
+                               WeightSource, check_tensors, write_random_model, write_safetensors)
+
+
+def _needs(which="A"):
+    raw = P.tiny_config(which)
+    arch = find_architecture(raw)
+    return raw, tensor_needs(arch.spec(arch.parse(raw), None))
+
+
+def test_reader_against_the_safetensors_package(tmp_path):
+    from safetensors.torch import save_file
+    t = {"a": torch.randn(3, 5).bfloat16(), "b": torch.randn(7), "c": torch.arange(6, dtype=torch.int64).view(2, 3),
+         "d": torch.randn(2, 2).half(), "e": torch.zeros(0, 4)}
+    save_file(t, str(tmp_path / "model.safetensors"))
+    ck = Checkpoint(str(tmp_path))
+    assert sorted(ck.names()) == sorted(t)
+    assert ck.read("a").dtype == torch.bfloat16 and torch.equal(ck.read("a"), t["a"])
+    assert ck.read("b").dtype == torch.float32 and torch.equal(ck.read("b"), t["b"])      # 32-bit stays 32-bit
+    assert ck.read("c").dtype == torch.int32 and torch.equal(ck.read("c").long(), t["c"])  # tables as int32
+    assert ck.read("d").dtype == torch.float32 and torch.equal(ck.read("d"), t["d"].float())
+    assert ck.read("e").shape == (0, 4)
+
+
+def test_own_writer_is_read_by_the_package(tmp_path):
+    from safetensors.torch import load_file
+    t = {"x": torch.randn(4, 3).bfloat16(), "y": torch.randn(5)}
+    write_safetensors(str(tmp_path / "m.safetensors"), t)
+    back = load_file(str(tmp_path / "m.safetensors"))
+    assert torch.equal(back["x"], t["x"]) and torch.equal(back["y"], t["y"])
+
+
+def test_random_model_round_trip(tmp_path):
+    raw, needs = _needs("B")
+    write_random_model(raw, 7, str(tmp_path))
+    ck = Checkpoint(str(tmp_path))
+    src = WeightSource(ck, needs)
+    assert json.load(open(tmp_path / "config.json")) == raw
+    again = str(tmp_path / "again")
+    write_random_model(raw, 7, again)
+    other = str(tmp_path / "other")
+    write_random_model(raw, 8, other)
+    for n in needs:
+        a = src.get(n.name)
+        assert a.dtype == torch.bfloat16 and tuple(a.shape) == n.shape
+        assert torch.equal(a, Checkpoint(again).read(n.name))
+    assert not torch.equal(src.get(needs[0].name), Checkpoint(other).read(needs[0].name))
+    emb = src.get("model.embed_tokens.weight").float()
+    assert 0.015 < float(emb.std()) < 0.025
+    assert 0.05 < float(src.get("model.norm.weight").float().std()) < 0.2
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    raw, needs = _needs("A")
+    w = P.random_weights(raw, 0)
+    del w["model.layers.1.mlp.up_proj.weight"]
+    del w["model.norm.weight"]
+    w["model.layers.0.self_attn.q_proj.weight"] = torch.zeros(5, 5)
+    w["model.layers.9.extra.weight"] = torch.zeros(1)
+    with pytest.raises(WeightError) as ei:
+        DictWeightSource(w, needs)
+    e = ei.value
+    assert e.missing == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
+    assert e.unexpected == ["model.layers.9.extra.weight"]
+    assert e.wrong_shape == [("model.layers.0.self_attn.q_proj.weight", (5, 5), (128, 64))]
+    text = str(e)
+    for word in ("missing (2)", "unexpected (1)", "wrong shape (1)", "up_proj", "extra", "[5, 5]", "[128, 64]"):
+        assert word in text
+    # the same through a folder
+    from safetensors.torch import save_file
+    save_file({k: v.contiguous() for k, v in w.items()}, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightError, match="missing"):
+        WeightSource(Checkpoint(str(tmp_path)), needs)
+    check_tensors({"a": (1,)}, [TensorNeed("a", (1,))])
+
+
+def _raw_file(path, header: bytes, data: bytes = b"", hlen=None):
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(header) if hlen is None else hlen))
+        f.write(header)
+        f.write(data)
+
+
+def test_container_errors(tmp_path):
+    # mirrors the parser cases of src/format/safetensors.zig:2198-2296
+    d = tmp_path
+    with pytest.raises(SafetensorsError, match="no .safetensors"):
+        Checkpoint(str(d))
+    p = str(d / "model.safetensors")
+    open(p, "wb").write(b"abc")
+    with pytest.raises(SafetensorsError, match="too short"):
+        Checkpoint(str(d))
+    _raw_file(p, b"{}", hlen=1 << 40)
+    with pytest.raises(SafetensorsError, match="exceeds the file"):
+        Checkpoint(str(d))
+    _raw_file(p, b"{not json")
+    with pytest.raises(SafetensorsError, match="JSON"):
+        Checkpoint(str(d))
+    _raw_file(p, json.dumps({"t": {"dtype": "F32", "shape": [2], "data_offsets": [8, 0]}}).encode(), b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="before start"):
+        Checkpoint(str(d))
+    _raw_file(p, json.dumps({"t": {"dtype": "F32", "shape": [4], "data_offsets": [0, 16]}}).encode(), b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="past the file"):
+        Checkpoint(str(d))
+    _raw_file(p, json.dumps({"t": {"dtype": "Q4_K", "shape": [2], "data_offsets": [0, 8]}}).encode(), b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="unsupported dtype"):
+        Checkpoint(str(d))
+    _raw_file(p, json.dumps({"t": {"dtype": "F32", "shape": [3], "data_offsets": [0, 8]}}).encode(), b"\0" * 8)
+    with pytest.raises(SafetensorsError, match="needs 12 bytes"):
+        Checkpoint(str(d))
+    _raw_file(p, json.dumps({"__metadata__": {"format": "pt"},
+                             "t": {"dtype": "F32", "shape": [2], "data_offsets": [0, 8]}}).encode(),
+              struct.pack("<ff", 1.5, -2.0))
+    assert Checkpoint(str(d)).read("t").tolist() == [1.5, -2.0]
+
+
+def test_sharded_folder_with_index(tmp_path):
+    from safetensors.torch import save_file
+    save_file({"a": torch.ones(2)}, str(tmp_path / "model-00001-of-00002.safetensors"))
+    save_file({"b": torch.zeros(3)}, str(tmp_path / "model-00002-of-00002.safetensors"))
+    idx = {"weight_map": {"a": "model-00001-of-00002.safetensors", "b": "model-00002-of-00002.safetensors"}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(idx))
+    ck = Checkpoint(str(tmp_path))
+    assert ck.read("a").tolist() == [1, 1] and ck.read("b").tolist() == [0, 0, 0]
+    idx["weight_map"]["c"] = "../evil.safetensors"
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(idx))
+    with pytest.raises(SafetensorsError, match="bad shard name"):
+        Checkpoint(str(tmp_path))
+    idx["weight_map"]["c"] = "gone.safetensors"
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(idx))
+    with pytest.raises(SafetensorsError, match="not found"):
+        Checkpoint(str(tmp_path))
