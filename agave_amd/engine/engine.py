@@ -20,7 +20,7 @@ from ..cache import PAGE, GroupKey, KVCache
 from ..config import find_architecture, read_config_json
 from ..config.spec import ModelSpec
 from ..parts import BuildEnv, Workspace
-from ..weights import Checkpoint, DictWeightSource, WeightSource
+from ..weights import Checkpoint, DictWeightSource, RandomWeightSource, WeightSource
 from .model import Model, tensor_needs
 from .step import Step, StepPlanner, Want
 
@@ -94,6 +94,16 @@ class Engine:
         cfg = arch.parse(raw_config)
         spec = arch.spec(cfg, tensors.keys())
         return cls(spec, DictWeightSource(tensors, tensor_needs(spec)), config=cfg, **kw)
+
+    @classmethod
+    def from_random(cls, raw_config: dict, seed: int = 0, **kw) -> "Engine":
+        """Random weights made on the GPU (for measurements; no folder is written)."""
+        arch = find_architecture(raw_config)
+        cfg = arch.parse(raw_config)
+        spec = arch.spec(cfg, None)
+        device = require_gpu(kw.get("device"))
+        wdtype = parse_dtype(kw.get("dtype", "bfloat16"))
+        return cls(spec, RandomWeightSource(tensor_needs(spec), seed, device, wdtype), config=cfg, **kw)
 
     # ------------------------------------------------------------------ the reference's accessors
     @property

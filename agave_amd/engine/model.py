@@ -15,7 +15,7 @@ import torch
 from ..cache import GroupKey, StateNeed
 from ..config.spec import ModelSpec
 from ..ops import kernels
-from ..parts import BuildEnv, Linear, add_pending_and_norm, lookup
+from ..parts import BuildEnv, Linear, add_pending_and_norm, lookup, part_tensors
 from ..weights.loader import TensorNeed
 
 
@@ -81,31 +81,9 @@ class Model:
         return needs
 
     def weight_bytes(self) -> int:
-        seen, total = set(), 0
-
-        def add(t):
-            nonlocal total
-            if isinstance(t, torch.Tensor) and t.data_ptr() not in seen:
-                seen.add(t.data_ptr())
-                total += t.numel() * t.element_size()
-
-        def walk(obj, depth=0):
-            if isinstance(obj, torch.Tensor):
-                add(obj)
-            elif depth < 4 and hasattr(obj, "__dict__"):
-                for v in vars(obj).values():
-                    if isinstance(v, (list, tuple)):
-                        for x in v:
-                            walk(x, depth + 1)
-                    elif isinstance(v, torch.Tensor) or hasattr(v, "__dict__"):
-                        if v is not self.env and not isinstance(v, (BuildEnv,)):
-                            walk(v, depth + 1)
-        add(self.embed_table)
-        for b in self.blocks:
-            walk(b)
-        walk(self.final_norm)
-        walk(self.head)
-        return total
+        """Bytes of all weights on the device, shared tensors counted once."""
+        parts = [self.embed_table, self.blocks, self.final_norm, self.head]
+        return sum(t.numel() * t.element_size() for t in part_tensors(parts))
 
     # ------------------------------------------------------------------ one step
     def forward(self, step) -> Optional[torch.Tensor]:

@@ -1,5 +1,5 @@
 """The parts a layer is put together from, and their registries."""
-from .base import BuildEnv, Workspace, lookup, register, registered
+from .base import BuildEnv, Workspace, lookup, part_tensors, register, registered
 from . import norm, position, attention, ffn, block  # noqa: F401  (registers the built-in kinds)
 from .attention import Attention
 from .block import PreNormBlock, SandwichBlock, add_pending_and_norm
@@ -8,6 +8,6 @@ from .linear import Linear
 from .norm import RmsNorm
 from .position import NoPosition, RotaryPosition
 
-__all__ = ["BuildEnv", "Workspace", "lookup", "register", "registered", "Attention", "GatedFfn",
+__all__ = ["BuildEnv", "Workspace", "lookup", "part_tensors", "register", "registered", "Attention", "GatedFfn",
            "Linear", "RmsNorm", "RotaryPosition", "NoPosition", "SandwichBlock", "PreNormBlock",
            "add_pending_and_norm"]

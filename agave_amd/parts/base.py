@@ -81,3 +81,26 @@ def lookup(category: str, kind: str) -> Callable:
 
 def registered(category: str) -> List[str]:
     return sorted(_REGISTRIES[category])
+
+
+def part_tensors(obj, _seen=None, _depth=0):
+    """Every device tensor a part (and the parts inside it) holds, each once."""
+    seen = _seen if _seen is not None else set()
+    if isinstance(obj, torch.Tensor):
+        if obj.data_ptr() not in seen:
+            seen.add(obj.data_ptr())
+            yield obj
+        return
+    if _depth > 6 or obj is None or isinstance(obj, (BuildEnv, Workspace, str, int, float, bool)):
+        return
+    if isinstance(obj, (list, tuple)):
+        for x in obj:
+            yield from part_tensors(x, seen, _depth + 1)
+        return
+    if isinstance(obj, dict):
+        for x in obj.values():
+            yield from part_tensors(x, seen, _depth + 1)
+        return
+    if hasattr(obj, "__dict__") and not hasattr(obj, "__dataclass_fields__"):
+        for v in vars(obj).values():
+            yield from part_tensors(v, seen, _depth + 1)

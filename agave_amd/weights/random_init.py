@@ -42,3 +42,23 @@ def write_random_model(raw_config: dict, seed: int, out_dir: str,
     with open(os.path.join(out_dir, "config.json"), "w", encoding="utf-8") as f:
         json.dump(raw_config, f, indent=1)
     return out_dir
+
+
+class RandomWeightSource:
+    """Random tensors made on the device, tensor by tensor, without a folder: for measurements,
+    where writing and reading back gigabytes would only cost time.  Same distributions as
+    :func:`random_tensors`; the values come from the device's generator."""
+
+    def __init__(self, needs, seed: int, device, dtype: torch.dtype = torch.bfloat16,
+                 std: float = 0.02, norm_std: float = 0.1):
+        self._needs = {n.name: (i, n) for i, n in enumerate(needs)}
+        self._seed, self._device, self._dtype = int(seed), device, dtype
+        self._std, self._norm_std = std, norm_std
+
+    def get(self, name: str) -> torch.Tensor:
+        i, need = self._needs[name]
+        g = torch.Generator(device=self._device).manual_seed((self._seed * 1_000_003 + i) & 0x7FFFFFFFFFFFFFFF)
+        s = self._norm_std if len(need.shape) == 1 else self._std
+        t = torch.empty(need.shape, dtype=torch.float32 if len(need.shape) == 1 else self._dtype, device=self._device)
+        t.normal_(0.0, s, generator=g)
+        return t

@@ -1,0 +1,197 @@
+"""Decode and prefill throughput of the Gemma 3 4B text decoder (random bf16 weights) on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one decode step of the whole batch: planning on the host, every kernel of the
+model, sampling (greedy) and the copy of the new token ids back to the host.  The default run
+has the layer sizes of BASELINE.json's configs[2], a batch of 8, prompts of 1,024 tokens and
+256 decoded tokens per sequence (W warm-up steps, then K timed ones).  One JSON line is
+printed: ``value`` is decoded tokens a second; ``prefill`` is one 2,048-token prompt;
+``roofline`` prices the decode step by the bytes it has to read (every weight once, and the
+cache of the live requests) against 8 TB/s; ``points`` holds decode at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+# BASELINE.json configs[2]: Gemma 3 4B text decoder
+GEMMA3_4B = dict(
+    architectures=["Gemma3ForCausalLM"], model_type="gemma3_text", vocab_size=262208, hidden_size=2560,
+    num_hidden_layers=34, num_attention_heads=8, num_key_value_heads=4, head_dim=256,
+    query_pre_attn_scalar=256, intermediate_size=10240, sliding_window=1024, sliding_window_pattern=6,
+    rope_theta=1e6, rope_local_base_freq=1e4, rope_scaling={"rope_type": "linear", "factor": 8.0},
+    rms_norm_eps=1e-6, tie_word_embeddings=True, hidden_activation="gelu_pytorch_tanh",
+    max_position_embeddings=131072, bos_token_id=2, eos_token_id=1)
+
+PROMPT_LEN, DECODE_LEN, CONTEXT, PREFILL_LEN = 1024, 256, 4096, 2048
+
+
+def model_numbers(cfg: dict, n_layers: int):
+    e, nh, nkv, hd = cfg["hidden_size"], cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    ff, v = cfg["intermediate_size"], cfg["vocab_size"]
+    qd, kvd = nh * hd, nkv * hd
+    pattern = cfg["sliding_window_pattern"]
+    sliding = [(i + 1) % pattern != 0 for i in range(n_layers)]
+    per_layer = e * (qd + 2 * kvd) + qd * e + 3 * e * ff
+    norms = n_layers * (4 * e + 2 * hd) + e
+    return dict(e=e, qd=qd, kvd=kvd, ff=ff, v=v, sliding=sliding, window=cfg["sliding_window"],
+                linear_params=per_layer * n_layers, table_params=v * e, norm_params=norms)
+
+
+def decode_step_bytes(m: dict, contexts) -> float:
+    """Bytes one decode step has to read: every weight once (bf16; the tied table once, as the
+    output matrix; norm gains in 32-bit) and the keys and values each live request attends to."""
+    weights = 2 * (m["linear_params"] + m["table_params"]) + 4 * m["norm_params"]
+    kv = 0
+    for ctx in contexts:
+        for s in m["sliding"]:
+            kv += (min(ctx, m["window"]) if s else ctx) * m["kvd"] * 2 * 2
+    return float(weights + kv)
+
+
+def prefill_flops(m: dict, t: int) -> float:
+    """Multiply-adds of one prompt of t tokens, twice: the linear layers on every token, the
+    output matrix on the one wanted row, and attention over the visible pairs."""
+    linear = 2.0 * t * m["linear_params"] + 2.0 * m["table_params"]
+    attn = 0.0
+    for s in m["sliding"]:
+        pairs = sum(min(i + 1, m["window"]) for i in range(t)) if s else t * (t + 1) // 2
+        attn += 4.0 * m["qd"] * pairs
+    return linear + attn
+
+
+def random_prompts(n: int, length: int, vocab: int, seed: int):
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, vocab, size=length).tolist() for _ in range(n)]
+
+
+def run_decode(engine, batch: int, steps: int, warmup: int, seed: int):
+    """Prefill ``batch`` prompts of PROMPT_LEN tokens, then time ``steps`` decode steps."""
+    import torch
+    from agave_amd.engine.generate import RowSampling
+    prompts = random_prompts(batch, PROMPT_LEN, engine.vocab_size, seed)
+    slots = [engine.alloc_slot() for _ in range(batch)]
+    rows = [RowSampling(0.0, 0, 1.0, 1.0, 0.0, []) for _ in range(batch)]
+    try:
+        engine.prefill_chunk = 2048 if batch > 8 else 0
+        if batch > 8:                       # keep the untimed prefill's workspace small
+            toks = None
+            for i in range(0, batch, 8):
+                part = engine.step_sample(slots[i:i + 8], prompts[i:i + 8], rows[i:i + 8])
+                toks = part if toks is None else toks + part
+        else:
+            toks = engine.step_sample(slots, prompts, rows)
+        for _ in range(warmup):
+            toks = engine.step_sample(slots, [[t] for t in toks], rows)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            toks = engine.step_sample(slots, [[t] for t in toks], rows)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        first_ctx = PROMPT_LEN + warmup + 1          # keys the first timed step attends to
+        contexts = [first_ctx + (steps - 1) / 2.0] * batch
+        return dt, contexts
+    finally:
+        for s in slots:
+            engine.free_slot(s)
+        engine.prefill_chunk = 0
+
+
+def run_prefill(engine, seed: int, repeats: int = 3):
+    import torch
+    from agave_amd.engine.generate import RowSampling
+    prompt = random_prompts(1, PREFILL_LEN, engine.vocab_size, seed)
+    row = [RowSampling(0.0, 0, 1.0, 1.0, 0.0, [])]
+    times = []
+    for r in range(repeats + 1):                     # the first pass warms up
+        slot = engine.alloc_slot()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step_sample([slot], prompt, row)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.free_slot(slot)
+        if r > 0:
+            times.append(dt)
+    return min(times)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=240)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=GEMMA3_4B["num_hidden_layers"],
+                    help="run fewer layers of the same sizes (reported in config)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    args = ap.parse_args()
+    world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.gpus != 1 or world != 1:
+        if int(os.environ.get("RANK", "0")) == 0:
+            print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    if args.steps + args.warmup > CONTEXT - PROMPT_LEN:
+        ap.error(f"--steps + --warmup must stay within {CONTEXT - PROMPT_LEN} decoded tokens")
+
+    import torch
+    from agave_amd.engine import Engine
+
+    cfg = dict(GEMMA3_4B, num_hidden_layers=args.layers)
+    m = model_numbers(cfg, args.layers)
+    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    per_seq = -(-(PROMPT_LEN + DECODE_LEN + 64) // 64) * 64
+    cache_tokens = max(max_batch * per_seq, -(-PREFILL_LEN // 64) * 64 + 64)
+    engine = Engine.from_random(cfg, seed=0, dtype=args.dtype, max_slots=max_batch, max_context=CONTEXT,
+                                cache_tokens=cache_tokens, device="cuda:0")
+    dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
+
+    dt, contexts = run_decode(engine, args.batch, args.steps, args.warmup, seed=1)
+    ms_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    need = decode_step_bytes(m, contexts)
+    achieved = need / (ms_step * 1e-3) / 1e9
+    out = {
+        "metric": "decode tok/s, Gemma3-4B bf16, batch 8, 1024-token prompts + 256 decoded",
+        "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dkey, "data": "synthetic: uniform-random token ids, random N(0,0.02) weights",
+        "config": {"model": "gemma3-4b-text", "layers": args.layers, "layers_of_config": GEMMA3_4B["num_hidden_layers"],
+                   "hidden": m["e"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+                   "head_dim": cfg["head_dim"], "intermediate": m["ff"], "vocab": m["v"],
+                   "sliding_window": m["window"], "sliding_pattern": cfg["sliding_window_pattern"],
+                   "global_batch": args.batch, "seq_len": PROMPT_LEN + DECODE_LEN, "prompt_len": PROMPT_LEN,
+                   "context": CONTEXT, "prefill_len": PREFILL_LEN, "parallelism": "single GPU",
+                   "sampling": "greedy", "weights_gb": round(2 * (m["linear_params"] + m["table_params"]) / 1e9, 3)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        pdt = run_prefill(engine, seed=2)
+        flops = prefill_flops(m, PREFILL_LEN)
+        out["prefill"] = {"value": round(PREFILL_LEN / pdt, 1), "tokens": PREFILL_LEN, "ms": round(pdt * 1e3, 3),
+                          "frac": round(flops / pdt / PEAK_FLOPS[dkey], 4)}
+        points = {}
+        for b, k in ((1, 64), (64, 32)):
+            d, _ = run_decode(engine, b, k, 8, seed=3 + b)
+            points[f"decode_b{b}"] = round(b * k / d, 2)
+        out["points"] = points
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
