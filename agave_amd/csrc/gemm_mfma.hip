@@ -1,0 +1,260 @@
+// bfloat16 matrix products on the matrix cores of gfx950: Y[M,N] = X[M,K] * W[N,K]^T with
+// 32-bit accumulation, W in the packed layout of mfma.h.
+//
+//  * pack_w16: row-major W -> packed tiles (optionally interleaving the rows of a stacked
+//    [gate; up] matrix so that one lane ends up with gate and up of the same column);
+//  * embed_scale_packed: the embedding gather reading rows out of a packed table (tied head);
+//  * gemm_skinny: M <= 64 tokens (decode): the weight streams through once at memory speed,
+//    K is split over the four waves of a workgroup, partial sums meet in LDS;
+//  * gemm_tiled: large M (prefill): 128x128 tiles per workgroup, X staged through LDS.
+//
+// The reference computes the same products row by row: one workgroup per output row with a
+// block reduction (src/backend/kernels/rocm/gemv_bf16.zig:6-24), looped over tokens for a
+// batch (src/backend/rocm.zig:1177-1190).
+#include "common_impl.h"
+#include "mfma.h"
+
+// ------------------------------------------------------------------ packing
+// mode 0: packed row p is source row p.
+// mode 1: the source is [gate (ff rows); up (ff rows)]; within a block of 16 packed rows, rows
+//         4q+0, 4q+1 are gate[8nb+2q], gate[8nb+2q+1] and rows 4q+2, 4q+3 the same two of up.
+__global__ void pack_w16_kernel(const bf16* __restrict__ W, long ldw, uint4* __restrict__ P, int N, int K,
+                                int NB, int KB, int mode, int ff) {
+    const long tile = blockIdx.x;          // nb * KB + kb
+    const int nb = (int)(tile / KB), kb = (int)(tile % KB);
+    const int lane = threadIdx.x;
+    const int i = lane & 15, g = lane >> 4;
+    long src = -1;
+    if (mode == 0) {
+        const int p = nb * 16 + i;
+        if (p < N) src = p;
+    } else {
+        const int q = i >> 2, e = i & 3;
+        const int col = 8 * nb + 2 * q + (e & 1);
+        if (col < ff) src = (e < 2) ? col : (long)ff + col;
+    }
+    frag16 f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int k = kb * 32 + g * 8 + e;
+        bf16 z;
+        z.x = 0;
+        f.h[e] = (src >= 0 && k < K) ? W[src * ldw + k] : z;
+    }
+    P[tile * 64 + lane] = f.u;
+}
+
+extern "C" int agave_pack_w16(const void* W, long ldw, void* P, int N, int K, int mode, int ff, hipStream_t stream) {
+    AGAVE_CHECK(N > 0 && K > 0 && ldw >= K, "pack_w16: bad sizes N=%d K=%d ldw=%ld", N, K, ldw);
+    AGAVE_CHECK(mode == 0 || (mode == 1 && N == 2 * ff), "pack_w16: interleaved mode needs N == 2*ff");
+    const int rows = mode == 0 ? N : ff * 2;
+    const int NB = mode == 0 ? (N + 15) / 16 : (ff + 7) / 8;
+    const int KB = (K + 31) / 32;
+    (void)rows;
+    AGAVE_CHECK((long)NB * KB < 2147483647L, "pack_w16: too many tiles");
+    pack_w16_kernel<<<NB * KB, 64, 0, stream>>>((const bf16*)W, ldw, (uint4*)P, N, K, NB, KB, mode, ff);
+    AGAVE_LAUNCH_CHECK("pack_w16");
+    return 0;
+}
+
+// ------------------------------------------------------------------ embedding from a packed table
+__global__ void embed_scale_packed_kernel(const int* __restrict__ tokens, const uint4* __restrict__ P, float scale,
+                                          float* __restrict__ out, int e, int vocab, int KB) {
+    const int t = blockIdx.x;
+    int tok = tokens[t];
+    tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
+    const int nb = tok >> 4, i = tok & 15;
+    float* o = out + (size_t)t * e;
+    for (int piece = threadIdx.x; piece * 8 < e; piece += blockDim.x) {     // 8 columns per piece
+        const int kb = piece >> 2, g = piece & 3;
+        frag16 f;
+        f.u = P[((size_t)nb * KB + kb) * 64 + i + 16 * g];
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+            const int k = piece * 8 + x;
+            if (k < e) o[k] = bf16_to_f32(f.h[x]) * scale;
+        }
+    }
+}
+
+extern "C" int agave_embed_scale_packed(const int* tokens, const void* P, float scale, float* out, int n_tokens,
+                                        int e, int vocab, hipStream_t stream) {
+    AGAVE_CHECK(n_tokens >= 0 && e > 0 && vocab > 0, "embed_scale_packed: bad sizes");
+    if (n_tokens == 0) return 0;
+    embed_scale_packed_kernel<<<n_tokens, 64, 0, stream>>>(tokens, (const uint4*)P, scale, out, e, vocab, (e + 31) / 32);
+    AGAVE_LAUNCH_CHECK("embed_scale_packed");
+    return 0;
+}
+
+// ------------------------------------------------------------------ skinny product (decode)
+__device__ __forceinline__ float gelu_tanh_f(float x) {
+    const float c = 0.7978845608028654f;
+    return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
+}
+
+#define SK_KS 4                    // k-steps (tiles of 32 columns) per chunk
+#define SK_ROW (SK_KS * 32 + 8)    // bf16 per staged X row: 128 columns + 16 bytes of padding
+
+// R: row blocks (of 16 weight rows) per workgroup; MT: tiles of 16 tokens; EPI 0: store, 1: GeGLU.
+template <int R, int MT, int EPI, typename TC>
+__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict__ X, long ldx,
+                                                          const uint4* __restrict__ Wp, TC* __restrict__ Y,
+                                                          long ldy, int M, int N, int K, int KB, int NB) {
+    // staged X: [wave][MT][16 rows][SK_ROW]; afterwards the same memory holds the waves' partial sums
+    constexpr int XS_WAVE = MT * 16 * SK_ROW;                       // bf16 elements
+    constexpr int RED_WAVE = R * MT * 64 * 4;                       // floats
+    constexpr int LDS_BYTES = (4 * XS_WAVE * 2 > 4 * RED_WAVE * 4) ? 4 * XS_WAVE * 2 : 4 * RED_WAVE * 4;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
+    bf16* xs = reinterpret_cast<bf16*>(smem);
+    float* red = reinterpret_cast<float*>(smem);
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int j = lane & 15, g = lane >> 4;
+    const int nb0 = blockIdx.x * R;
+    const int n_chunks = (KB + SK_KS - 1) / SK_KS;
+    const int n_iter = (n_chunks + 3) / 4;
+
+    f32x4_t acc[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[r][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    frag16 wreg[R][SK_KS];
+    uint4 xreg[MT][4];
+    bf16* my_xs = xs + wave * XS_WAVE;
+
+    auto load_global = [&](int it) {
+        const int c = it * 4 + wave;                 // chunks are dealt to the waves in turn
+        const bool active = c < n_chunks;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int ks = 0; ks < SK_KS; ++ks) {
+                const int kb = c * SK_KS + ks;
+                if (active && kb < KB && nb0 + r < NB)
+                    wreg[r][ks].u = Wp[((size_t)(nb0 + r) * KB + kb) * 64 + lane];
+                else
+                    wreg[r][ks].u = uint4{0, 0, 0, 0};
+            }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = mt * 16 + 4 * i + g;              // 4 rows per instruction, 16 lanes a row
+                const int k = c * (SK_KS * 32) + j * 8;
+                if (active && row < M && k < K)
+                    xreg[mt][i] = *reinterpret_cast<const uint4*>(X + (size_t)row * ldx + k);
+                else
+                    xreg[mt][i] = uint4{0, 0, 0, 0};
+            }
+    };
+
+    load_global(0);
+    for (int it = 0; it < n_iter; ++it) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<uint4*>(my_xs + (mt * 16 + 4 * i + g) * SK_ROW + j * 8) = xreg[mt][i];
+        frag16 wcur[R][SK_KS];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int ks = 0; ks < SK_KS; ++ks) wcur[r][ks] = wreg[r][ks];
+        if (it + 1 < n_iter) load_global(it + 1);
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < SK_KS; ++ks)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                frag16 xb;
+                xb.u = *reinterpret_cast<const uint4*>(my_xs + (mt * 16 + j) * SK_ROW + ks * 32 + g * 8);
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r][mt] = mfma_16x16x32(wcur[r][ks], xb, acc[r][mt]);
+            }
+        __syncthreads();
+    }
+
+    // the four waves' partial sums meet in LDS
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            *reinterpret_cast<f32x4_t*>(red + ((size_t)wave * R * MT + r * MT + mt) * 256 + lane * 4) = acc[r][mt];
+    __syncthreads();
+    for (int tile = wave; tile < R * MT; tile += 4) {
+        const int r = tile / MT, mt = tile % MT;
+        f32x4_t s = *reinterpret_cast<const f32x4_t*>(red + (size_t)tile * 256 + lane * 4);
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const f32x4_t p = *reinterpret_cast<const f32x4_t*>(red + ((size_t)w * R * MT + tile) * 256 + lane * 4);
+            s += p;
+        }
+        const int m = mt * 16 + j;
+        if (m >= M || nb0 + r >= NB) continue;
+        if (EPI == 0) {
+            const int n = (nb0 + r) * 16 + g * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < N) st(Y + (size_t)m * ldy + n + e, s[e]);
+        } else {
+            const int n = (nb0 + r) * 8 + g * 2;      // N counts output columns (ff)
+            if (n < N) st(Y + (size_t)m * ldy + n, gelu_tanh_f(s[0]) * s[2]);
+            if (n + 1 < N) st(Y + (size_t)m * ldy + n + 1, gelu_tanh_f(s[1]) * s[3]);
+        }
+    }
+}
+
+template <int R, int MT, int EPI, typename TC>
+static void launch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
+                          int NB, hipStream_t stream) {
+    const int grid = (NB + R - 1) / R;
+    gemm_skinny_kernel<R, MT, EPI, TC><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy, M,
+                                                                N, K, KB, NB);
+}
+
+template <int EPI, typename TC>
+static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
+                           int NB, hipStream_t stream) {
+    const int mt = (M + 15) / 16;
+    // two row blocks per workgroup once there are plenty of them, so that X is staged half as often
+    const bool wide = NB >= 4096;
+#define SK_CASE(R_, MT_)                                                                        \
+    launch_skinny<R_, MT_, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);              \
+    break
+    switch (mt) {
+        case 1: if (wide) { SK_CASE(2, 1); } else { SK_CASE(1, 1); }
+        case 2: if (wide) { SK_CASE(2, 2); } else { SK_CASE(1, 2); }
+        case 3: if (wide) { SK_CASE(2, 3); } else { SK_CASE(1, 3); }
+        case 4: if (wide) { SK_CASE(2, 4); } else { SK_CASE(1, 4); }
+        default: AGAVE_CHECK(false, "gemm_skinny: M=%d exceeds 64", M);
+    }
+#undef SK_CASE
+    return 0;
+}
+
+// N: logical outputs (rows of W, or ff for the GeGLU epilogue); Wp holds NB row blocks.
+extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,
+                                 int K, int epilogue, hipStream_t stream) {
+    AGAVE_CHECK(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d (M <= 64)", M, N, K);
+    AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
+                "gemm_skinny: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
+    AGAVE_CHECK(ldx >= K && ldy >= N, "gemm_skinny: a row stride is too small");
+    AGAVE_CHECK(epilogue == 0 || epilogue == 1, "gemm_skinny: unknown epilogue %d", epilogue);
+    if (M == 0) return 0;
+    const int KB = (K + 31) / 32;
+    const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
+    int rc;
+    if (epilogue == 0) {
+        if (dt_y == AGAVE_BF16) rc = dispatch_skinny<0, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        else if (dt_y == AGAVE_F32) rc = dispatch_skinny<0, float>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        else AGAVE_CHECK(false, "gemm_skinny: unknown output dtype %d", dt_y);
+    } else {
+        AGAVE_CHECK(dt_y == AGAVE_BF16, "gemm_skinny: the GeGLU epilogue writes bfloat16");
+        rc = dispatch_skinny<1, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    }
+    if (rc != 0) return rc;
+    AGAVE_LAUNCH_CHECK("gemm_skinny");
+    return 0;
+}

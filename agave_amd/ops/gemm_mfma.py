@@ -1,9 +1,62 @@
-"""Matrix-core (MFMA) matrix products for bfloat16.  Filled in after the plain path."""
+"""Matrix-core (MFMA) matrix products for bfloat16 weights in the packed layout."""
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
+
+from . import kernels, library
+from .kernels import _F, _I, _L, _P
+
+kernels.register_signatures("gemm_mfma", {
+    "agave_pack_w16": [_P, _L, _P, _I, _I, _I, _I, _P],
+    "agave_embed_scale_packed": [_P, _P, _F, _P, _I, _I, _I, _P],
+    "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P],
+})
+
+SKINNY_MAX_M = 64
+
+
+def pack_weight(weight: torch.Tensor, interleave_ff: int = 0) -> torch.Tensor:
+    """Row-major bfloat16 W[N, K] -> packed tiles of 16 rows by 32 columns (a flat bfloat16
+    tensor).  ``interleave_ff`` > 0: W is a stacked [gate; up] matrix of 2*ff rows whose rows are
+    interleaved for the GeGLU epilogue."""
+    if not weight.is_cuda or weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.stride(1) != 1:
+        raise TypeError("pack_weight takes a bfloat16 GPU matrix with contiguous rows")
+    n, k = weight.shape
+    nb = (interleave_ff + 7) // 8 if interleave_ff else (n + 15) // 16
+    kb = (k + 31) // 32
+    packed = torch.empty(nb * kb * 512, dtype=torch.bfloat16, device=weight.device)
+    library.call(kernels.lib("gemm_mfma"), "agave_pack_w16", weight.data_ptr(), weight.stride(0), packed.data_ptr(),
+                 n, k, 1 if interleave_ff else 0, interleave_ff, kernels.stream())
+    return packed
+
+
+def _x_ok(x: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.shape[1] % 8 == 0
+            and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0)
+
+
+def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, epilogue: int = 0) -> None:
+    """out[M, n_out] = x[M, K] @ W^T (epilogue 0) or gelu_tanh(gate) * up (epilogue 1) for M <= 64."""
+    if not (x.is_cuda and packed.is_cuda and out.is_cuda):
+        raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
+    m, k = x.shape
+    if not _x_ok(x):
+        raise ValueError("skinny product: x must be bfloat16, 16-byte aligned, K and row stride multiples of 8")
+    if out.dim() != 2 or out.shape != (m, n_out) or out.stride(1) != 1:
+        raise ValueError(f"skinny product: out must be [{m}, {n_out}] with contiguous rows")
+    nb = (n_out + 7) // 8 if epilogue else (n_out + 15) // 16
+    if packed.numel() != nb * ((k + 31) // 32) * 512:
+        raise ValueError("skinny product: the packed weight does not fit these sizes")
+    library.call(kernels.lib("gemm_mfma"), "agave_gemm_skinny", x.data_ptr(), x.stride(0), packed.data_ptr(),
+                 kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue, kernels.stream())
 
 
 def try_linear(x: torch.Tensor, lin, out: torch.Tensor) -> bool:
     """Run the product on the matrix cores if a kernel takes these sizes; False otherwise."""
-    return False
+    packed = getattr(lin, "packed", None)
+    if packed is None or x.shape[0] > SKINNY_MAX_M or not _x_ok(x):
+        return False
+    skinny(x, packed, out, lin.out_features, 0)
+    return True

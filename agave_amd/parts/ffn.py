@@ -27,6 +27,11 @@ class GatedFfn:
         self.env = env
         self.gate_up = Linear([weights.get(spec.gate_proj), weights.get(spec.up_proj)], env, "gate_up")
         self.down = Linear([weights.get(spec.down_proj)], env, "ffn_down")
+        self.gate_up_fused = None   # [gate; up] with interleaved rows, for the product that ends in GeGLU
+        if self.gate_up.packed is not None:
+            from ..ops import gemm_mfma
+            self.gate_up_fused = gemm_mfma.pack_weight(self.gate_up.weight, interleave_ff=spec.intermediate)
+            self.gate_up.packed = None
 
     @staticmethod
     def tensor_needs(spec: GatedFfnSpec) -> List[TensorNeed]:
@@ -37,9 +42,13 @@ class GatedFfn:
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
         ff = self.spec.intermediate
         n = x.shape[0]
-        gu = self.gate_up.forward(x, tag="gate_up")
         act = self.env.workspace.get("ffn_act", n, ff, x.dtype)
-        kernels.geglu(gu[:, :ff], gu[:, ff:], act)
+        if self.gate_up_fused is not None and n <= 64 and x.dtype == torch.bfloat16:
+            from ..ops import gemm_mfma
+            gemm_mfma.skinny(x, self.gate_up_fused, act, ff, epilogue=1)
+        else:
+            gu = self.gate_up.forward(x, tag="gate_up")
+            kernels.geglu(gu[:, :ff], gu[:, ff:], act)
         return self.down.forward(act, tag="ffn_down")
 
 

@@ -33,7 +33,10 @@ class Linear:
         self.out_features, self.in_features = self.weight.shape
         self.env = env
         self.name = name
-        self.packed = None          # set by the matrix-core module when it repacks the weight
+        self.packed = None          # the weight in the matrix cores' tile layout (bfloat16 engines)
+        if env.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16:
+            from ..ops import gemm_mfma
+            self.packed = gemm_mfma.pack_weight(self.weight)
 
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, tag: Optional[str] = None) -> torch.Tensor:

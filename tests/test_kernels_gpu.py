@@ -334,3 +334,48 @@ def test_repeat_penalty(S):
 def test_cpu_tensors_are_refused(K):
     with pytest.raises(RuntimeError, match="GPU"):
         K.gemm_plain(torch.zeros(2, 2), torch.zeros(2, 2), torch.zeros(2, 2))
+
+
+# ---------------------------------------------------------------- matrix-core products
+@pytest.fixture(scope="module")
+def G():
+    from agave_amd.ops import gemm_mfma
+    return gemm_mfma
+
+
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 40, 64])
+@pytest.mark.parametrize("n,k", [(53, 72), (256, 2560), (1000, 96), (4100, 136), (160, 10240)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_skinny(G, m, n, k, out_dtype):
+    g = torch.Generator().manual_seed(m * 1000 + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    packed = G.pack_weight(w.to(DEV))
+    out = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+    G.skinny(x.to(DEV), packed, out, n)
+    ref = x.double() @ w.double().T
+    scale = float(ref.abs().max())
+    tol = 2e-5 * scale * math.sqrt(k / 64) if out_dtype == torch.float32 else 6e-3 * scale
+    assert float((out.cpu().double() - ref).abs().max()) <= tol
+
+
+@pytest.mark.parametrize("m,ff,k", [(1, 192, 64), (8, 1000, 96), (33, 10240, 256), (64, 20, 40)])
+def test_gemm_skinny_geglu(G, m, ff, k):
+    g = torch.Generator().manual_seed(ff + m)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(2 * ff, k, generator=g) * 0.2).bfloat16()
+    packed = G.pack_weight(w.to(DEV), interleave_ff=ff)
+    out = torch.full((m, ff), float("nan"), dtype=torch.bfloat16, device=DEV)
+    G.skinny(x.to(DEV), packed, out, ff, epilogue=1)
+    gu = x.double() @ w.double().T
+    ref = P.gelu_tanh(gu[:, :ff]) * gu[:, ff:]
+    assert float((out.cpu().double() - ref).abs().max()) <= 8e-3 * float(ref.abs().max())
+
+
+def test_gemm_skinny_refuses_what_it_cannot_do(G):
+    w = G.pack_weight(torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV))
+    out = torch.empty(65, 32, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(Exception, match="64"):
+        G.skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w, out, 32)
+    with pytest.raises(ValueError):
+        G.skinny(torch.zeros(4, 60, dtype=torch.bfloat16, device=DEV), w, out[:4], 32)   # K no multiple of 8
