@@ -69,13 +69,18 @@ class KVCache:
         self.groups: List[GroupPages] = [GroupPages(k, pages_per_group[k], max_slots) for k in self.group_keys]
         self.k_store: List[Optional[torch.Tensor]] = []
         self.v_store: List[Optional[torch.Tensor]] = []
-        for key, mems in zip(self.group_keys, members):
+        # bfloat16 groups whose head size is a multiple of 16 (up to 256) keep their pages in the
+        # matrix cores' tile order; the others row by row
+        self.packed: List[bool] = [dtype == torch.bfloat16 and k.head_dim % 16 == 0 and k.head_dim <= 256
+                                   for k in self.group_keys]
+        for key, mems, packed in zip(self.group_keys, members, self.packed):
             n = pages_per_group[key]
+            hd_k = (key.head_dim + 31) // 32 * 32 if packed else key.head_dim
             if device is None:
                 self.k_store.append(None)
                 self.v_store.append(None)
             else:
-                self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, key.head_dim), dtype=dtype, device=device))
+                self.k_store.append(torch.zeros((len(mems), n, key.n_kv_heads, PAGE, hd_k), dtype=dtype, device=device))
                 self.v_store.append(torch.zeros((len(mems), n, key.n_kv_heads, key.head_dim, PAGE), dtype=dtype, device=device))
         self.state_needs = dict(state_needs)
         self.state: Dict[int, Optional[torch.Tensor]] = {}
@@ -142,10 +147,10 @@ class KVCache:
                 g.commit(s, self.slots.length[s])
 
     # ------------------------------------------------------------------ storage
-    def pages_of(self, memory: int) -> Tuple[torch.Tensor, torch.Tensor]:
-        """(K pages, V pages) of one memory."""
+    def pages_of(self, memory: int) -> Tuple[torch.Tensor, torch.Tensor, bool]:
+        """(K pages, V pages, whether they are in the matrix cores' tile order) of one memory."""
         g, i = self.group_of_memory[memory], self.index_in_group[memory]
-        return self.k_store[g][i], self.v_store[g][i]
+        return self.k_store[g][i], self.v_store[g][i], self.packed[g]
 
     def bytes(self) -> int:
         total = 0

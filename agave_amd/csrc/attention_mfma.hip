@@ -1,0 +1,397 @@
+// bfloat16 attention over the paged cache on the matrix cores of gfx950 (head sizes in steps
+// of 16 up to 256): a decode kernel that splits a sequence's keys over workgroups
+// (flash-decoding) with a combine pass, and a prefill kernel for steps that bring many tokens.
+// Scores, the running maximum and sum, and the output accumulate in 32-bit; probabilities
+// are rounded to bfloat16 only as the operand of the P*V product.
+//
+// Reference for the arithmetic: src/backend/kernels/cpu/sdpa.zig:34-88, 184-234 (scores *
+// scale, max-subtracted softmax, weighted sum of V); window bounds as
+// src/ops/attention.zig:92-93 (a query at position p sees keys max(0, p-W+1) .. p).  The
+// reference's GPU kernel keeps one workgroup per head with all scores in LDS
+// (src/backend/kernels/rocm/sdpa.zig:99-184) and skips probabilities below 1e-6; nothing is
+// skipped here.
+//
+// Packed cache pages (64 positions).  With KS = ceil(hd/32) and the MFMA layouts of mfma.h:
+//   K page: tiles [kt 0..3][ks 0..KS-1], tile = 64 lanes x 8: lane (i, g) element e holds
+//           K[16*kt + i][32*ks + 8*g + e]   (zero where the column is >= hd)
+//   V page: tiles [dt 0..hd/16-1][s 0..1]:  lane (j, g) element e holds V[key][16*dt + j] with
+//           key = 32*s + (e < 4 ? 4*g + e : 16 + 4*g + e - 4)
+// The odd order of V's keys is the order in which a lane holds the scores of two 16-key tiles
+// after S^T = K * Q^T, so probabilities go into the P*V product without leaving their lane.
+#include "common_impl.h"
+#include "mfma.h"
+#include <math.h>
+
+#define QT_MAX 4        // most q tiles (of 16 query slots) a wave takes
+
+struct AttnArgs {
+    const bf16* q;
+    long ldq;
+    bf16* out;
+    long ldo;
+    float* part_o;       // [token][head][split][hd]   (decode with splits)
+    float* part_ml;      // [token][head][split][2]
+    const uint4* k_pages;
+    const uint4* v_pages;
+    const int* table;
+    int width;
+    const int* base;
+    int n_pages;
+    const int* tok_seq;
+    const int* tok_pos;
+    const int* cu;       // prefill: first token of each sequence in the step
+    int n_seqs;
+    int nh, nkv, hd;
+    float scale;
+    int window;
+    int splits, pages_per_split;
+};
+
+// One wave: QT tiles of 16 query slots against the pages [page_lo, page_hi] of one sequence
+// and kv head.  Slot j of tile t has position pos[t] (per lane: the lane's column j = lane%16)
+// and sees keys lo[t] .. pos[t].
+template <int HDT, int QT_MAX_>
+struct WaveAttn {
+    static constexpr int KS = (HDT + 1) / 2;
+    static constexpr int QTM = QT_MAX_;
+    f32x4_t o[QTM][HDT];
+    float m[QTM], l[QTM];
+    frag16 qf[QTM][KS];
+
+    __device__ __forceinline__ void init(int qt) {
+#pragma unroll
+        for (int t = 0; t < QTM; ++t) {
+            m[t] = -INFINITY;
+            l[t] = 0.f;
+#pragma unroll
+            for (int d = 0; d < HDT; ++d) o[t][d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+        (void)qt;
+    }
+
+    // q_row[t]: pointer to the head's hd values of this lane's slot in tile t, or null
+    __device__ __forceinline__ void load_q(const bf16* const* q_row, int qt, int hd, int lane) {
+        const int g = lane >> 4;
+#pragma unroll
+        for (int t = 0; t < QTM; ++t)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int d0 = 32 * ks + 8 * g;
+                if (t < qt && q_row[t] != nullptr && d0 < hd)
+                    qf[t][ks].u = *reinterpret_cast<const uint4*>(q_row[t] + d0);
+                else
+                    qf[t][ks].u = uint4{0, 0, 0, 0};
+            }
+    }
+
+    __device__ __forceinline__ void page(const uint4* __restrict__ kp, const uint4* __restrict__ vp, int page_idx,
+                                         int qt, int hd, float scale, const int* pos, const int* lo, int lane) {
+        const int g = lane >> 4;
+        const int hdt = hd >> 4, ks_n = (hd + 31) >> 5;
+        f32x4_t st[QTM][4];
+#pragma unroll
+        for (int t = 0; t < QTM; ++t)
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) st[t][kt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        // S^T = K * Q^T: rows are keys, columns are query slots
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                if (ks < ks_n) {
+                    frag16 a;
+                    a.u = kp[(kt * ks_n + ks) * 64 + lane];
+#pragma unroll
+                    for (int t = 0; t < QTM; ++t)
+                        if (t < qt) st[t][kt] = mfma_16x16x32(a, qf[t][ks], st[t][kt]);
+                }
+            }
+        frag16 pf[QTM][2];
+        float alpha[QTM];
+#pragma unroll
+        for (int t = 0; t < QTM; ++t) {
+            if (t >= qt) continue;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int key = page_idx * AGAVE_PAGE + kt * 16 + 4 * g + e;
+                    float s = st[t][kt][e] * scale;
+                    if (key > pos[t] || key < lo[t]) s = -INFINITY;
+                    st[t][kt][e] = s;
+                    mx = fmaxf(mx, s);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m[t], mx);
+            const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;   // a slot may see no key of this page
+            alpha[t] = __expf(m[t] - m_safe);
+            m[t] = m_new;
+            float sum = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float pe = __expf(st[t][kt][e] - m_safe);
+                    sum += pe;
+                    pf[t][kt >> 1].h[(kt & 1) * 4 + e] = f32_to_bf16(pe);
+                }
+            l[t] = l[t] * alpha[t] + sum;       // this lane's share; the four lanes of a column meet at the end
+        }
+        // the output's rows are query slots 4*(lane/16) + e: fetch their factors from the columns
+#pragma unroll
+        for (int t = 0; t < QTM; ++t) {
+            if (t >= qt) continue;
+            float a4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a4[e] = __shfl(alpha[t], 4 * g + e, 64);
+#pragma unroll
+            for (int d = 0; d < HDT; ++d)
+                if (d < hdt) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[t][d][e] *= a4[e];
+                }
+        }
+        // O += P * V
+#pragma unroll
+        for (int d = 0; d < HDT; ++d)
+            if (d < hdt) {
+#pragma unroll
+                for (int s = 0; s < 2; ++s) {
+                    frag16 b;
+                    b.u = vp[(d * 2 + s) * 64 + lane];
+#pragma unroll
+                    for (int t = 0; t < QTM; ++t)
+                        if (t < qt) o[t][d] = mfma_16x16x32(pf[t][s], b, o[t][d]);
+                }
+            }
+    }
+
+    __device__ __forceinline__ void finish_sums(int qt) {
+#pragma unroll
+        for (int t = 0; t < QTM; ++t)
+            if (t < qt) {
+                l[t] += __shfl_xor(l[t], 16, 64);
+                l[t] += __shfl_xor(l[t], 32, 64);
+            }
+    }
+};
+
+__device__ __forceinline__ long page_of(const AttnArgs& a, int b, int page_idx) {
+    const int col = page_idx - a.base[b];
+    if (col < 0 || col >= a.width) return -1;
+    const long pg = a.table[(size_t)b * a.width + col];
+    return (pg < 0 || pg >= a.n_pages) ? -1 : pg;
+}
+
+// ------------------------------------------------------------------ decode: one token per (z), splits over keys
+// grid (split, kv head * head chunks, token); one wave per workgroup.  Query slots are the
+// heads of the group (16 per chunk).
+template <int HDT>
+__global__ __launch_bounds__(64) void attn_decode_mfma_kernel(AttnArgs a) {
+    const int lane = threadIdx.x, j = lane & 15, g = lane >> 4;
+    const int G = a.nh / a.nkv;
+    const int chunks = (G + 15) / 16;
+    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int t = blockIdx.z, split = blockIdx.x;
+    const int b = a.tok_seq[t], p = a.tok_pos[t];
+    const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
+    const int first = lo / AGAVE_PAGE, last = p / AGAVE_PAGE;
+    const int page_lo = first + split * a.pages_per_split;
+    int page_hi = page_lo + a.pages_per_split - 1;
+    if (page_hi > last) page_hi = last;
+    const int hd = a.hd, hdt = hd >> 4;
+    const int head_j = kvh * G + chunk * 16 + j;                 // this lane's column as a head
+    const bool col_ok = chunk * 16 + j < G;
+
+    WaveAttn<HDT, 1> w;
+    w.init(1);
+    const bf16* q_row[1] = {col_ok ? a.q + (size_t)t * a.ldq + (size_t)head_j * hd : nullptr};
+    w.load_q(q_row, 1, hd, lane);
+    const int pos[1] = {p}, los[1] = {lo};
+    const size_t k_stride = (size_t)4 * ((hd + 31) >> 5) * 64, v_stride = (size_t)hdt * 2 * 64;   // uint4 per (page, kv head)
+    for (int pi = page_lo; pi <= page_hi; ++pi) {
+        const long pg = page_of(a, b, pi);
+        if (pg < 0) continue;
+        w.page(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride, a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride, pi, 1,
+               hd, a.scale, pos, los, lane);
+    }
+    w.finish_sums(1);
+    // rows of the output tiles are heads 4g + e of the chunk; their sums live in the columns
+    float l4[4], m4[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        l4[e] = __shfl(w.l[0], 4 * g + e, 64);
+        m4[e] = __shfl(w.m[0], 4 * g + e, 64);
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int hq = chunk * 16 + 4 * g + e;
+        if (hq >= G) continue;
+        const int head = kvh * G + hq;
+        if (a.splits == 1) {
+            const float inv = l4[e] > 0.f ? 1.0f / l4[e] : 0.f;
+            bf16* dst = a.out + (size_t)t * a.ldo + (size_t)head * hd;
+#pragma unroll
+            for (int d = 0; d < HDT; ++d)
+                if (d < hdt) dst[16 * d + j] = f32_to_bf16(w.o[0][d][e] * inv);
+        } else {
+            const size_t slot = ((size_t)t * a.nh + head) * a.splits + split;
+            float* dst = a.part_o + slot * hd;
+#pragma unroll
+            for (int d = 0; d < HDT; ++d)
+                if (d < hdt) dst[16 * d + j] = w.o[0][d][e];
+            if (j == 0) {
+                a.part_ml[slot * 2 + 0] = m4[e];
+                a.part_ml[slot * 2 + 1] = l4[e];
+            }
+        }
+    }
+}
+
+// out[t][head] = sum_s O_s * exp(m_s - m) / sum_s l_s * exp(m_s - m)
+__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                    bf16* __restrict__ out, long ldo, int nh, int hd, int splits) {
+    const int t = blockIdx.x / nh, head = blockIdx.x % nh;
+    const size_t slot0 = ((size_t)t * nh + head) * splits;
+    float m = -INFINITY;
+    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
+    float l = 0.f;
+    for (int s = 0; s < splits; ++s) {
+        const float ms = part_ml[(slot0 + s) * 2];
+        if (ms != -INFINITY) l += part_ml[(slot0 + s) * 2 + 1] * __expf(ms - m);
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float acc = 0.f;
+        for (int s = 0; s < splits; ++s) {
+            const float ms = part_ml[(slot0 + s) * 2];
+            if (ms != -INFINITY) acc += part_o[(slot0 + s) * hd + d] * __expf(ms - m);
+        }
+        out[(size_t)t * ldo + (size_t)head * hd + d] = f32_to_bf16(acc * inv);
+    }
+}
+
+// ------------------------------------------------------------------ prefill: 16 positions x QT heads per wave
+// grid (position tile, kv head * head chunks, sequence); 4 waves per workgroup take 4
+// consecutive position tiles.  Slot j of tile t is position first + j of head chunk*QT + t.
+template <int HDT, int QT>
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int qt_heads) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
+    const int G = a.nh / a.nkv;
+    const int chunks = (G + qt_heads - 1) / qt_heads;
+    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int b = blockIdx.z;
+    const int t0 = a.cu[b], n_new = a.cu[b + 1] - t0;
+    const int tile0 = (blockIdx.x * 4 + wave) * 16;              // first step-token of this wave's tile
+    if (tile0 >= n_new) return;
+    const int qt = (G - chunk * qt_heads < qt_heads) ? G - chunk * qt_heads : qt_heads;
+    const int hd = a.hd, hdt = hd >> 4;
+    const bool col_ok = tile0 + j < n_new;
+    const int tok = t0 + (col_ok ? tile0 + j : n_new - 1);       // padding columns repeat the last token
+    const int p = a.tok_pos[tok];
+    const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
+
+    WaveAttn<HDT, QT> w;
+    w.init(qt);
+    const bf16* q_row[QT];
+    int pos[QT], los[QT];
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        const int head = kvh * G + chunk * qt_heads + t;
+        q_row[t] = (t < qt) ? a.q + (size_t)tok * a.ldq + (size_t)head * hd : nullptr;
+        pos[t] = p;
+        los[t] = lo;
+    }
+    w.load_q(q_row, qt, hd, lane);
+    // pages from the first column's lower bound to the last column's position
+    const int lo_min = __shfl(lo, 0, 64), p_max = __shfl(p, 15, 64);
+    const size_t k_stride = (size_t)4 * ((hd + 31) >> 5) * 64, v_stride = (size_t)hdt * 2 * 64;
+    for (int pi = lo_min / AGAVE_PAGE; pi <= p_max / AGAVE_PAGE; ++pi) {
+        const long pg = page_of(a, b, pi);
+        if (pg < 0) continue;
+        w.page(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride, a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride, pi, qt,
+               hd, a.scale, pos, los, lane);
+    }
+    w.finish_sums(qt);
+#pragma unroll
+    for (int t = 0; t < QT; ++t) {
+        if (t >= qt) continue;
+        const int head = kvh * G + chunk * qt_heads + t;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 4 * g + e;                            // slot (position) this lane's values belong to
+            const float lr = __shfl(w.l[t], row, 64);
+            if (tile0 + row >= n_new) continue;
+            const float inv = lr > 0.f ? 1.0f / lr : 0.f;
+            bf16* dst = a.out + (size_t)(t0 + tile0 + row) * a.ldo + (size_t)head * hd;
+#pragma unroll
+            for (int d = 0; d < HDT; ++d)
+                if (d < hdt) dst[16 * d + j] = f32_to_bf16(w.o[t][d][e] * inv);
+        }
+    }
+}
+
+// ------------------------------------------------------------------ host side
+static int check_common(const char* who, const AttnArgs& a, int N) {
+    AGAVE_CHECK(N >= 0 && a.nh > 0 && a.nkv > 0 && a.hd > 0, "%s: bad sizes N=%d nh=%d nkv=%d hd=%d", who, N, a.nh, a.nkv, a.hd);
+    AGAVE_CHECK(a.nh % a.nkv == 0, "%s: %d query heads are not a multiple of %d kv heads", who, a.nh, a.nkv);
+    AGAVE_CHECK(a.hd % 16 == 0 && a.hd <= 256, "%s: head_dim %d is not a multiple of 16 up to 256", who, a.hd);
+    AGAVE_CHECK(a.ldq >= (long)a.nh * a.hd && a.ldo >= (long)a.nh * a.hd, "%s: a row stride is below nh*hd", who);
+    AGAVE_CHECK(a.ldq % 8 == 0 && ((uintptr_t)a.q % 16) == 0, "%s: q must be 16-byte aligned with a row stride multiple of 8", who);
+    AGAVE_CHECK(a.q && a.out && a.k_pages && a.v_pages && a.table && a.base && a.tok_seq && a.tok_pos && a.width > 0 &&
+                    a.n_pages > 0, "%s: null buffer or empty table", who);
+    AGAVE_CHECK(a.window >= 0, "%s: negative window", who);
+    return 0;
+}
+
+extern "C" int agave_attn_decode_mfma(const void* q, long ldq, void* out, long ldo, float* part_o, float* part_ml,
+                                      const void* k_pages, const void* v_pages, const int* table, int width,
+                                      const int* base, int n_pages, const int* tok_seq, const int* tok_pos, int N,
+                                      int nh, int nkv, int hd, float scale, int window, int splits,
+                                      int pages_per_split, hipStream_t stream) {
+    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
+               table, width, base, n_pages, tok_seq, tok_pos, nullptr, 0, nh, nkv, hd, scale, window, splits,
+               pages_per_split};
+    if (check_common("attn_decode_mfma", a, N)) return -1;
+    AGAVE_CHECK(splits >= 1 && pages_per_split >= 1, "attn_decode_mfma: bad split plan %d x %d", splits, pages_per_split);
+    AGAVE_CHECK(splits == 1 || (part_o && part_ml), "attn_decode_mfma: splits need the partial buffers");
+    AGAVE_CHECK(N <= 65535, "attn_decode_mfma: %d tokens exceed the grid limit", N);
+    if (N == 0) return 0;
+    const int G = nh / nkv;
+    dim3 grid(splits, nkv * ((G + 15) / 16), N);
+    if (hd <= 64) attn_decode_mfma_kernel<4><<<grid, 64, 0, stream>>>(a);
+    else if (hd <= 128) attn_decode_mfma_kernel<8><<<grid, 64, 0, stream>>>(a);
+    else attn_decode_mfma_kernel<16><<<grid, 64, 0, stream>>>(a);
+    AGAVE_LAUNCH_CHECK("attn_decode_mfma");
+    if (splits > 1) {
+        attn_combine_kernel<<<N * nh, hd >= 128 ? 128 : 64, 0, stream>>>(part_o, part_ml, (bf16*)out, ldo, nh, hd, splits);
+        AGAVE_LAUNCH_CHECK("attn_combine");
+    }
+    return 0;
+}
+
+extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long ldo, const void* k_pages,
+                                       const void* v_pages, const int* table, int width, const int* base,
+                                       int n_pages, const int* tok_seq, const int* tok_pos, const int* cu, int n_seqs,
+                                       int max_new, int N, int nh, int nkv, int hd, float scale, int window,
+                                       hipStream_t stream) {
+    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, nullptr, nullptr, (const uint4*)k_pages, (const uint4*)v_pages,
+               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, 1, 0};
+    if (check_common("attn_prefill_mfma", a, N)) return -1;
+    AGAVE_CHECK(cu && n_seqs > 0 && max_new > 0, "attn_prefill_mfma: needs the sequences' token ranges");
+    AGAVE_CHECK(n_seqs <= 65535, "attn_prefill_mfma: %d sequences exceed the grid limit", n_seqs);
+    if (N == 0) return 0;
+    const int G = nh / nkv;
+    const int qt_cap = hd > 128 ? 1 : (hd > 64 ? 2 : QT_MAX);       // what fits the register file
+    const int qt_heads = G < qt_cap ? G : qt_cap;
+    const int chunks = (G + qt_heads - 1) / qt_heads;
+    AGAVE_CHECK(nkv * chunks <= 65535, "attn_prefill_mfma: too many head chunks");
+    dim3 grid((max_new + 63) / 64, nkv * chunks, n_seqs);
+    if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, 0, stream>>>(a, qt_heads);
+    else if (hd <= 128) attn_prefill_mfma_kernel<8, 2><<<grid, 256, 0, stream>>>(a, qt_heads);
+    else attn_prefill_mfma_kernel<16, 1><<<grid, 256, 0, stream>>>(a, qt_heads);
+    AGAVE_LAUNCH_CHECK("attn_prefill_mfma");
+    return 0;
+}

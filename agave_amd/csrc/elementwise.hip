@@ -119,7 +119,8 @@ __global__ void qk_norm_rope_kv_kernel(const T* q, long ldq, const T* __restrict
                                        int rot_half, float pos_scale, const int* __restrict__ tok_seq,
                                        const int* __restrict__ tok_pos, T* __restrict__ k_pages,
                                        T* __restrict__ v_pages, const int* __restrict__ table, int width,
-                                       const int* __restrict__ base, int n_pages, int N, int nh, int nkv, int hd) {
+                                       const int* __restrict__ base, int n_pages, int N, int nh, int nkv, int hd,
+                                       int packed) {
     __shared__ float buf[4][QK_HD_MAX];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int heads = nh + nkv;
@@ -147,35 +148,52 @@ __global__ void qk_norm_rope_kv_kernel(const T* q, long ldq, const T* __restrict
         for (int d = lane; d < hd; d += 64) y[d] = y[d] * inv * gain[d];
     }
     __syncthreads();
-    if (!active) return;
 
-    const int p = tok_pos[t];
-    T* dst;
-    long pg = -1;
-    int row = 0;
-    if (is_q) {
-        dst = q_out + (size_t)t * ldqo + (size_t)head * hd;
-    } else {
-        const int b = tok_seq[t];
-        const int col = p / AGAVE_PAGE - base[b];
-        row = p % AGAVE_PAGE;
-        if (col >= 0 && col < width) pg = table[(size_t)b * width + col];
-        if (pg < 0 || pg >= n_pages) return;   // a table the host built wrongly: write nothing
-        dst = k_pages + (((size_t)pg * nkv + head) * AGAVE_PAGE + row) * hd;
-    }
+    const int p = active ? tok_pos[t] : 0;
     const float pf = (float)p * pos_scale;
-    for (int i = lane; i < rot_half; i += 64) {
+    // rotation, in place in LDS: y[i], y[i + rot_half] <- rotated pair
+    for (int i = lane; active && i < rot_half; i += 64) {
         const float a = y[i], b2 = y[i + rot_half];
         float s, c;
         sincosf(pf * inv_freq[i], &s, &c);
-        st(dst + i, a * c - b2 * s);
-        st(dst + i + rot_half, a * s + b2 * c);
+        y[i] = a * c - b2 * s;
+        y[i + rot_half] = a * s + b2 * c;
     }
-    for (int d = 2 * rot_half + lane; d < hd; d += 64) st(dst + d, y[d]);
-    if (!is_q) {
-        const T* sv = v + (size_t)t * ldv + (size_t)head * hd;
+    __syncthreads();
+    if (!active) return;
+    if (is_q) {
+        T* dst = q_out + (size_t)t * ldqo + (size_t)head * hd;
+        for (int d = lane; d < hd; d += 64) st(dst + d, y[d]);
+        return;
+    }
+    const int b = tok_seq[t];
+    const int col = p / AGAVE_PAGE - base[b];
+    const int row = p % AGAVE_PAGE;
+    long pg = -1;
+    if (col >= 0 && col < width) pg = table[(size_t)b * width + col];
+    if (pg < 0 || pg >= n_pages) return;   // a table the host built wrongly: write nothing
+    const T* sv = v + (size_t)t * ldv + (size_t)head * hd;
+    if (!packed) {
+        T* dk = k_pages + (((size_t)pg * nkv + head) * AGAVE_PAGE + row) * hd;
         T* dv = v_pages + ((size_t)pg * nkv + head) * hd * AGAVE_PAGE + row;
-        for (int d = lane; d < hd; d += 64) dv[(size_t)d * AGAVE_PAGE] = sv[d];
+        for (int d = lane; d < hd; d += 64) {
+            st(dk + d, y[d]);
+            dv[(size_t)d * AGAVE_PAGE] = sv[d];
+        }
+    } else {
+        // matrix-core tile order (see attention_mfma.hip)
+        const int ks_n = (hd + 31) >> 5;
+        T* dk = k_pages + ((size_t)pg * nkv + head) * (size_t)(AGAVE_PAGE * ks_n * 32);
+        T* dv = v_pages + ((size_t)pg * nkv + head) * (size_t)hd * AGAVE_PAGE;
+        const int kt = row >> 4, ki = row & 15;
+        const int s2 = row >> 5, r32 = row & 31;
+        const int vg = (r32 & 15) >> 2, ve = (r32 & 3) + ((r32 >> 4) << 2);
+        for (int d = lane; d < hd; d += 64) {
+            const int ks = d >> 5, g = (d & 31) >> 3, e = d & 7;
+            st(dk + ((size_t)(kt * ks_n + ks) * 64 + ki + 16 * g) * 8 + e, y[d]);
+            const int dt = d >> 4, j = d & 15;
+            dv[((size_t)(dt * 2 + s2) * 64 + j + 16 * vg) * 8 + ve] = sv[d];
+        }
     }
 }
 
@@ -184,7 +202,7 @@ extern "C" int agave_qk_norm_rope_kv(int dtype, const void* q, long ldq, const v
                                      float eps_q, float eps_k, const float* inv_freq, int rot_half, float pos_scale,
                                      const int* tok_seq, const int* tok_pos, void* k_pages, void* v_pages,
                                      const int* table, int width, const int* base, int n_pages, int N, int nh,
-                                     int nkv, int hd, hipStream_t stream) {
+                                     int nkv, int hd, int packed, hipStream_t stream) {
     AGAVE_CHECK(N >= 0 && nh >= 0 && nkv >= 0 && hd > 0, "qk_norm_rope_kv: bad sizes N=%d nh=%d nkv=%d hd=%d", N, nh, nkv, hd);
     AGAVE_CHECK(hd <= QK_HD_MAX, "qk_norm_rope_kv: head_dim %d exceeds the supported maximum %d", hd, QK_HD_MAX);
     AGAVE_CHECK(rot_half >= 0 && 2 * rot_half <= hd, "qk_norm_rope_kv: rotary_dim %d exceeds head_dim %d", 2 * rot_half, hd);
@@ -194,6 +212,7 @@ extern "C" int agave_qk_norm_rope_kv(int dtype, const void* q, long ldq, const v
                              ldk >= (long)nkv * hd && ldv >= (long)nkv * hd),
                 "qk_norm_rope_kv: bad k/v buffers or cache table");
     AGAVE_CHECK(tok_pos != nullptr, "qk_norm_rope_kv: positions are null");
+    AGAVE_CHECK(!packed || (dtype == AGAVE_BF16 && hd % 16 == 0), "qk_norm_rope_kv: packed pages need bfloat16 and head_dim %% 16 == 0");
     const long units = (long)N * (nh + nkv);
     if (units == 0) return 0;
     const int blocks = (int)((units + 3) / 4);
@@ -201,12 +220,12 @@ extern "C" int agave_qk_norm_rope_kv(int dtype, const void* q, long ldq, const v
         qk_norm_rope_kv_kernel<float><<<blocks, 256, 0, stream>>>(
             (const float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv, (float*)q_out, ldqo, q_gain, k_gain,
             eps_q, eps_k, inv_freq, rot_half, pos_scale, tok_seq, tok_pos, (float*)k_pages, (float*)v_pages, table,
-            width, base, n_pages, N, nh, nkv, hd);
+            width, base, n_pages, N, nh, nkv, hd, packed);
     else if (dtype == AGAVE_BF16)
         qk_norm_rope_kv_kernel<bf16><<<blocks, 256, 0, stream>>>(
             (const bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv, (bf16*)q_out, ldqo, q_gain, k_gain, eps_q,
             eps_k, inv_freq, rot_half, pos_scale, tok_seq, tok_pos, (bf16*)k_pages, (bf16*)v_pages, table, width,
-            base, n_pages, N, nh, nkv, hd);
+            base, n_pages, N, nh, nkv, hd, packed);
     else
         AGAVE_CHECK(false, "qk_norm_rope_kv: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("qk_norm_rope_kv");

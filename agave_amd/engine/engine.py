@@ -73,7 +73,7 @@ class Engine:
         pages: Dict[GroupKey, int] = {key: n_pages for key in set(kv_needs.values())}
         self.cache = KVCache(kv_needs, self.model.state_needs(), max_slots, pages, self.dtype, self.device,
                              self.max_context)
-        self.planner = StepPlanner(self.cache, spec.vocab_size, self.device)
+        self.planner = StepPlanner(self.cache, spec.vocab_size, self.device, self.workspace)
         self.prefill_chunk = 0          # > 0: prompts enter in pieces of at most this many tokens
 
     # ------------------------------------------------------------------ construction

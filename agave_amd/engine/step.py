@@ -51,6 +51,22 @@ class Step:
     want_rows: torch.Tensor         # int32 [n_want]: rows of the step whose logits are wanted
     tables: List[Tuple[torch.Tensor, torch.Tensor]]   # per cache group: (pages [B, width], base [B])
     cache: KVCache
+    workspace: object = None
+    fixed_span: Optional[int] = None    # a captured decode graph plans its splits for this many pages
+
+    def page_span(self, window: Optional[int]) -> int:
+        """Most pages any sequence's last token of this step reaches back over."""
+        if self.fixed_span is not None:
+            span = self.fixed_span
+            if window is not None:
+                span = min(span, (window + 62) // 64 + 1)
+            return max(1, span)
+        span = 1
+        for p0, n in zip(self.pos0, self.n_new):
+            p = p0 + n - 1
+            lo = max(0, p - window + 1) if window is not None else 0
+            span = max(span, p // 64 - lo // 64 + 1)
+        return span
 
     @property
     def is_decode(self) -> bool:
@@ -82,8 +98,9 @@ class StepPlanner:
     """Turns (slots, tokens, want) into a :class:`Step`: checks the request, takes cache
     pages, and uploads the step's description in one copy."""
 
-    def __init__(self, cache: KVCache, vocab_size: int, device: torch.device):
+    def __init__(self, cache: KVCache, vocab_size: int, device: torch.device, workspace=None):
         self.cache = cache
+        self.workspace = workspace
         self.vocab_size = vocab_size
         self.device = device
         self._host: Optional[torch.Tensor] = None
@@ -167,7 +184,8 @@ class StepPlanner:
             max_new=max(n_new), max_len=max(p + k for p, k in zip(pos0, n_new)),
             tokens=view(s_tok), tok_seq=view(s_seq), tok_pos=view(s_pos), slots_dev=view(s_slots),
             pos0_dev=view(s_pos0), cu_dev=view(s_cu), want_rows=view(s_want),
-            tables=[(view(t).view(b, w), view(sb)) for t, sb, w in s_tables], cache=self.cache)
+            tables=[(view(t).view(b, w), view(sb)) for t, sb, w in s_tables], cache=self.cache,
+            workspace=self.workspace)
 
     def commit(self, step: Step) -> None:
         self.cache.commit_step(step.slots, step.n_new)

@@ -10,13 +10,13 @@ from . import kernels
 
 def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
               table: torch.Tensor, base: torch.Tensor, step, n_heads: int, n_kv: int, head_dim: int,
-              scale: float, window: Optional[int]) -> None:
+              scale: float, window: Optional[int], packed: bool = False) -> None:
     """Attention of the step's tokens over their sequences' cache pages (which already hold the
-    step's own keys and values)."""
-    if q.dtype == torch.bfloat16:
+    step's own keys and values).  Pages in the matrix cores' tile order go to the MFMA kernels,
+    pages stored row by row to the plain kernel."""
+    if packed:
         from . import attention_mfma
-        if attention_mfma.try_attention(q, out, k_pages, v_pages, table, base, step, n_heads, n_kv,
-                                        head_dim, scale, window):
-            return
+        attention_mfma.attention(q, out, k_pages, v_pages, table, base, step, n_heads, n_kv, head_dim, scale, window)
+        return
     kernels.attn_plain(q, out, k_pages, v_pages, table, base, step.tok_seq, step.tok_pos,
                        n_heads, n_kv, head_dim, scale, window)

@@ -1,6 +1,58 @@
-"""Matrix-core (MFMA) attention for bfloat16.  Filled in after the plain path."""
+"""Matrix-core (MFMA) attention over cache pages in tile order (bfloat16)."""
 from __future__ import annotations
 
+from typing import Optional
 
-def try_attention(q, out, k_pages, v_pages, table, base, step, n_heads, n_kv, head_dim, scale, window) -> bool:
-    return False
+import torch
+
+from . import kernels, library
+from .kernels import _F, _I, _L, _P
+
+kernels.register_signatures("attention_mfma", {
+    "agave_attn_decode_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "agave_attn_prefill_mfma": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+})
+
+TARGET_WAVES = 2048          # workgroups a decode launch aims for (8 per compute unit)
+
+
+def split_plan(page_span: int, units: int):
+    """(splits, pages per split) for sequences spanning at most ``page_span`` pages when the launch
+    has ``units`` (token, kv head) pairs."""
+    want = max(1, min(page_span, -(-TARGET_WAVES // max(units, 1))))
+    per = -(-page_span // want)
+    return -(-page_span // per), per
+
+
+def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, table: torch.Tensor,
+              base: torch.Tensor, step, n_heads: int, n_kv: int, head_dim: int, scale: float,
+              window: Optional[int]) -> None:
+    if not (q.is_cuda and out.is_cuda and k_pages.is_cuda):
+        raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
+    n = step.n_tokens
+    if q.dtype != torch.bfloat16 or q.shape != (n, n_heads * head_dim) or out.shape != q.shape or out.dtype != q.dtype:
+        raise ValueError(f"attention: q and out must be bfloat16 [{n}, {n_heads * head_dim}]")
+    if q.stride(1) != 1 or out.stride(1) != 1:
+        raise ValueError("attention: q and out need contiguous rows")
+    n_pages = kernels._check_pages(k_pages, v_pages, n_kv, head_dim, q.dtype, packed=True)
+    width = kernels._check_table(table, base, step.tok_seq)
+    lib = kernels.lib("attention_mfma")
+    w = int(window or 0)
+    if step.is_decode:
+        span = step.page_span(window)
+        chunks = -(-(n_heads // n_kv) // 16)
+        splits, per = split_plan(span, n * n_kv * chunks)
+        part_o = part_ml = None
+        if splits > 1:
+            ws = step.workspace
+            part_o = ws.get("attn_part_o", n * n_heads * splits, head_dim, torch.float32)
+            part_ml = ws.get("attn_part_ml", n * n_heads * splits, 2, torch.float32)
+        library.call(lib, "agave_attn_decode_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+                     kernels.ptr(part_o), kernels.ptr(part_ml), k_pages.data_ptr(), v_pages.data_ptr(),
+                     table.data_ptr(), width, base.data_ptr(), n_pages, step.tok_seq.data_ptr(),
+                     step.tok_pos.data_ptr(), n, n_heads, n_kv, head_dim, scale, w, splits, per, kernels.stream())
+    else:
+        library.call(lib, "agave_attn_prefill_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+                     k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width, base.data_ptr(), n_pages,
+                     step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), step.cu_dev.data_ptr(), step.n_seqs,
+                     step.max_new, n, n_heads, n_kv, head_dim, scale, w, kernels.stream())

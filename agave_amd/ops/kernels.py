@@ -23,7 +23,7 @@ _SIGNATURES = {
         "agave_embed_scale": [_I, _P, _P, _F, _P, _I, _I, _I, _P],
         "agave_residual_norm": [_I, _P, _P, _L, _P, _F, _P, _L, _P, _F, _P, _I, _I, _P],
         "agave_qk_norm_rope_kv": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F,
-                                  _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+                                  _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
         "agave_cast": [_I, _P, _I, _P, _L, _P],
     },
@@ -153,9 +153,10 @@ def qk_norm_rope_kv(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Opt
                     eps_q: float, eps_k: float, inv_freq: Optional[torch.Tensor], pos_scale: float,
                     tok_seq: torch.Tensor, tok_pos: torch.Tensor, k_pages: Optional[torch.Tensor],
                     v_pages: Optional[torch.Tensor], table: Optional[torch.Tensor], base: Optional[torch.Tensor],
-                    n_heads: int, n_kv: int, head_dim: int) -> None:
+                    n_heads: int, n_kv: int, head_dim: int, packed: bool = False) -> None:
     """Per-head RMSNorm of q and k, rotation, q to ``q_out`` and k, v into their cache pages.
-    ``k`` None: only q is processed (a layer that reads another layer's cache)."""
+    ``k`` None: only q is processed (a layer that reads another layer's cache).  ``packed``:
+    the pages are in the matrix cores' tile order."""
     _dev(q, k, v, q_out, q_gain, k_gain, inv_freq, tok_seq, tok_pos, k_pages, v_pages, table, base)
     n = tok_pos.numel()
     _i32(tok_pos, "tok_pos")
@@ -177,7 +178,7 @@ def qk_norm_rope_kv(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Opt
         if k.shape != (n, nkv * head_dim) or v.shape != (n, nkv * head_dim) or k.dtype != ref.dtype or v.dtype != ref.dtype:
             raise ValueError(f"k and v must be [{n}, {nkv * head_dim}] of the activations' dtype")
         _f32vec(k_gain, "k_gain", head_dim)
-        n_pages = _check_pages(k_pages, v_pages, nkv, head_dim, ref.dtype)
+        n_pages = _check_pages(k_pages, v_pages, nkv, head_dim, ref.dtype, packed)
         width = _check_table(table, base, tok_seq)
     rot_half = 0
     if inv_freq is not None:
@@ -186,12 +187,16 @@ def qk_norm_rope_kv(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Opt
     library.call(lib("elementwise"), "agave_qk_norm_rope_kv", d, ptr(q), ldq, ptr(k), ldk, ptr(v), ldv, ptr(q_out),
                  ldqo, ptr(q_gain), ptr(k_gain), eps_q, eps_k, ptr(inv_freq), rot_half, pos_scale, ptr(tok_seq),
                  ptr(tok_pos), ptr(k_pages), ptr(v_pages), ptr(table), width, ptr(base), n_pages, n, nh, nkv,
-                 head_dim, stream())
+                 head_dim, 1 if (packed and k is not None) else 0, stream())
 
 
-def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, nkv: int, hd: int, dtype: torch.dtype) -> int:
-    if k_pages.dim() != 4 or tuple(k_pages.shape[1:]) != (nkv, 64, hd) or not k_pages.is_contiguous():
-        raise ValueError(f"K pages must be contiguous [pages, {nkv}, 64, {hd}], got {tuple(k_pages.shape)}")
+def _check_pages(k_pages: torch.Tensor, v_pages: torch.Tensor, nkv: int, hd: int, dtype: torch.dtype,
+                 packed: bool = False) -> int:
+    hd_k = (hd + 31) // 32 * 32 if packed else hd       # packed K rows are padded to whole tiles
+    if packed and (dtype != torch.bfloat16 or hd % 16):
+        raise ValueError("packed cache pages need bfloat16 and a head size that is a multiple of 16")
+    if k_pages.dim() != 4 or tuple(k_pages.shape[1:]) != (nkv, 64, hd_k) or not k_pages.is_contiguous():
+        raise ValueError(f"K pages must be contiguous [pages, {nkv}, 64, {hd_k}], got {tuple(k_pages.shape)}")
     if v_pages.dim() != 4 or tuple(v_pages.shape[1:]) != (nkv, hd, 64) or not v_pages.is_contiguous():
         raise ValueError(f"V pages must be contiguous [pages, {nkv}, {hd}, 64], got {tuple(v_pages.shape)}")
     if k_pages.shape[0] != v_pages.shape[0] or k_pages.dtype != dtype or v_pages.dtype != dtype:

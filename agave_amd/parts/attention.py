@@ -57,7 +57,7 @@ class Attention:
     def forward(self, x: torch.Tensor, step, memory: int, writes: bool = True) -> torch.Tensor:
         s, ws = self.spec, self.env.workspace
         n = x.shape[0]
-        k_pages, v_pages = step.cache.pages_of(memory)
+        k_pages, v_pages, packed = step.cache.pages_of(memory)
         table, base = step.tables[step.cache.group_of_memory[memory]]
         inv_freq, pos_scale = (None, 1.0)
         fused = getattr(self.position, "fused_rotation", None)
@@ -78,10 +78,10 @@ class Attention:
             self.q_norm.gain if self.q_norm else None, self.k_norm.gain if self.k_norm else None,
             self.q_norm.eps if self.q_norm else 0.0, self.k_norm.eps if self.k_norm else 0.0,
             inv_freq, pos_scale, step.tok_seq, step.tok_pos, k_pages, v_pages, table, base,
-            s.n_heads, s.n_kv_heads, s.head_dim)
+            s.n_heads, s.n_kv_heads, s.head_dim, packed)
         ctx_out = ws.get("attn_ctx", n, self.qd, x.dtype)
         attn_ops.attention(q_out, ctx_out, k_pages, v_pages, table, base, step, s.n_heads, s.n_kv_heads,
-                           s.head_dim, s.scale, s.window)
+                           s.head_dim, s.scale, s.window, packed)
         return self.o.forward(ctx_out, tag="attn_o")
 
 

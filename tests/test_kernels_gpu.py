@@ -379,3 +379,105 @@ def test_gemm_skinny_refuses_what_it_cannot_do(G):
         G.skinny(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w, out, 32)
     with pytest.raises(ValueError):
         G.skinny(torch.zeros(4, 60, dtype=torch.bfloat16, device=DEV), w, out[:4], 32)   # K no multiple of 8
+
+
+# ---------------------------------------------------------------- matrix-core attention over packed pages
+class _FakeStep:
+    """What the attention op reads of a step."""
+
+    def __init__(self, lens, queries_from, window):
+        from agave_amd.parts import Workspace
+        self.pos0 = [queries_from(L) for L in lens]
+        self.n_new = [L - p for L, p in zip(lens, self.pos0)]
+        self.n_seqs = len(lens)
+        self.n_tokens = sum(self.n_new)
+        self.max_new = max(self.n_new)
+        cu = [0]
+        for n in self.n_new:
+            cu.append(cu[-1] + n)
+        self.cu_dev = _i32(cu)
+        self.tok_seq = _i32([b for b, n in enumerate(self.n_new) for _ in range(n)])
+        self.tok_pos = _i32([p + i for p, n in zip(self.pos0, self.n_new) for i in range(n)])
+        self.workspace = Workspace(torch.device(DEV))
+        self.fixed_span = None
+
+    @property
+    def is_decode(self):
+        return self.max_new == 1
+
+    def page_span(self, window):
+        span = 1
+        for p0, n in zip(self.pos0, self.n_new):
+            p = p0 + n - 1
+            lo = max(0, p - window + 1) if window is not None else 0
+            span = max(span, p // 64 - lo // 64 + 1)
+        return span
+
+
+def _mfma_attn_case(K, nh, nkv, hd, lens, window, scale, decode, seed=0, boost=None):
+    """Keys and values go into packed pages through the q/k kernel (no norm, no rotation); then
+    either every position is a query (prefill) or only each sequence's last one (decode)."""
+    from agave_amd.ops import attention_mfma
+    g = torch.Generator().manual_seed(seed)
+    hd_k = (hd + 31) // 32 * 32
+    n_pages = sum((L + 63) // 64 for L in lens) + 2
+    kp = torch.zeros(n_pages, nkv, 64, hd_k, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros(n_pages, nkv, hd, 64, dtype=torch.bfloat16, device=DEV)
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    width = max((L + 63) // 64 for L in lens)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    ks, vs, qs = [], [], []
+    for b, L in enumerate(lens):
+        k = torch.randn(L, nkv, hd, generator=g).bfloat16()
+        v = torch.randn(L, nkv, hd, generator=g).bfloat16()
+        q = torch.randn(L, nh, hd, generator=g).bfloat16()
+        if boost is not None:
+            k = (k.float() - k.float().mean(dim=-1, keepdim=True)).bfloat16()
+            k[boost] = 1.0
+            q[L - 1] = 20.0 / (hd * scale)
+        for i in range((L + 63) // 64):
+            table[b, i] = perm.pop()
+        ks.append(k); vs.append(v); qs.append(q)
+    table, base = table.to(DEV), _i32([0] * len(lens))
+    seq_all = _i32([b for b, L in enumerate(lens) for _ in range(L)])
+    pos_all = _i32([i for L in lens for i in range(L)])
+    k_all = torch.cat(ks).reshape(-1, nkv * hd).to(DEV)
+    v_all = torch.cat(vs).reshape(-1, nkv * hd).to(DEV)
+    K.qk_norm_rope_kv(None, k_all, v_all, None, None, None, 0.0, 0.0, None, 1.0, seq_all, pos_all, kp, vp, table, base,
+                      0, nkv, hd, packed=True)
+    step = _FakeStep(lens, (lambda L: L - 1) if decode else (lambda L: 0), window)
+    q_sel = torch.cat([q[p0:] for q, p0 in zip(qs, step.pos0)]).reshape(-1, nh * hd).to(DEV)
+    out = torch.full_like(q_sel, float("nan"))
+    attention_mfma.attention(q_sel, out, kp, vp, table, base, step, nh, nkv, hd, scale, window)
+    refs = [P.attention_core(q.double(), k.double(), v.double(), scale, window)[p0:]
+            for q, k, v, p0 in zip(qs, ks, vs, step.pos0)]
+    return out.cpu().double().view(-1, nh, hd), torch.cat(refs), vs
+
+
+@pytest.mark.parametrize("decode", [True, False])
+@pytest.mark.parametrize("nh,nkv,hd,window", [(4, 2, 64, None), (6, 1, 16, 70), (3, 3, 48, 300), (8, 4, 256, 64),
+                                              (2, 1, 128, None), (20, 1, 32, 129), (8, 2, 96, 1)])
+def test_attn_mfma(K, decode, nh, nkv, hd, window):
+    got, ref, _ = _mfma_attn_case(K, nh, nkv, hd, [1, 77, 300, 64, 65], window, 0.21 * (16 / hd) ** 0.5, decode)
+    assert torch.isfinite(got).all()
+    assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("decode", [True, False])
+def test_attn_mfma_long_sequences_split_over_workgroups(K, decode):
+    from agave_amd.ops import attention_mfma
+    assert attention_mfma.split_plan(40, 4)[0] > 1          # the decode launch below is split
+    got, ref, _ = _mfma_attn_case(K, 4, 2, 128, [2500, 1031], None, 0.05, decode, seed=3)
+    assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
+    got, ref, _ = _mfma_attn_case(K, 4, 2, 128, [2500, 1031], 1024, 0.05, decode, seed=4)
+    assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("decode", [True, False])
+def test_attn_mfma_far_key_and_window_edge(K, decode):
+    got, ref, vs = _mfma_attn_case(K, 2, 1, 32, [700], None, 0.5, decode, seed=1, boost=3)
+    assert torch.allclose(got[-1, 0], vs[0][3, 0].double(), atol=2e-2)
+    got_w, _, _ = _mfma_attn_case(K, 2, 1, 32, [700], 696, 0.5, decode, seed=1, boost=3)      # key 3 just outside
+    assert not torch.allclose(got_w[-1, 0], vs[0][3, 0].double(), atol=1e-1)
+    got_e, _, _ = _mfma_attn_case(K, 2, 1, 32, [700], 697, 0.5, decode, seed=1, boost=3)      # just inside
+    assert torch.allclose(got_e[-1, 0], vs[0][3, 0].double(), atol=2e-2)
