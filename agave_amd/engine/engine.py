@@ -14,6 +14,8 @@ from __future__ import annotations
 
 from typing import Dict, List, Optional, Sequence
 
+import os
+
 import torch
 
 from ..cache import PAGE, GroupKey, KVCache
@@ -21,6 +23,7 @@ from ..config import find_architecture, read_config_json
 from ..config.spec import ModelSpec
 from ..parts import BuildEnv, Workspace
 from ..weights import Checkpoint, DictWeightSource, RandomWeightSource, WeightSource
+from .graphs import DecodeGraphs, span_bucket
 from .model import Model, tensor_needs
 from .step import Step, StepPlanner, Want
 
@@ -75,6 +78,9 @@ class Engine:
                              self.max_context)
         self.planner = StepPlanner(self.cache, spec.vocab_size, self.device, self.workspace)
         self.prefill_chunk = 0          # > 0: prompts enter in pieces of at most this many tokens
+        self.use_graphs = os.environ.get("AGAVE_AMD_NO_GRAPHS", "") not in ("1", "true", "yes")
+        self.graphs = DecodeGraphs(self)
+        self._decode_widths = [g.table_width(self.max_context, 1) for g in self.cache.groups]
 
     # ------------------------------------------------------------------ construction
     @classmethod
@@ -132,8 +138,12 @@ class Engine:
         """Run ``tokens[i]`` as the next tokens of the sequence in ``slots[i]``.  Returns the
         float32 logits [wanted, vocab] on the GPU in the order of the sequences and of their
         wanted places (valid until the next step), or None if nothing is wanted."""
-        step = self.planner.plan(slots, tokens, want)
-        logits = self.model.forward(step)
+        step = self.planner.plan(slots, tokens, want, decode_widths=self._decode_widths if self.use_graphs else None)
+        if self.use_graphs and step.is_decode and step.n_want == step.n_tokens:
+            step.fixed_span = span_bucket(step.page_span(None))
+            logits = self.graphs.run(step)
+        else:
+            logits = self.model.forward(step)
         self.planner.commit(step)
         return logits
 

@@ -107,6 +107,7 @@ class StepPlanner:
         self._dev: Optional[torch.Tensor] = None
         self._copied = None          # event: the last upload has left the host buffer
         self.fixed_width: Optional[List[int]] = None   # table widths pinned for graph capture
+        self.buffer_generation = 0   # changes when the device buffer of the step's description moves
 
     def _buffers(self, n: int) -> None:
         if self._host is None or self._host.numel() < n:
@@ -115,8 +116,12 @@ class StepPlanner:
                 self._copied.synchronize()
             self._host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
             self._dev = torch.empty(cap, dtype=torch.int32, device=self.device)
+            self.buffer_generation += 1
 
-    def plan(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want = "last") -> Step:
+    def plan(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want = "last",
+             decode_widths: Optional[List[int]] = None) -> Step:
+        """``decode_widths``: table widths to use if this turns out to be a decode step (one token per
+        sequence), so that all decode steps of a batch size have the same layout on the device."""
         if len(slots) != len(tokens) or len(slots) == 0:
             raise StepError("a step needs as many token lists as slots, and at least one")
         n_new = [len(t) for t in tokens]
@@ -135,12 +140,11 @@ class StepPlanner:
             cu.append(cu[-1] + x)
         want_rows = [cu[i] + x for i, w in enumerate(wanted) for x in w]
         widths = []
+        fixed = decode_widths if (decode_widths is not None and max(n_new) == 1) else self.fixed_width
         for gi, p in enumerate(plans):
             w = max(len(r) for r in p.rows)
-            if self.fixed_width is not None:
-                if w > self.fixed_width[gi]:
-                    raise StepError(f"step needs {w} table columns, the captured width is {self.fixed_width[gi]}")
-                w = self.fixed_width[gi]
+            if fixed is not None and w <= fixed[gi]:
+                w = fixed[gi]
             widths.append(w)
         total = 3 * n + 3 * b + 1 + len(want_rows) + sum(b + b * w for w in widths)
         self._buffers(total)

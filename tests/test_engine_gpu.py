@@ -104,3 +104,31 @@ def test_cutting_gives_the_same_numbers(engine_of):
     scale = float(whole.abs().max())
     assert float((whole - tail).abs().max()) <= tol * scale
     assert float((whole - batched).abs().max()) <= tol * scale
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replays_equal_eager_steps(tiny, dtype):
+    """Decode steps are recorded into a HIP graph on their second occurrence.  Every replay, with
+    eager steps of other batches and synchronisations in between, must give what an engine
+    without graphs gives."""
+    from agave_amd.engine import Engine
+    which, cfg, weights, folder = tiny
+    a = Engine.from_folder(folder, dtype=dtype, max_slots=4, max_context=256)
+    b = Engine.from_folder(folder, dtype=dtype, max_slots=4, max_context=256)
+    b.use_graphs = False
+    v = cfg["vocab_size"]
+    prompts = [U.random_tokens(n, v, 200 + i) for i, n in enumerate((70, 3, 129))]
+    sa = [a.alloc_slot() for _ in prompts]
+    sb = [b.alloc_slot() for _ in prompts]
+    a.step(sa, prompts, "last")
+    b.step(sb, prompts, "last")
+    other = a.alloc_slot()
+    for i in range(70):                       # crosses page boundaries and, for window 70, its edge
+        toks = [[(7 * i + 3 * j) % v] for j in range(3)]
+        la = a.step(sa, toks, "last").clone()
+        lb = b.step(sb, toks, "last").clone()
+        assert torch.equal(la, lb), f"step {i}"
+        if i % 9 == 0:                        # eager work of another sequence between replays
+            a.step([other], [U.random_tokens(5, v, i)], "last")
+            torch.cuda.synchronize()
+    assert len(a.graphs._graphs) >= 1
