@@ -1,6 +1,6 @@
 // bfloat16 attention over the paged cache on the matrix cores of gfx950 (head sizes in steps
 // of 16 up to 256): a decode kernel that splits a sequence's keys over workgroups
-// (flash-decoding) with a combine pass, and a prefill kernel for steps that bring many tokens.
+// (flash-decoding) whose last workgroup adds the splits up, and a prefill kernel for steps that bring many tokens.
 // Scores, the running maximum and sum, and the output accumulate in 32-bit; probabilities
 // are rounded to bfloat16 only as the operand of the P*V product.
 //
@@ -45,6 +45,8 @@ struct AttnArgs {
     float scale;
     int window;
     int splits, pages_per_split;
+    int* counters;       // decode with splits: one zeroed counter per (token, kv head chunk); left zeroed
+    int seq_is_token;    // decode: sequence index == token index
 };
 
 // One wave: QT tiles of 16 query slots against the pages [page_lo, page_hi] of one sequence
@@ -195,7 +197,7 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(AttnArgs a) {
     const int chunks = (G + 15) / 16;
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
     const int t = blockIdx.z, split = blockIdx.x;
-    const int b = a.tok_seq[t], p = a.tok_pos[t];
+    const int b = a.seq_is_token ? t : a.tok_seq[t], p = a.tok_pos[t];
     const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
     const int first = lo / AGAVE_PAGE, last = p / AGAVE_PAGE;
     const int page_lo = first + split * a.pages_per_split;
@@ -248,29 +250,37 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(AttnArgs a) {
             }
         }
     }
-}
-
-// out[t][head] = sum_s O_s * exp(m_s - m) / sum_s l_s * exp(m_s - m)
-__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                    bf16* __restrict__ out, long ldo, int nh, int hd, int splits) {
-    const int t = blockIdx.x / nh, head = blockIdx.x % nh;
-    const size_t slot0 = ((size_t)t * nh + head) * splits;
-    float m = -INFINITY;
-    for (int s = 0; s < splits; ++s) m = fmaxf(m, part_ml[(slot0 + s) * 2]);
-    float l = 0.f;
-    for (int s = 0; s < splits; ++s) {
-        const float ms = part_ml[(slot0 + s) * 2];
-        if (ms != -INFINITY) l += part_ml[(slot0 + s) * 2 + 1] * __expf(ms - m);
-    }
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-        float acc = 0.f;
-        for (int s = 0; s < splits; ++s) {
-            const float ms = part_ml[(slot0 + s) * 2];
-            if (ms != -INFINITY) acc += part_o[(slot0 + s) * hd + d] * __expf(ms - m);
+    if (a.splits == 1) return;
+    // The workgroup that finishes last for this (token, kv head chunk) adds the splits up, in
+    // the order of the splits:  out = sum_s O_s e^(m_s - m) / sum_s l_s e^(m_s - m).
+    __threadfence();
+    const int unit = t * gridDim.y + blockIdx.y;
+    int done = 0;
+    if (lane == 0) done = atomicAdd(a.counters + unit, 1);
+    done = __shfl(done, 0, 64);
+    if (done != a.splits - 1) return;
+    __threadfence();
+    for (int hq = 0; hq < 16 && chunk * 16 + hq < G; ++hq) {
+        const int head = kvh * G + chunk * 16 + hq;
+        const size_t slot0 = ((size_t)t * a.nh + head) * a.splits;
+        float mm = -INFINITY;
+        for (int s = 0; s < a.splits; ++s) mm = fmaxf(mm, a.part_ml[(slot0 + s) * 2]);
+        float ll = 0.f;
+        for (int s = 0; s < a.splits; ++s) {
+            const float ms = a.part_ml[(slot0 + s) * 2];
+            if (ms != -INFINITY) ll += a.part_ml[(slot0 + s) * 2 + 1] * __expf(ms - mm);
         }
-        out[(size_t)t * ldo + (size_t)head * hd + d] = f32_to_bf16(acc * inv);
+        const float inv = ll > 0.f ? 1.0f / ll : 0.f;
+        for (int d = lane; d < hd; d += 64) {
+            float acc = 0.f;
+            for (int s = 0; s < a.splits; ++s) {
+                const float ms = a.part_ml[(slot0 + s) * 2];
+                if (ms != -INFINITY) acc += a.part_o[(slot0 + s) * hd + d] * __expf(ms - mm);
+            }
+            a.out[(size_t)t * a.ldo + (size_t)head * hd + d] = f32_to_bf16(acc * inv);
+        }
     }
+    if (lane == 0) a.counters[unit] = 0;
 }
 
 // ------------------------------------------------------------------ prefill: 16 positions x QT heads per wave
@@ -350,13 +360,13 @@ extern "C" int agave_attn_decode_mfma(const void* q, long ldq, void* out, long l
                                       const void* k_pages, const void* v_pages, const int* table, int width,
                                       const int* base, int n_pages, const int* tok_seq, const int* tok_pos, int N,
                                       int nh, int nkv, int hd, float scale, int window, int splits,
-                                      int pages_per_split, hipStream_t stream) {
+                                      int pages_per_split, int* counters, int seq_is_token, hipStream_t stream) {
     AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
                table, width, base, n_pages, tok_seq, tok_pos, nullptr, 0, nh, nkv, hd, scale, window, splits,
-               pages_per_split};
+               pages_per_split, counters, seq_is_token};
     if (check_common("attn_decode_mfma", a, N)) return -1;
     AGAVE_CHECK(splits >= 1 && pages_per_split >= 1, "attn_decode_mfma: bad split plan %d x %d", splits, pages_per_split);
-    AGAVE_CHECK(splits == 1 || (part_o && part_ml), "attn_decode_mfma: splits need the partial buffers");
+    AGAVE_CHECK(splits == 1 || (part_o && part_ml && counters), "attn_decode_mfma: splits need the partial buffers and counters");
     AGAVE_CHECK(N <= 65535, "attn_decode_mfma: %d tokens exceed the grid limit", N);
     if (N == 0) return 0;
     const int G = nh / nkv;
@@ -365,10 +375,6 @@ extern "C" int agave_attn_decode_mfma(const void* q, long ldq, void* out, long l
     else if (hd <= 128) attn_decode_mfma_kernel<8><<<grid, 64, 0, stream>>>(a);
     else attn_decode_mfma_kernel<16><<<grid, 64, 0, stream>>>(a);
     AGAVE_LAUNCH_CHECK("attn_decode_mfma");
-    if (splits > 1) {
-        attn_combine_kernel<<<N * nh, hd >= 128 ? 128 : 64, 0, stream>>>(part_o, part_ml, (bf16*)out, ldo, nh, hd, splits);
-        AGAVE_LAUNCH_CHECK("attn_combine");
-    }
     return 0;
 }
 
@@ -378,7 +384,7 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
                                        int max_new, int N, int nh, int nkv, int hd, float scale, int window,
                                        hipStream_t stream) {
     AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, nullptr, nullptr, (const uint4*)k_pages, (const uint4*)v_pages,
-               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, 1, 0};
+               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, 1, 0, nullptr, 0};
     if (check_common("attn_prefill_mfma", a, N)) return -1;
     AGAVE_CHECK(cu && n_seqs > 0 && max_new > 0, "attn_prefill_mfma: needs the sequences' token ranges");
     AGAVE_CHECK(n_seqs <= 65535, "attn_prefill_mfma: %d sequences exceed the grid limit", n_seqs);

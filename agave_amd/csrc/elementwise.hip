@@ -82,6 +82,112 @@ __global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict_
     }
 }
 
+// The same with the row held in registers (one read of every input, one write of every
+// output): for rows of up to threads * 4 * VPT elements whose pointers allow 4-wide accesses.
+template <typename T> __device__ __forceinline__ float4 load4(const T* p);
+template <> __device__ __forceinline__ float4 load4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <> __device__ __forceinline__ float4 load4<bf16>(const bf16* p) {
+    const uint2 u = *reinterpret_cast<const uint2*>(p);
+    float4 r;
+    r.x = __uint_as_float(u.x << 16);
+    r.y = __uint_as_float(u.x & 0xffff0000u);
+    r.z = __uint_as_float(u.y << 16);
+    r.w = __uint_as_float(u.y & 0xffff0000u);
+    return r;
+}
+template <typename T> __device__ __forceinline__ void store4(T* p, float4 v);
+template <> __device__ __forceinline__ void store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16(v.x).x | ((uint32_t)f32_to_bf16(v.y).x << 16);
+    u.y = (uint32_t)f32_to_bf16(v.z).x | ((uint32_t)f32_to_bf16(v.w).x << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+
+template <typename T, int VPT>
+__global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb,
+                                          const float* __restrict__ post_gain, float post_eps,
+                                          T* __restrict__ out, long ldo, const float* __restrict__ pre_gain,
+                                          float pre_eps, const int* __restrict__ rows, int e) {
+    __shared__ float red[16];
+    const int i = blockIdx.x;
+    const int r = rows ? rows[i] : i;
+    float* hr = h + (size_t)r * e;
+    float4 hv[VPT], bv[VPT], g1[VPT], g2[VPT];
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+        const int c = (threadIdx.x + v * blockDim.x) * 4;
+        const bool in = c < e;
+        const float4 z = float4{0.f, 0.f, 0.f, 0.f};
+        hv[v] = in ? *reinterpret_cast<const float4*>(hr + c) : z;
+        bv[v] = (in && branch) ? load4(branch + (size_t)r * ldb + c) : z;
+        g1[v] = (in && branch && post_gain) ? *reinterpret_cast<const float4*>(post_gain + c) : z;
+        g2[v] = (in && out) ? *reinterpret_cast<const float4*>(pre_gain + c) : z;
+    }
+    if (branch) {
+        float inv = 1.0f;
+        if (post_gain) {
+            float ss = 0.f;
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) ss += bv[v].x * bv[v].x + bv[v].y * bv[v].y + bv[v].z * bv[v].z + bv[v].w * bv[v].w;
+            ss = block_sum(ss, red);
+            inv = 1.0f / sqrtf(ss / (float)e + post_eps);
+        }
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            if (post_gain) {
+                hv[v].x += bv[v].x * inv * g1[v].x;
+                hv[v].y += bv[v].y * inv * g1[v].y;
+                hv[v].z += bv[v].z * inv * g1[v].z;
+                hv[v].w += bv[v].w * inv * g1[v].w;
+            } else {
+                hv[v].x += bv[v].x;
+                hv[v].y += bv[v].y;
+                hv[v].z += bv[v].z;
+                hv[v].w += bv[v].w;
+            }
+            const int c = (threadIdx.x + v * blockDim.x) * 4;
+            if (c < e) *reinterpret_cast<float4*>(hr + c) = hv[v];
+        }
+    }
+    if (out) {
+        float ss = 0.f;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) ss += hv[v].x * hv[v].x + hv[v].y * hv[v].y + hv[v].z * hv[v].z + hv[v].w * hv[v].w;
+        ss = block_sum(ss, red);
+        const float inv = 1.0f / sqrtf(ss / (float)e + pre_eps);
+        T* o = out + (size_t)i * ldo;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int c = (threadIdx.x + v * blockDim.x) * 4;
+            if (c < e)
+                store4(o + c, float4{hv[v].x * inv * g2[v].x, hv[v].y * inv * g2[v].y, hv[v].z * inv * g2[v].z,
+                                     hv[v].w * inv * g2[v].w});
+        }
+    }
+}
+
+template <typename T>
+static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, const float* post_gain, float post_eps,
+                                      void* out, long ldo, const float* pre_gain, float pre_eps, const int* rows,
+                                      int n_rows, int e, hipStream_t stream) {
+    const size_t align = sizeof(T) * 4;
+    if (e % 4 != 0 || e > 16384 || (branch && (ldb % 4 != 0 || (uintptr_t)branch % align != 0)) ||
+        (out && (ldo % 4 != 0 || (uintptr_t)out % align != 0)) || (uintptr_t)h % 16 != 0 ||
+        (post_gain && (uintptr_t)post_gain % 16 != 0) || (pre_gain && (uintptr_t)pre_gain % 16 != 0))
+        return false;
+    const int threads = e <= 1024 ? 64 * ((e / 4 + 63) / 64) : (e <= 4096 ? 256 : 1024);
+    const int vpt = (e / 4 + threads - 1) / threads;
+#define RN_FAST(V)                                                                                                    \
+    residual_norm_fast_kernel<T, V><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, post_gain, post_eps,   \
+                                                                    (T*)out, ldo, pre_gain, pre_eps, rows, e)
+    if (vpt <= 1) RN_FAST(1);
+    else if (vpt <= 2) RN_FAST(2);
+    else RN_FAST(4);
+#undef RN_FAST
+    return true;
+}
+
 extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long ldb, const float* post_gain,
                                    float post_eps, void* out, long ldo, const float* pre_gain, float pre_eps,
                                    const int* rows, int n_rows, int e, hipStream_t stream) {
@@ -93,7 +199,11 @@ extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long
     AGAVE_CHECK(!(rows && branch), "residual_norm: row gather with a branch is not supported");
     if (n_rows == 0 || (!branch && !out)) return 0;
     const int threads = e >= 2048 ? 512 : (e >= 512 ? 256 : 64);
-    if (dtype == AGAVE_F32)
+    if (dtype == AGAVE_F32 && launch_residual_norm_fast<float>(h, branch, ldb, post_gain, post_eps, out, ldo, pre_gain,
+                                                              pre_eps, rows, n_rows, e, stream)) {
+    } else if (dtype == AGAVE_BF16 && launch_residual_norm_fast<bf16>(h, branch, ldb, post_gain, post_eps, out, ldo,
+                                                                     pre_gain, pre_eps, rows, n_rows, e, stream)) {
+    } else if (dtype == AGAVE_F32)
         residual_norm_kernel<float><<<n_rows, threads, 0, stream>>>(h, (const float*)branch, ldb, post_gain, post_eps,
                                                                     (float*)out, ldo, pre_gain, pre_eps, rows, e);
     else if (dtype == AGAVE_BF16)

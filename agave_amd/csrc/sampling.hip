@@ -95,11 +95,41 @@ __device__ void block_argmax(const float* __restrict__ x, int n, float mult, flo
     *out_i = idx;
 }
 
+// Greedy rows, first pass: the row is cut into ARGMAX_PARTS pieces, one workgroup each, which
+// leave (max, lowest index holding it); sample_kernel picks among them.
+#define ARGMAX_PARTS 64
+__global__ __launch_bounds__(256) void argmax_parts_kernel(const float* __restrict__ logits, long ld,
+                                                           const float* __restrict__ params,
+                                                           float* __restrict__ part_v, int* __restrict__ part_i, int V) {
+    __shared__ float red_v[16];
+    __shared__ int red_i[16];
+    const int b = blockIdx.y, part = blockIdx.x;
+    if (params[b * 4] != 0.f) return;                       // only rows that take the argmax
+    const int per = (V + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+    const int lo = part * per;
+    int n = V - lo;
+    if (n > per) n = per;
+    float mx = -INFINITY;
+    int idx = 0;
+    if (n > 0) {
+        block_argmax(logits + (size_t)b * ld + lo, n, 1.0f, red_v, red_i, &mx, &idx);
+        idx += lo;
+    } else {
+        idx = 0x7fffffff;
+    }
+    if (threadIdx.x == 0) {
+        part_v[b * ARGMAX_PARTS + part] = mx;
+        part_i[b * ARGMAX_PARTS + part] = idx;
+    }
+}
+
 // params[b] = {temperature, top_k, top_p, u}
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits, long ld,
                                                                 float* __restrict__ work, long ldw,
                                                                 const float* __restrict__ params,
-                                                                int* __restrict__ out, int V) {
+                                                                int* __restrict__ out, int V,
+                                                                const float* __restrict__ part_v,
+                                                                const int* __restrict__ part_i) {
     __shared__ float red[16];
     __shared__ float red_v[16];
     __shared__ int red_i[16];
@@ -122,6 +152,23 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     float mx;
     int amax;
     if (temperature == 0.f) {
+        if (part_v) {                                         // the pieces' winners; ties go to the lowest index
+            if (tid < 64) {
+                float v = part_v[b * ARGMAX_PARTS + tid];
+                int i = part_i[b * ARGMAX_PARTS + tid];
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) {
+                    const float ov = __shfl_xor(v, o, 64);
+                    const int oi = __shfl_xor(i, o, 64);
+                    if (ov > v || (ov == v && oi < i)) {
+                        v = ov;
+                        i = oi;
+                    }
+                }
+                if (tid == 0) out[b] = i;
+            }
+            return;
+        }
         block_argmax(x, V, 1.0f, red_v, red_i, &mx, &amax);
         if (tid == 0) out[b] = amax;
         return;
@@ -242,13 +289,22 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     if (tid == 0) out[b] = sh_result;
 }
 
+// scratch: B * 64 floats followed by B * 64 ints for the greedy rows' first pass, or null.
 extern "C" int agave_sample(const float* logits, long ld, float* work, long ldw, const float* params, int* out,
-                            int B, int V, hipStream_t stream) {
+                            int B, int V, float* scratch, hipStream_t stream) {
     AGAVE_CHECK(B >= 0 && V > 0, "sample: bad sizes B=%d V=%d", B, V);
     AGAVE_CHECK(ld >= V && ldw >= V, "sample: a row stride is below the vocabulary");
     AGAVE_CHECK(logits && work && params && out, "sample: null buffer");
     if (B == 0) return 0;
-    sample_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, ld, work, ldw, params, out, V);
+    float* part_v = nullptr;
+    int* part_i = nullptr;
+    if (scratch && V >= 4096 && B <= 65535) {
+        part_v = scratch;
+        part_i = reinterpret_cast<int*>(scratch + (size_t)B * ARGMAX_PARTS);
+        argmax_parts_kernel<<<dim3(ARGMAX_PARTS, B), 256, 0, stream>>>(logits, ld, params, part_v, part_i, V);
+        AGAVE_LAUNCH_CHECK("argmax_parts");
+    }
+    sample_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, ld, work, ldw, params, out, V, part_v, part_i);
     AGAVE_LAUNCH_CHECK("sample");
     return 0;
 }

@@ -186,7 +186,8 @@ class Engine:
                               dtype=torch.float32, device=self.device)
         work = self.workspace.get("sample_work", b, self.spec.vocab_size, torch.float32)
         out = self.workspace.get("sampled", b, 1, torch.int32).view(-1)
-        sample_ops.sample(logits, work, params, out)
+        scratch = self.workspace.get("sample_scratch", b, 128, torch.float32).view(-1)
+        sample_ops.sample(logits, work, params, out, scratch)
         return out.cpu().tolist()
 
     def generate(self, prompts, params=None, max_batch: Optional[int] = None, stats=None):

@@ -7,7 +7,7 @@ from . import kernels, library
 from .kernels import _I, _L, _P
 
 kernels.register_signatures("sampling", {
-    "agave_sample": [_P, _L, _P, _L, _P, _P, _I, _I, _P],
+    "agave_sample": [_P, _L, _P, _L, _P, _P, _I, _I, _P, _P],
     "agave_repeat_penalty": [_P, _L, _P, _P, _P, _I, _I, _P],
 })
 
@@ -20,10 +20,12 @@ def _logits(logits: torch.Tensor) -> int:
     return logits.stride(0)
 
 
-def sample(logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor) -> None:
+def sample(logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor,
+           scratch: torch.Tensor = None) -> None:
     """out[b] = a token drawn from row b.  ``params`` float32 [rows, 4] = temperature, top_k,
     top_p, u; temperature 0 takes the argmax (first index on ties).  ``work``: float32 scratch
-    of the logits' shape."""
+    of the logits' shape.  ``scratch`` (128 float32 per row) lets greedy rows of a large vocabulary be
+    searched by 64 workgroups each."""
     ld = _logits(logits)
     b, v = logits.shape
     if work.dtype != torch.float32 or work.shape != logits.shape or work.stride(1) != 1 or not work.is_cuda:
@@ -32,8 +34,11 @@ def sample(logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: 
         raise TypeError(f"sample: params must be contiguous float32 [{b}, 4] on the GPU")
     if out.dtype != torch.int32 or out.numel() != b or not out.is_contiguous() or not out.is_cuda:
         raise TypeError(f"sample: out must be {b} contiguous int32 on the GPU")
+    if scratch is not None and (scratch.dtype != torch.float32 or scratch.numel() < 128 * b or not scratch.is_cuda
+                                or not scratch.is_contiguous()):
+        raise TypeError(f"sample: scratch must be {128 * b} contiguous float32 on the GPU")
     library.call(kernels.lib("sampling"), "agave_sample", logits.data_ptr(), ld, work.data_ptr(), work.stride(0),
-                 params.data_ptr(), out.data_ptr(), b, v, kernels.stream())
+                 params.data_ptr(), out.data_ptr(), b, v, kernels.ptr(scratch), kernels.stream())
 
 
 def repeat_penalty(logits: torch.Tensor, ids: torch.Tensor, cu: torch.Tensor, penalty: torch.Tensor) -> None:

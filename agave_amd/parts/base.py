@@ -59,6 +59,17 @@ class Workspace:
     def reserve(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> None:
         self.get(name, rows, cols, dtype)
 
+    def zeros(self, name: str, n: int, dtype: torch.dtype = torch.int32) -> torch.Tensor:
+        """A zero-filled buffer that is zeroed only when it is made: for counters that every
+        kernel using them leaves at zero again."""
+        key = f"zeros:{name}:{dtype}"
+        buf = self._buffers.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.zeros(max(n, 1024 if buf is None else 2 * buf.numel()), dtype=dtype, device=self.device)
+            self._buffers[key] = buf
+            self.generation += 1
+        return buf[:n]
+
 
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {"norm": {}, "position": {}, "mixer": {}, "ffn": {}, "block": {}}
 

@@ -261,7 +261,11 @@ def _sample(S, logits, params):
     work = torch.empty_like(lg)
     out = torch.empty(lg.shape[0], dtype=torch.int32, device=DEV)
     S.sample(lg, work, torch.tensor(params, dtype=torch.float32, device=DEV), out)
-    return out.cpu().tolist()
+    got = out.cpu().tolist()
+    scratch = torch.empty(128 * lg.shape[0], dtype=torch.float32, device=DEV)     # greedy rows in 64 pieces
+    S.sample(lg, work, torch.tensor(params, dtype=torch.float32, device=DEV), out, scratch)
+    assert out.cpu().tolist() == got
+    return got
 
 
 def test_argmax_first_of_ties(S):
