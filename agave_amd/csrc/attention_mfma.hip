@@ -1,6 +1,6 @@
 // bfloat16 attention over the paged cache on the matrix cores of gfx950 (head sizes in steps
 // of 16 up to 256): a decode kernel that splits a sequence's keys over workgroups
-// (flash-decoding) whose last workgroup adds the splits up, and a prefill kernel for steps that bring many tokens.
+// (flash-decoding) with a combine pass, and a prefill kernel for steps that bring many tokens.
 // Scores, the running maximum and sum, and the output accumulate in 32-bit; probabilities
 // are rounded to bfloat16 only as the operand of the P*V product.
 //
@@ -45,8 +45,8 @@ struct AttnArgs {
     float scale;
     int window;
     int splits, pages_per_split;
-    int* counters;       // decode with splits: one zeroed counter per (token, kv head chunk); left zeroed
     int seq_is_token;    // decode: sequence index == token index
+    int table_from_reach; // decode: each table row starts at the first page its token reaches (base[b] == lo / 64)
 };
 
 // One wave: QT tiles of 16 query slots against the pages [page_lo, page_hi] of one sequence
@@ -188,16 +188,24 @@ __device__ __forceinline__ long page_of(const AttnArgs& a, int b, int page_idx) 
 }
 
 // ------------------------------------------------------------------ decode: one token per (z), splits over keys
-// grid (split, kv head * head chunks, token); one wave per workgroup.  Query slots are the
-// heads of the group (16 per chunk).
+// grid (split, kv head * head chunks, token); 4 waves per workgroup take the split's pages in
+// turn and merge in LDS.  Query slots are the heads of the group (16 per chunk).
 template <int HDT>
-__global__ __launch_bounds__(64) void attn_decode_mfma_kernel(AttnArgs a) {
-    const int lane = threadIdx.x, j = lane & 15, g = lane >> 4;
+__global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(AttnArgs a) {
+    extern __shared__ float lds[];            // [4 waves][slots][hd] outputs, then [4][16][2] (max, sum)
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
     const int G = a.nh / a.nkv;
     const int chunks = (G + 15) / 16;
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int slots = (G - chunk * 16 < 16) ? G - chunk * 16 : 16;
     const int t = blockIdx.z, split = blockIdx.x;
-    const int b = a.seq_is_token ? t : a.tok_seq[t], p = a.tok_pos[t];
+    const int b = a.seq_is_token ? t : a.tok_seq[t];
+    // when table rows start at the first page the token reaches, this wave's first page id needs
+    // nothing but the grid position: fetch it before anything that waits for the position
+    const int col0 = split * a.pages_per_split + wave;
+    long pg0 = -1;
+    if (a.table_from_reach && col0 < a.width) pg0 = a.table[(size_t)b * a.width + col0];
+    const int p = a.tok_pos[t];
     const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
     const int first = lo / AGAVE_PAGE, last = p / AGAVE_PAGE;
     const int page_lo = first + split * a.pages_per_split;
@@ -205,7 +213,7 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(AttnArgs a) {
     if (page_hi > last) page_hi = last;
     const int hd = a.hd, hdt = hd >> 4;
     const int head_j = kvh * G + chunk * 16 + j;                 // this lane's column as a head
-    const bool col_ok = chunk * 16 + j < G;
+    const bool col_ok = j < slots;
 
     WaveAttn<HDT, 1> w;
     w.init(1);
@@ -213,74 +221,104 @@ __global__ __launch_bounds__(64) void attn_decode_mfma_kernel(AttnArgs a) {
     w.load_q(q_row, 1, hd, lane);
     const int pos[1] = {p}, los[1] = {lo};
     const size_t k_stride = (size_t)4 * ((hd + 31) >> 5) * 64, v_stride = (size_t)hdt * 2 * 64;   // uint4 per (page, kv head)
-    for (int pi = page_lo; pi <= page_hi; ++pi) {
-        const long pg = page_of(a, b, pi);
+    for (int pi = page_lo + wave; pi <= page_hi; pi += 4) {
+        long pg;
+        if (a.table_from_reach) {
+            const int col = pi - first;
+            pg = (col == col0) ? pg0 : (col < a.width ? a.table[(size_t)b * a.width + col] : -1);
+            if (pg >= a.n_pages) pg = -1;
+        } else {
+            pg = page_of(a, b, pi);
+        }
         if (pg < 0) continue;
         w.page(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride, a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride, pi, 1,
                hd, a.scale, pos, los, lane);
     }
     w.finish_sums(1);
-    // rows of the output tiles are heads 4g + e of the chunk; their sums live in the columns
-    float l4[4], m4[4];
+    // every wave leaves its (unnormalised) rows, maxima and sums in LDS
+    float* sm_o = lds;
+    float* sm_ml = lds + (size_t)4 * slots * hd;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-        l4[e] = __shfl(w.l[0], 4 * g + e, 64);
-        m4[e] = __shfl(w.m[0], 4 * g + e, 64);
-    }
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const int hq = chunk * 16 + 4 * g + e;
-        if (hq >= G) continue;
-        const int head = kvh * G + hq;
-        if (a.splits == 1) {
-            const float inv = l4[e] > 0.f ? 1.0f / l4[e] : 0.f;
-            bf16* dst = a.out + (size_t)t * a.ldo + (size_t)head * hd;
-#pragma unroll
-            for (int d = 0; d < HDT; ++d)
-                if (d < hdt) dst[16 * d + j] = f32_to_bf16(w.o[0][d][e] * inv);
-        } else {
-            const size_t slot = ((size_t)t * a.nh + head) * a.splits + split;
-            float* dst = a.part_o + slot * hd;
+        const int slot = 4 * g + e;
+        if (slot < slots) {
+            float* dst = sm_o + ((size_t)wave * slots + slot) * hd;
 #pragma unroll
             for (int d = 0; d < HDT; ++d)
                 if (d < hdt) dst[16 * d + j] = w.o[0][d][e];
-            if (j == 0) {
-                a.part_ml[slot * 2 + 0] = m4[e];
-                a.part_ml[slot * 2 + 1] = l4[e];
-            }
         }
     }
-    if (a.splits == 1) return;
-    // The workgroup that finishes last for this (token, kv head chunk) adds the splits up, in
-    // the order of the splits:  out = sum_s O_s e^(m_s - m) / sum_s l_s e^(m_s - m).
-    __threadfence();
-    const int unit = t * gridDim.y + blockIdx.y;
-    int done = 0;
-    if (lane == 0) done = atomicAdd(a.counters + unit, 1);
-    done = __shfl(done, 0, 64);
-    if (done != a.splits - 1) return;
-    __threadfence();
-    for (int hq = 0; hq < 16 && chunk * 16 + hq < G; ++hq) {
-        const int head = kvh * G + chunk * 16 + hq;
-        const size_t slot0 = ((size_t)t * a.nh + head) * a.splits;
+    if (lane < 16) {
+        sm_ml[(wave * 16 + lane) * 2 + 0] = w.m[0];
+        sm_ml[(wave * 16 + lane) * 2 + 1] = w.l[0];
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < slots * hd; idx += 256) {
+        const int slot = idx / hd, d = idx % hd;
         float mm = -INFINITY;
-        for (int s = 0; s < a.splits; ++s) mm = fmaxf(mm, a.part_ml[(slot0 + s) * 2]);
-        float ll = 0.f;
-        for (int s = 0; s < a.splits; ++s) {
-            const float ms = a.part_ml[(slot0 + s) * 2];
-            if (ms != -INFINITY) ll += a.part_ml[(slot0 + s) * 2 + 1] * __expf(ms - mm);
-        }
-        const float inv = ll > 0.f ? 1.0f / ll : 0.f;
-        for (int d = lane; d < hd; d += 64) {
-            float acc = 0.f;
-            for (int s = 0; s < a.splits; ++s) {
-                const float ms = a.part_ml[(slot0 + s) * 2];
-                if (ms != -INFINITY) acc += a.part_o[(slot0 + s) * hd + d] * __expf(ms - mm);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) mm = fmaxf(mm, sm_ml[(x * 16 + slot) * 2]);
+        float acc = 0.f, ll = 0.f;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const float mx = sm_ml[(x * 16 + slot) * 2];
+            if (mx != -INFINITY) {
+                const float f = __expf(mx - mm);
+                acc += sm_o[((size_t)x * slots + slot) * hd + d] * f;
+                ll += sm_ml[(x * 16 + slot) * 2 + 1] * f;
             }
-            a.out[(size_t)t * a.ldo + (size_t)head * hd + d] = f32_to_bf16(acc * inv);
+        }
+        const int head = kvh * G + chunk * 16 + slot;
+        if (a.splits == 1) {
+            a.out[(size_t)t * a.ldo + (size_t)head * hd + d] = f32_to_bf16(ll > 0.f ? acc / ll : 0.f);
+        } else {
+            const size_t ps = ((size_t)t * a.nh + head) * a.splits + split;
+            a.part_o[ps * hd + d] = acc;
+            if (d == 0) {
+                a.part_ml[ps * 2 + 0] = mm;
+                a.part_ml[ps * 2 + 1] = ll;
+            }
         }
     }
-    if (lane == 0) a.counters[unit] = 0;
+}
+
+// out[t][head] = sum_s O_s * exp(m_s - m) / sum_s l_s * exp(m_s - m)
+#define COMBINE_MAX_SPLITS 256
+__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                    bf16* __restrict__ out, long ldo, int nh, int hd, int splits) {
+    __shared__ float wgt[COMBINE_MAX_SPLITS];
+    __shared__ float red[16];
+    const int t = blockIdx.x / nh, head = blockIdx.x % nh;
+    const size_t slot0 = ((size_t)t * nh + head) * splits;
+    // every split's maximum and sum are fetched at once, one split per thread
+    float ms[COMBINE_MAX_SPLITS / 64], ls[COMBINE_MAX_SPLITS / 64];
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < COMBINE_MAX_SPLITS / 64; ++i) {
+        const int sidx = threadIdx.x + i * blockDim.x;
+        const bool in = i * (int)blockDim.x < splits && sidx < splits;
+        ms[i] = in ? part_ml[(slot0 + sidx) * 2] : -INFINITY;
+        ls[i] = in ? part_ml[(slot0 + sidx) * 2 + 1] : 0.f;
+        m = fmaxf(m, ms[i]);
+    }
+    m = block_max(m, red);
+    float l = 0.f;
+#pragma unroll
+    for (int i = 0; i < COMBINE_MAX_SPLITS / 64; ++i) {
+        const int sidx = threadIdx.x + i * blockDim.x;
+        const float f = (ms[i] != -INFINITY) ? __expf(ms[i] - m) : 0.f;
+        if (sidx < COMBINE_MAX_SPLITS) wgt[sidx] = f;
+        l += ls[i] * f;
+    }
+    l = block_sum(l, red);            // its barriers also publish wgt[]
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+        float acc = 0.f;
+        const float* po = part_o + slot0 * hd + d;
+#pragma unroll 8
+        for (int sp = 0; sp < splits; ++sp) acc += po[(size_t)sp * hd] * wgt[sp];
+        out[(size_t)t * ldo + (size_t)head * hd + d] = f32_to_bf16(acc * inv);
+    }
 }
 
 // ------------------------------------------------------------------ prefill: 16 positions x QT heads per wave
@@ -360,21 +398,35 @@ extern "C" int agave_attn_decode_mfma(const void* q, long ldq, void* out, long l
                                       const void* k_pages, const void* v_pages, const int* table, int width,
                                       const int* base, int n_pages, const int* tok_seq, const int* tok_pos, int N,
                                       int nh, int nkv, int hd, float scale, int window, int splits,
-                                      int pages_per_split, int* counters, int seq_is_token, hipStream_t stream) {
+                                      int pages_per_split, int seq_is_token, int table_from_reach,
+                                      hipStream_t stream) {
     AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
                table, width, base, n_pages, tok_seq, tok_pos, nullptr, 0, nh, nkv, hd, scale, window, splits,
-               pages_per_split, counters, seq_is_token};
+               pages_per_split, seq_is_token, table_from_reach};
     if (check_common("attn_decode_mfma", a, N)) return -1;
-    AGAVE_CHECK(splits >= 1 && pages_per_split >= 1, "attn_decode_mfma: bad split plan %d x %d", splits, pages_per_split);
-    AGAVE_CHECK(splits == 1 || (part_o && part_ml && counters), "attn_decode_mfma: splits need the partial buffers and counters");
+    AGAVE_CHECK(splits >= 1 && splits <= COMBINE_MAX_SPLITS && pages_per_split >= 1, "attn_decode_mfma: bad split plan %d x %d", splits, pages_per_split);
+    AGAVE_CHECK(splits == 1 || (part_o && part_ml), "attn_decode_mfma: splits need the partial buffers");
     AGAVE_CHECK(N <= 65535, "attn_decode_mfma: %d tokens exceed the grid limit", N);
     if (N == 0) return 0;
     const int G = nh / nkv;
     dim3 grid(splits, nkv * ((G + 15) / 16), N);
-    if (hd <= 64) attn_decode_mfma_kernel<4><<<grid, 64, 0, stream>>>(a);
-    else if (hd <= 128) attn_decode_mfma_kernel<8><<<grid, 64, 0, stream>>>(a);
-    else attn_decode_mfma_kernel<16><<<grid, 64, 0, stream>>>(a);
+    const int slots = G < 16 ? G : 16;
+    const size_t lds = ((size_t)4 * slots * hd + 4 * 16 * 2) * sizeof(float);
+    AGAVE_CHECK(lds <= 96 * 1024, "attn_decode_mfma: %zu bytes of LDS exceed what a workgroup may take", lds);
+    if (lds > 48 * 1024) {       // more than the default allowance: ask for it (once per kernel would do)
+        hipError_t e1 = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        hipError_t e2 = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        hipError_t e3 = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        AGAVE_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "attn_decode_mfma: cannot raise the LDS allowance");
+    }
+    if (hd <= 64) attn_decode_mfma_kernel<4><<<grid, 256, lds, stream>>>(a);
+    else if (hd <= 128) attn_decode_mfma_kernel<8><<<grid, 256, lds, stream>>>(a);
+    else attn_decode_mfma_kernel<16><<<grid, 256, lds, stream>>>(a);
     AGAVE_LAUNCH_CHECK("attn_decode_mfma");
+    if (splits > 1) {
+        attn_combine_kernel<<<N * nh, hd >= 256 ? 256 : (hd >= 128 ? 128 : 64), 0, stream>>>(part_o, part_ml, (bf16*)out, ldo, nh, hd, splits);
+        AGAVE_LAUNCH_CHECK("attn_combine");
+    }
     return 0;
 }
 
@@ -384,7 +436,7 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
                                        int max_new, int N, int nh, int nkv, int hd, float scale, int window,
                                        hipStream_t stream) {
     AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, nullptr, nullptr, (const uint4*)k_pages, (const uint4*)v_pages,
-               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, 1, 0, nullptr, 0};
+               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, 1, 0, 0, 0};
     if (check_common("attn_prefill_mfma", a, N)) return -1;
     AGAVE_CHECK(cu && n_seqs > 0 && max_new > 0, "attn_prefill_mfma: needs the sequences' token ranges");
     AGAVE_CHECK(n_seqs <= 65535, "attn_prefill_mfma: %d sequences exceed the grid limit", n_seqs);

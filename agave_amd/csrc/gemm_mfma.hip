@@ -95,19 +95,17 @@ __device__ __forceinline__ float gelu_tanh_f(float x) {
 #define SK_KS 4                    // k-steps (tiles of 32 columns) per chunk
 #define SK_ROW (SK_KS * 32 + 8)    // bf16 per staged X row: 128 columns + 16 bytes of padding
 
-// R: row blocks (of 16 weight rows) per workgroup; MT: tiles of 16 tokens; EPI 0: store, 1: GeGLU.
-// With SK = gridDim.y > 1 the columns are split over SK workgroups as well: each leaves its
-// partial sums in `part`, and the one that finishes last for a row block adds them up in the
-// order of the splits (so the result does not depend on which one that is).
-template <int R, int MT, int EPI, typename TC>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict__ X, long ldx,
+// R: row blocks (of 16 weight rows) per workgroup; MT: tiles of 16 tokens; EPI 0: store, 1: GeGLU;
+// NW: waves per workgroup, which share the columns (few row blocks -> many waves each, so
+// that a small matrix still has enough loads in flight; the sums meet in LDS, never in memory).
+template <int R, int MT, int EPI, int NW, typename TC>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ X, long ldx,
                                                           const uint4* __restrict__ Wp, TC* __restrict__ Y,
-                                                          long ldy, int M, int N, int K, int KB, int NB,
-                                                          float* __restrict__ part, int* __restrict__ counters) {
+                                                          long ldy, int M, int N, int K, int KB, int NB) {
     // staged X: [wave][MT][16 rows][SK_ROW]; afterwards the same memory holds the waves' partial sums
     constexpr int XS_WAVE = MT * 16 * SK_ROW;                       // bf16 elements
     constexpr int RED_WAVE = R * MT * 64 * 4;                       // floats
-    constexpr int LDS_BYTES = (4 * XS_WAVE * 2 > 4 * RED_WAVE * 4) ? 4 * XS_WAVE * 2 : 4 * RED_WAVE * 4;
+    constexpr int LDS_BYTES = (NW * XS_WAVE * 2 > NW * RED_WAVE * 4) ? NW * XS_WAVE * 2 : NW * RED_WAVE * 4;
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
     bf16* xs = reinterpret_cast<bf16*>(smem);
     float* red = reinterpret_cast<float*>(smem);
@@ -116,9 +114,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
     const int j = lane & 15, g = lane >> 4;
     const int nb0 = blockIdx.x * R;
     const int n_chunks = (KB + SK_KS - 1) / SK_KS;
-    const int SK = gridDim.y, sk = blockIdx.y;
-    const int gw = sk * 4 + wave, GW = 4 * SK;         // this wave among all that share the columns
-    const int n_iter = (n_chunks + GW - 1) / GW;
+    const int n_iter = (n_chunks + NW - 1) / NW;
 
     f32x4_t acc[R][MT];
 #pragma unroll
@@ -131,7 +127,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
     bf16* my_xs = xs + wave * XS_WAVE;
 
     auto load_global = [&](int it) {
-        const int c = it * GW + gw;                  // chunks are dealt to the waves in turn
+        const int c = it * NW + wave;                // chunks are dealt to the waves in turn
         const bool active = c < n_chunks;
 #pragma unroll
         for (int r = 0; r < R; ++r)
@@ -182,42 +178,20 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
         __syncthreads();
     }
 
-    // the four waves' partial sums meet in LDS
+    // the waves' partial sums meet in LDS
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
             *reinterpret_cast<f32x4_t*>(red + ((size_t)wave * R * MT + r * MT + mt) * 256 + lane * 4) = acc[r][mt];
     __syncthreads();
-    __shared__ int is_last;
-    if (SK > 1) {
-        // this workgroup's sums go to memory; the last workgroup of the row block carries on
-        for (int tile = wave; tile < R * MT; tile += 4) {
-            f32x4_t s = *reinterpret_cast<const f32x4_t*>(red + (size_t)tile * 256 + lane * 4);
-#pragma unroll
-            for (int w = 1; w < 4; ++w)
-                s += *reinterpret_cast<const f32x4_t*>(red + ((size_t)w * R * MT + tile) * 256 + lane * 4);
-            *reinterpret_cast<f32x4_t*>(part + (((size_t)blockIdx.x * SK + sk) * R * MT + tile) * 256 + lane * 4) = s;
-        }
-        __threadfence();
-        __syncthreads();
-        if (threadIdx.x == 0) is_last = (atomicAdd(counters + blockIdx.x, 1) == SK - 1);
-        __syncthreads();
-        if (!is_last) return;
-        __threadfence();
-    }
-    for (int tile = wave; tile < R * MT; tile += 4) {
+    for (int tile = wave; tile < R * MT; tile += NW) {
         const int r = tile / MT, mt = tile % MT;
-        f32x4_t s;
-        if (SK > 1) {
-            s = *reinterpret_cast<const f32x4_t*>(part + (((size_t)blockIdx.x * SK) * R * MT + tile) * 256 + lane * 4);
-            for (int k2 = 1; k2 < SK; ++k2)
-                s += *reinterpret_cast<const f32x4_t*>(part + (((size_t)blockIdx.x * SK + k2) * R * MT + tile) * 256 + lane * 4);
-        } else {
-            s = *reinterpret_cast<const f32x4_t*>(red + (size_t)tile * 256 + lane * 4);
+        f32x4_t s = *reinterpret_cast<const f32x4_t*>(red + (size_t)tile * 256 + lane * 4);
 #pragma unroll
-            for (int w = 1; w < 4; ++w)
-                s += *reinterpret_cast<const f32x4_t*>(red + ((size_t)w * R * MT + tile) * 256 + lane * 4);
+        for (int w = 1; w < NW; ++w) {
+            const f32x4_t p = *reinterpret_cast<const f32x4_t*>(red + ((size_t)w * R * MT + tile) * 256 + lane * 4);
+            s += p;
         }
         const int m = mt * 16 + j;
         if (m >= M || nb0 + r >= NB) continue;
@@ -232,54 +206,43 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16* __restrict
             if (n + 1 < N) st(Y + (size_t)m * ldy + n + 1, gelu_tanh_f(s[1]) * s[3]);
         }
     }
-    if (SK > 1 && threadIdx.x == 0) counters[blockIdx.x] = 0;      // left zeroed for the next launch
 }
 
-// How many workgroups share the columns of one row block: enough to fill the chip when there
-// are few row blocks, and dividing the chunks of columns evenly.
-static int pick_split(int row_groups, int n_chunks) {
-    if (row_groups >= 1024) return 1;
-    int best = 1;
-    double best_score = -1.0;
-    for (int sk = 1; sk <= 16; ++sk) {
-        const int gw = 4 * sk;
-        if (sk > 1 && gw > n_chunks) break;
-        const int n_iter = (n_chunks + gw - 1) / gw;
-        const double even = (double)n_chunks / ((double)n_iter * gw);          // 1: no idle wave
-        const double fill = row_groups * sk >= 1024 ? 1.0 : (double)(row_groups * sk) / 1024.0;
-        const double score = even * fill - 0.01 * sk;
-        if (score > best_score) {
-            best_score = score;
-            best = sk;
-        }
-    }
-    return best;
+template <int R, int MT, int EPI, int NW, typename TC>
+static void launch_skinny_nw(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
+                             int NB, hipStream_t stream) {
+    const int grid = (NB + R - 1) / R;
+    gemm_skinny_kernel<R, MT, EPI, NW, TC><<<grid, NW * 64, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y,
+                                                                        ldy, M, N, K, KB, NB);
 }
-
-#define SK_PART_FLOATS_PER_TILE 256
-extern "C" long agave_gemm_skinny_scratch_floats() { return (long)2048 * 4 * SK_PART_FLOATS_PER_TILE + 4096; }
-extern "C" int agave_gemm_skinny_counters() { return 1024; }
 
 template <int R, int MT, int EPI, typename TC>
 static void launch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
-                          int NB, float* part, int* counters, hipStream_t stream) {
-    const int groups = (NB + R - 1) / R;
+                          int NB, hipStream_t stream) {
+    // waves per workgroup: as many as the chunks of columns and the LDS allow while row blocks are few
     const int n_chunks = (KB + SK_KS - 1) / SK_KS;
-    int sk = (part && counters) ? pick_split(groups, n_chunks) : 1;
-    if (sk > 1 && (groups > 1024 || (long)groups * sk * R * MT > 2048L * 4)) sk = 1;     // what the scratch holds
-    dim3 grid(groups, sk);
-    gemm_skinny_kernel<R, MT, EPI, TC><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy, M,
-                                                                N, K, KB, NB, part, counters);
+    const int groups = (NB + R - 1) / R;
+    int nw = groups >= 1536 ? 4 : (groups >= 640 ? 8 : 16);
+    if (MT >= 3 && nw > 4) nw = 4;
+    if (MT == 2 && nw > 8) nw = 8;
+    while (nw > 4 && nw > n_chunks) nw /= 2;
+    if (nw == 16) {
+        if constexpr (MT == 1) launch_skinny_nw<R, MT, EPI, 16, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    } else if (nw == 8) {
+        if constexpr (MT <= 2) launch_skinny_nw<R, MT, EPI, 8, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    } else {
+        launch_skinny_nw<R, MT, EPI, 4, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    }
 }
 
 template <int EPI, typename TC>
 static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
-                           int NB, float* part, int* counters, hipStream_t stream) {
+                           int NB, hipStream_t stream) {
     const int mt = (M + 15) / 16;
     // two row blocks per workgroup once there are plenty of them, so that X is staged half as often
     const bool wide = NB >= 4096;
 #define SK_CASE(R_, MT_)                                                                        \
-    launch_skinny<R_, MT_, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, part, counters, stream); \
+    launch_skinny<R_, MT_, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);              \
     break
     switch (mt) {
         case 1: if (wide) { SK_CASE(2, 1); } else { SK_CASE(1, 1); }
@@ -293,10 +256,8 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
 }
 
 // N: logical outputs (rows of W, or ff for the GeGLU epilogue); Wp holds NB row blocks.
-// part / counters: scratch of agave_gemm_skinny_scratch_floats() floats and
-// agave_gemm_skinny_counters() zeroed ints (left zeroed), or null to keep each row block in one workgroup.
 extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,
-                                 int K, int epilogue, float* part, int* counters, hipStream_t stream) {
+                                 int K, int epilogue, hipStream_t stream) {
     AGAVE_CHECK(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d (M <= 64)", M, N, K);
     AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
                 "gemm_skinny: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
@@ -307,12 +268,12 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
     const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
     int rc;
     if (epilogue == 0) {
-        if (dt_y == AGAVE_BF16) rc = dispatch_skinny<0, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, part, counters, stream);
-        else if (dt_y == AGAVE_F32) rc = dispatch_skinny<0, float>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, part, counters, stream);
+        if (dt_y == AGAVE_BF16) rc = dispatch_skinny<0, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        else if (dt_y == AGAVE_F32) rc = dispatch_skinny<0, float>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
         else AGAVE_CHECK(false, "gemm_skinny: unknown output dtype %d", dt_y);
     } else {
         AGAVE_CHECK(dt_y == AGAVE_BF16, "gemm_skinny: the GeGLU epilogue writes bfloat16");
-        rc = dispatch_skinny<1, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, part, counters, stream);
+        rc = dispatch_skinny<1, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     }
     if (rc != 0) return rc;
     AGAVE_LAUNCH_CHECK("gemm_skinny");

@@ -53,6 +53,7 @@ class Step:
     cache: KVCache
     workspace: object = None
     fixed_span: Optional[int] = None    # a captured decode graph plans its splits for this many pages
+    tables_start_at_reach: bool = False  # decode: column 0 of every table row is the first page the token reaches
 
     def page_span(self, window: Optional[int]) -> int:
         """Most pages any sequence's last token of this step reaches back over."""
@@ -189,7 +190,7 @@ class StepPlanner:
             tokens=view(s_tok), tok_seq=view(s_seq), tok_pos=view(s_pos), slots_dev=view(s_slots),
             pos0_dev=view(s_pos0), cu_dev=view(s_cu), want_rows=view(s_want),
             tables=[(view(t).view(b, w), view(sb)) for t, sb, w in s_tables], cache=self.cache,
-            workspace=self.workspace)
+            workspace=self.workspace, tables_start_at_reach=(max(n_new) == 1))
 
     def commit(self, step: Step) -> None:
         self.cache.commit_step(step.slots, step.n_new)

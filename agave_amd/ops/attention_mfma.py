@@ -9,18 +9,18 @@ from . import kernels, library
 from .kernels import _F, _I, _L, _P
 
 kernels.register_signatures("attention_mfma", {
-    "agave_attn_decode_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _P, _I,
-                               _P],
+    "agave_attn_decode_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _I,
+                               _I, _P],
     "agave_attn_prefill_mfma": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
 })
 
-TARGET_WAVES = 2048          # workgroups a decode launch aims for (8 per compute unit)
+TARGET_WORKGROUPS = 256      # workgroups (of 4 waves) a decode launch aims for: one per compute unit
 
 
 def split_plan(page_span: int, units: int):
     """(splits, pages per split) for sequences spanning at most ``page_span`` pages when the launch
-    has ``units`` (token, kv head) pairs."""
-    want = max(1, min(page_span, -(-TARGET_WAVES // max(units, 1))))
+    has ``units`` (token, kv head) pairs.  A workgroup's four waves take one page each at a time."""
+    want = max(1, min(page_span, -(-TARGET_WORKGROUPS // max(units, 1))))
     per = -(-page_span // want)
     return -(-page_span // per), per
 
@@ -43,17 +43,17 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
         span = step.page_span(window)
         chunks = -(-(n_heads // n_kv) // 16)
         splits, per = split_plan(span, n * n_kv * chunks)
-        part_o = part_ml = counters = None
+        part_o = part_ml = None
         if splits > 1:
             ws = step.workspace
             part_o = ws.get("attn_part_o", n * n_heads * splits, head_dim, torch.float32)
             part_ml = ws.get("attn_part_ml", n * n_heads * splits, 2, torch.float32)
-            counters = ws.zeros("attn_counters", n * n_kv * chunks)      # the kernel leaves them zeroed
         library.call(lib, "agave_attn_decode_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
                      kernels.ptr(part_o), kernels.ptr(part_ml), k_pages.data_ptr(), v_pages.data_ptr(),
                      table.data_ptr(), width, base.data_ptr(), n_pages, step.tok_seq.data_ptr(),
                      step.tok_pos.data_ptr(), n, n_heads, n_kv, head_dim, scale, w, splits, per,
-                     kernels.ptr(counters), 1 if step.n_seqs == n else 0, kernels.stream())
+                     1 if step.n_seqs == n else 0, 1 if getattr(step, "tables_start_at_reach", False) else 0,
+                     kernels.stream())
     else:
         library.call(lib, "agave_attn_prefill_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
                      k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width, base.data_ptr(), n_pages,

@@ -3,8 +3,6 @@ from __future__ import annotations
 
 from typing import Optional
 
-import ctypes
-
 import torch
 
 from . import kernels, library
@@ -13,7 +11,7 @@ from .kernels import _F, _I, _L, _P
 kernels.register_signatures("gemm_mfma", {
     "agave_pack_w16": [_P, _L, _P, _I, _I, _I, _I, _P],
     "agave_embed_scale_packed": [_P, _P, _F, _P, _I, _I, _I, _P],
-    "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P, _P, _P],
+    "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P],
 })
 
 SKINNY_MAX_M = 64
@@ -39,22 +37,6 @@ def _x_ok(x: torch.Tensor) -> bool:
             and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0)
 
 
-_scratch = {}
-
-
-def _split_scratch(device):
-    """Scratch for products whose columns are split over workgroups: partial sums, and counters
-    that every launch leaves zeroed."""
-    got = _scratch.get(device)
-    if got is None:
-        h = kernels.lib("gemm_mfma")
-        h.agave_gemm_skinny_scratch_floats.restype = ctypes.c_long
-        part = torch.empty(h.agave_gemm_skinny_scratch_floats(), dtype=torch.float32, device=device)
-        counters = torch.zeros(h.agave_gemm_skinny_counters(), dtype=torch.int32, device=device)
-        got = _scratch[device] = (part, counters)
-    return got
-
-
 def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, epilogue: int = 0) -> None:
     """out[M, n_out] = x[M, K] @ W^T (epilogue 0) or gelu_tanh(gate) * up (epilogue 1) for M <= 64."""
     if not (x.is_cuda and packed.is_cuda and out.is_cuda):
@@ -67,10 +49,8 @@ def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int,
     nb = (n_out + 7) // 8 if epilogue else (n_out + 15) // 16
     if packed.numel() != nb * ((k + 31) // 32) * 512:
         raise ValueError("skinny product: the packed weight does not fit these sizes")
-    part, counters = _split_scratch(x.device)
     library.call(kernels.lib("gemm_mfma"), "agave_gemm_skinny", x.data_ptr(), x.stride(0), packed.data_ptr(),
-                 kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue, part.data_ptr(),
-                 counters.data_ptr(), kernels.stream())
+                 kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue, kernels.stream())
 
 
 def try_linear(x: torch.Tensor, lin, out: torch.Tensor) -> bool:
