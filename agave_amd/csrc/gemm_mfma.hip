@@ -279,3 +279,149 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
     AGAVE_LAUNCH_CHECK("gemm_skinny");
     return 0;
 }
+
+
+// ------------------------------------------------------------------ tiled product (prefill)
+// A workgroup of four waves (2 x 2) computes 128 weight rows x 256 tokens; a wave 64 rows x 128
+// tokens as 4 x 8 MFMA tiles, so every weight tile it loads (straight from the packed layout,
+// coalesced, no LDS) meets eight token tiles and every token tile (staged through LDS, shared
+// by the workgroup) meets four weight tiles.  Two k-steps of 32 columns per stage, the next
+// stage's loads are in flight while the current one is multiplied.
+// blockIdx.x walks the weight rows, so that workgroups sharing weight rows (ids a multiple of
+// the number of row tiles apart) tend to land on the same XCD and find them in its L2.
+#define TL_KT 2                       // k-steps per stage
+#define TL_ROW (TL_KT * 32 + 8)       // bf16 per staged token row (16 bytes of padding)
+#define TL_WM 8                       // token tiles per wave
+#define TL_WN 4                       // weight-row tiles per wave
+
+template <int EPI, typename TC>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
+                                                         const uint4* __restrict__ Wp, TC* __restrict__ Y, long ldy,
+                                                         int M, int N, int K, int KB, int NB) {
+    __shared__ __attribute__((aligned(16))) bf16 xs[2][256][TL_ROW];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int j = lane & 15, g = lane >> 4;
+    const int wn = wave & 1, wm = wave >> 1;
+    const int nb0 = blockIdx.x * 8 + wn * TL_WN;          // first weight-row tile of this wave
+    const int m0 = blockIdx.y * 256;                      // first token of this workgroup
+    const int n_stage = (KB + TL_KT - 1) / TL_KT;
+
+    f32x4_t acc[TL_WN][TL_WM];
+#pragma unroll
+    for (int a = 0; a < TL_WN; ++a)
+#pragma unroll
+        for (int b = 0; b < TL_WM; ++b) acc[a][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    frag16 wreg[TL_WN][TL_KT];
+    uint4 xreg[8];
+
+    auto load_stage = [&](int st) {
+#pragma unroll
+        for (int a = 0; a < TL_WN; ++a)
+#pragma unroll
+            for (int ks = 0; ks < TL_KT; ++ks) {
+                const int kb = st * TL_KT + ks;
+                if (kb < KB && nb0 + a < NB)
+                    wreg[a][ks].u = Wp[((size_t)(nb0 + a) * KB + kb) * 64 + lane];
+                else
+                    wreg[a][ks].u = uint4{0, 0, 0, 0};
+            }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int idx = threadIdx.x + 256 * i;        // 256 rows x 8 pieces of 8 columns
+            const int row = idx >> 3, piece = idx & 7;
+            const int k = st * (TL_KT * 32) + piece * 8;
+            if (m0 + row < M && k < K)
+                xreg[i] = *reinterpret_cast<const uint4*>(X + (size_t)(m0 + row) * ldx + k);
+            else
+                xreg[i] = uint4{0, 0, 0, 0};
+        }
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int idx = threadIdx.x + 256 * i;
+            *reinterpret_cast<uint4*>(&xs[buf][idx >> 3][(idx & 7) * 8]) = xreg[i];
+        }
+    };
+
+    load_stage(0);
+    store_x(0);
+    __syncthreads();
+    for (int st = 0; st < n_stage; ++st) {
+        const int buf = st & 1;
+        frag16 wcur[TL_WN][TL_KT];
+#pragma unroll
+        for (int a = 0; a < TL_WN; ++a)
+#pragma unroll
+            for (int ks = 0; ks < TL_KT; ++ks) wcur[a][ks] = wreg[a][ks];
+        if (st + 1 < n_stage) load_stage(st + 1);
+#pragma unroll
+        for (int ks = 0; ks < TL_KT; ++ks)
+#pragma unroll
+            for (int b = 0; b < TL_WM; ++b) {
+                frag16 xb;
+                xb.u = *reinterpret_cast<const uint4*>(&xs[buf][(wm * TL_WM + b) * 16 + j][ks * 32 + g * 8]);
+#pragma unroll
+                for (int a = 0; a < TL_WN; ++a) acc[a][b] = mfma_16x16x32(wcur[a][ks], xb, acc[a][b]);
+            }
+        if (st + 1 < n_stage) store_x(buf ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int a = 0; a < TL_WN; ++a) {
+        if (nb0 + a >= NB) continue;
+#pragma unroll
+        for (int b = 0; b < TL_WM; ++b) {
+            const int m = m0 + (wm * TL_WM + b) * 16 + j;
+            if (m >= M) continue;
+            const f32x4_t s = acc[a][b];
+            if (EPI == 0) {
+                const int n = (nb0 + a) * 16 + g * 4;
+                TC* dst = Y + (size_t)m * ldy + n;
+                if (n + 3 < N) {
+                    st(dst, s[0]);
+                    st(dst + 1, s[1]);
+                    st(dst + 2, s[2]);
+                    st(dst + 3, s[3]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (n + e < N) st(dst + e, s[e]);
+                }
+            } else {
+                const int n = (nb0 + a) * 8 + g * 2;
+                if (n < N) st(Y + (size_t)m * ldy + n, gelu_tanh_f(s[0]) * s[2]);
+                if (n + 1 < N) st(Y + (size_t)m * ldy + n + 1, gelu_tanh_f(s[1]) * s[3]);
+            }
+        }
+    }
+}
+
+extern "C" int agave_gemm_tiled(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,
+                                int K, int epilogue, hipStream_t stream) {
+    AGAVE_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
+    AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
+                "gemm_tiled: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
+    AGAVE_CHECK(ldx >= K && ldy >= N, "gemm_tiled: a row stride is too small");
+    AGAVE_CHECK(epilogue == 0 || epilogue == 1, "gemm_tiled: unknown epilogue %d", epilogue);
+    if (M == 0) return 0;
+    const int KB = (K + 31) / 32;
+    const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
+    dim3 grid((NB + 7) / 8, (M + 255) / 256);
+    AGAVE_CHECK(grid.y <= 65535, "gemm_tiled: M=%d exceeds the grid limit", M);
+    if (epilogue == 0) {
+        if (dt_y == AGAVE_BF16)
+            gemm_tiled_kernel<0, bf16><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (bf16*)Y, ldy, M, N, K, KB, NB);
+        else if (dt_y == AGAVE_F32)
+            gemm_tiled_kernel<0, float><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (float*)Y, ldy, M, N, K, KB, NB);
+        else
+            AGAVE_CHECK(false, "gemm_tiled: unknown output dtype %d", dt_y);
+    } else {
+        AGAVE_CHECK(dt_y == AGAVE_BF16, "gemm_tiled: the GeGLU epilogue writes bfloat16");
+        gemm_tiled_kernel<1, bf16><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (bf16*)Y, ldy, M, N, K, KB, NB);
+    }
+    AGAVE_LAUNCH_CHECK("gemm_tiled");
+    return 0;
+}

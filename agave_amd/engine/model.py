@@ -40,7 +40,7 @@ class Model:
             table = table.to(torch.float32)
         if table.dtype not in (torch.float32, torch.bfloat16):
             raise TypeError(f"embedding table has unsupported element type {table.dtype}")
-        self.embed_table = table.to(env.device).contiguous()
+        self.embed_table: Optional[torch.Tensor] = table.to(env.device).contiguous()
         self.blocks = [lookup("block", layer.kind)(layer, weights, env) for layer in spec.layers]
         self.final_norm = (lookup("norm", spec.final_norm.kind)(spec.final_norm, weights, env)
                            if spec.final_norm is not None else None)
@@ -48,6 +48,8 @@ class Model:
             self.head = Linear([weights.get(spec.head_weight)], env, "lm_head")
         else:
             self.head = Linear([self.embed_table], env, "lm_head")      # tied: the same device tensor
+            if self.head.packed is not None:
+                self.embed_table = None                                  # rows are gathered from the packed copy
         for entry in spec.order:
             if not (0 <= entry.layer < len(self.blocks)):
                 raise ValueError(f"run order names layer {entry.layer}, the model has {len(self.blocks)}")
@@ -91,7 +93,11 @@ class Model:
         ws = self.env.workspace
         n = step.n_tokens
         h = ws.get("residual", n, self.spec.hidden, torch.float32)
-        kernels.embed_scale(step.tokens, self.embed_table, self.spec.embed_scale, h)
+        if self.embed_table is not None:
+            kernels.embed_scale(step.tokens, self.embed_table, self.spec.embed_scale, h)
+        else:
+            from ..ops import gemm_mfma
+            gemm_mfma.embed_scale_packed(step.tokens, self.head.packed, self.spec.embed_scale, h, self.spec.vocab_size)
         pending = None
         for entry in self.spec.order:
             pending = self.blocks[entry.layer].forward(h, pending, step, entry.memory, entry.writes)

@@ -12,8 +12,10 @@ def linear(x: torch.Tensor, lin, out: torch.Tensor) -> None:
         raise ValueError(f"{lin.name}: input is {tuple(x.shape)}, weight takes {lin.in_features} columns")
     if out.shape != (x.shape[0], lin.out_features):
         raise ValueError(f"{lin.name}: output is {tuple(out.shape)}, needs {(x.shape[0], lin.out_features)}")
-    if x.dtype == torch.bfloat16 and lin.weight.dtype == torch.bfloat16:
+    if getattr(lin, "packed", None) is not None:
         from . import gemm_mfma
         if gemm_mfma.try_linear(x, lin, out):
             return
+        raise ValueError(f"{lin.name}: the matrix-core product needs a 16-byte aligned bfloat16 input whose row "
+                         f"stride is a multiple of 8, got {tuple(x.shape)} {x.dtype} strides {x.stride()}")
     kernels.gemm_plain(x, lin.weight, out)

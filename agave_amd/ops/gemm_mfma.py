@@ -12,6 +12,7 @@ kernels.register_signatures("gemm_mfma", {
     "agave_pack_w16": [_P, _L, _P, _I, _I, _I, _I, _P],
     "agave_embed_scale_packed": [_P, _P, _F, _P, _I, _I, _I, _P],
     "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P],
+    "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P],
 })
 
 SKINNY_MAX_M = 64
@@ -37,26 +38,52 @@ def _x_ok(x: torch.Tensor) -> bool:
             and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0)
 
 
+def product(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, epilogue: int = 0) -> None:
+    """out[M, n_out] = x[M, K] @ W^T (epilogue 0) or gelu_tanh(gate) * up (epilogue 1), any M: the
+    skinny kernel up to 64 rows, the tiled one above."""
+    if x.shape[0] <= SKINNY_MAX_M:
+        skinny(x, packed, out, n_out, epilogue)
+    else:
+        _launch("agave_gemm_tiled", x, packed, out, n_out, epilogue)
+
+
 def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, epilogue: int = 0) -> None:
     """out[M, n_out] = x[M, K] @ W^T (epilogue 0) or gelu_tanh(gate) * up (epilogue 1) for M <= 64."""
+    _launch("agave_gemm_skinny", x, packed, out, n_out, epilogue)
+
+
+def _launch(fn: str, x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, epilogue: int) -> None:
     if not (x.is_cuda and packed.is_cuda and out.is_cuda):
         raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
     m, k = x.shape
     if not _x_ok(x):
-        raise ValueError("skinny product: x must be bfloat16, 16-byte aligned, K and row stride multiples of 8")
+        raise ValueError("packed product: x must be bfloat16, 16-byte aligned, K and row stride multiples of 8")
     if out.dim() != 2 or out.shape != (m, n_out) or out.stride(1) != 1:
-        raise ValueError(f"skinny product: out must be [{m}, {n_out}] with contiguous rows")
+        raise ValueError(f"packed product: out must be [{m}, {n_out}] with contiguous rows")
     nb = (n_out + 7) // 8 if epilogue else (n_out + 15) // 16
     if packed.numel() != nb * ((k + 31) // 32) * 512:
-        raise ValueError("skinny product: the packed weight does not fit these sizes")
-    library.call(kernels.lib("gemm_mfma"), "agave_gemm_skinny", x.data_ptr(), x.stride(0), packed.data_ptr(),
+        raise ValueError("packed product: the packed weight does not fit these sizes")
+    library.call(kernels.lib("gemm_mfma"), fn, x.data_ptr(), x.stride(0), packed.data_ptr(),
                  kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue, kernels.stream())
 
 
 def try_linear(x: torch.Tensor, lin, out: torch.Tensor) -> bool:
     """Run the product on the matrix cores if a kernel takes these sizes; False otherwise."""
     packed = getattr(lin, "packed", None)
-    if packed is None or x.shape[0] > SKINNY_MAX_M or not _x_ok(x):
+    if packed is None or not _x_ok(x):
         return False
-    skinny(x, packed, out, lin.out_features, 0)
+    product(x, packed, out, lin.out_features, 0)
     return True
+
+
+def embed_scale_packed(tokens: torch.Tensor, packed: torch.Tensor, scale: float, out: torch.Tensor, vocab: int) -> None:
+    """out[t] = table[tokens[t]] * scale, the table being a packed [vocab, hidden] weight."""
+    if not (tokens.is_cuda and packed.is_cuda and out.is_cuda):
+        raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
+    n, e = out.shape
+    if tokens.dtype != torch.int32 or tokens.numel() != n or out.dtype != torch.float32 or not out.is_contiguous():
+        raise TypeError("embed_scale_packed: int32 tokens and a contiguous float32 [tokens, hidden] output")
+    if packed.numel() != ((vocab + 15) // 16) * ((e + 31) // 32) * 512:
+        raise ValueError("embed_scale_packed: the packed table does not fit these sizes")
+    library.call(kernels.lib("gemm_mfma"), "agave_embed_scale_packed", tokens.data_ptr(), packed.data_ptr(), scale,
+                 out.data_ptr(), n, e, vocab, kernels.stream())

@@ -32,7 +32,6 @@ class Attention:
         self.kvd = spec.n_kv_heads * spec.head_dim
         # q, k and v in one product: rows of the three matrices stacked
         self.qkv = Linear([weights.get(spec.q_proj), weights.get(spec.k_proj), weights.get(spec.v_proj)], env, "qkv")
-        self.q_only: Optional[Linear] = None       # built on demand for runs that only read a cache
         self.o = Linear([weights.get(spec.o_proj)], env, "attn_o")
         self.q_norm = lookup("norm", spec.q_norm.kind)(spec.q_norm, weights, env) if spec.q_norm else None
         self.k_norm = lookup("norm", spec.k_norm.kind)(spec.k_norm, weights, env) if spec.k_norm else None
@@ -61,13 +60,10 @@ class Attention:
         table, base = step.tables[step.cache.group_of_memory[memory]]
         inv_freq, pos_scale = (None, 1.0)
         fused = getattr(self.position, "fused_rotation", None)
-        if writes:
-            qkv = self.qkv.forward(x, tag="qkv")
-            q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
-        else:
-            if self.q_only is None:
-                self.q_only = Linear([self.qkv.weight[:self.qd]], self.env, "q_only")
-            q, k, v = self.q_only.forward(x, tag="q_only"), None, None
+        qkv = self.qkv.forward(x, tag="qkv")
+        q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
+        if not writes:
+            k = v = None            # a run that reads another run's cache appends nothing
         if fused is not None:
             inv_freq, pos_scale = fused()
         else:

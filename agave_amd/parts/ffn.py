@@ -25,13 +25,10 @@ class GatedFfn:
             raise ValueError(f"gated feed-forward: unsupported activation {spec.activation!r}; known: {_ACTIVATIONS}")
         self.spec = spec
         self.env = env
-        self.gate_up = Linear([weights.get(spec.gate_proj), weights.get(spec.up_proj)], env, "gate_up")
+        # [gate; up] stacked; on the matrix cores their rows are interleaved so that the product ends in GeGLU
+        self.gate_up = Linear([weights.get(spec.gate_proj), weights.get(spec.up_proj)], env, "gate_up",
+                              interleave_ff=spec.intermediate)
         self.down = Linear([weights.get(spec.down_proj)], env, "ffn_down")
-        self.gate_up_fused = None   # [gate; up] with interleaved rows, for the product that ends in GeGLU
-        if self.gate_up.packed is not None:
-            from ..ops import gemm_mfma
-            self.gate_up_fused = gemm_mfma.pack_weight(self.gate_up.weight, interleave_ff=spec.intermediate)
-            self.gate_up.packed = None
 
     @staticmethod
     def tensor_needs(spec: GatedFfnSpec) -> List[TensorNeed]:
@@ -43,10 +40,7 @@ class GatedFfn:
         ff = self.spec.intermediate
         n = x.shape[0]
         act = self.env.workspace.get("ffn_act", n, ff, x.dtype)
-        if self.gate_up_fused is not None and n <= 64 and x.dtype == torch.bfloat16:
-            from ..ops import gemm_mfma
-            gemm_mfma.skinny(x, self.gate_up_fused, act, ff, epilogue=1)
-        else:
+        if not self.gate_up.forward_geglu(x, act):
             gu = self.gate_up.forward(x, tag="gate_up")
             kernels.geglu(gu[:, :ff], gu[:, ff:], act)
         return self.down.forward(act, tag="ffn_down")

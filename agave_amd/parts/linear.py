@@ -17,8 +17,11 @@ from .base import BuildEnv
 
 
 class Linear:
-    def __init__(self, weights: Sequence[torch.Tensor], env: BuildEnv, name: str = "linear"):
-        """``weights``: one or more [out_i, in] matrices that are stacked along ``out``."""
+    def __init__(self, weights: Sequence[torch.Tensor], env: BuildEnv, name: str = "linear", pack: bool = True,
+                 interleave_ff: int = 0):
+        """``weights``: one or more [out_i, in] matrices that are stacked along ``out``.
+        ``interleave_ff``: the stack is [gate; up] of that many rows each; if the weight is packed
+        its rows are interleaved for the product that ends in GeGLU (see ``forward_geglu``)."""
         ws = []
         for w in weights:
             if w.dim() != 2:
@@ -34,9 +37,11 @@ class Linear:
         self.env = env
         self.name = name
         self.packed = None          # the weight in the matrix cores' tile layout (bfloat16 engines)
-        if env.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16:
+        if pack and env.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.in_features % 8 == 0:
             from ..ops import gemm_mfma
-            self.packed = gemm_mfma.pack_weight(self.weight)
+            self.packed = gemm_mfma.pack_weight(self.weight, interleave_ff=interleave_ff)
+            self.weight = None      # only the packed copy is kept
+        self.interleave_ff = interleave_ff if self.packed is not None else 0
 
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, tag: Optional[str] = None) -> torch.Tensor:
@@ -44,5 +49,15 @@ class Linear:
         if out is None:
             out = self.env.workspace.get(tag or self.name, n, self.out_features, out_dtype or x.dtype)
         from ..ops import gemm
+        if self.interleave_ff:
+            raise RuntimeError(f"{self.name}: a weight packed for GeGLU only serves forward_geglu")
         gemm.linear(x, self, out)
         return out
+
+    def forward_geglu(self, x: torch.Tensor, out: torch.Tensor) -> bool:
+        """out = gelu_tanh(gate x) * (up x) in one kernel, if the weight was packed for it."""
+        if not self.interleave_ff:
+            return False
+        from ..ops import gemm_mfma
+        gemm_mfma.product(x, self.packed, out, self.interleave_ff, epilogue=1)
+        return True

@@ -485,3 +485,40 @@ def test_attn_mfma_far_key_and_window_edge(K, decode):
     assert not torch.allclose(got_w[-1, 0], vs[0][3, 0].double(), atol=1e-1)
     got_e, _, _ = _mfma_attn_case(K, 2, 1, 32, [700], 697, 0.5, decode, seed=1, boost=3)      # just inside
     assert torch.allclose(got_e[-1, 0], vs[0][3, 0].double(), atol=2e-2)
+
+
+@pytest.mark.parametrize("m,n,k", [(65, 53, 72), (300, 256, 2560), (257, 1000, 96), (2048, 300, 136), (130, 4100, 64)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_gemm_tiled(G, m, n, k, out_dtype):
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    packed = G.pack_weight(w.to(DEV))
+    out = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+    G.product(x.to(DEV), packed, out, n)
+    ref = x.double() @ w.double().T
+    scale = float(ref.abs().max())
+    tol = 2e-5 * scale * math.sqrt(k / 64) if out_dtype == torch.float32 else 6e-3 * scale
+    assert float((out.cpu().double() - ref).abs().max()) <= tol
+
+
+@pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40)])
+def test_gemm_tiled_geglu(G, m, ff, k):
+    g = torch.Generator().manual_seed(ff + m)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(2 * ff, k, generator=g) * 0.2).bfloat16()
+    packed = G.pack_weight(w.to(DEV), interleave_ff=ff)
+    out = torch.full((m, ff), float("nan"), dtype=torch.bfloat16, device=DEV)
+    G.product(x.to(DEV), packed, out, ff, epilogue=1)
+    gu = x.double() @ w.double().T
+    ref = P.gelu_tanh(gu[:, :ff]) * gu[:, ff:]
+    assert float((out.cpu().double() - ref).abs().max()) <= 8e-3 * float(ref.abs().max())
+
+
+def test_embedding_from_a_packed_table(G):
+    table = (torch.randn(300, 72) * 0.05).bfloat16()
+    packed = G.pack_weight(table.to(DEV))
+    toks = [0, 299, 17, 17, 123, 16, 15]
+    out = torch.empty(len(toks), 72, dtype=torch.float32, device=DEV)
+    G.embed_scale_packed(_i32(toks), packed, math.sqrt(72.0), out, 300)
+    assert torch.allclose(out.cpu().double(), P.embed(toks, table.double(), 72), atol=1e-6, rtol=1e-6)
