@@ -86,7 +86,9 @@ struct WaveAttn {
             }
     }
 
-    __device__ __forceinline__ void page(const uint4* __restrict__ kp, const uint4* __restrict__ vp, int page_idx,
+    // PT: pointer (to u32x4_t) to the page's tiles, in global memory or in LDS
+    template <typename PT>
+    __device__ __forceinline__ void page(PT kp, PT vp, int page_idx,
                                          int qt, int hd, float scale, const int* pos, const int* lo, int lane) {
         const int g = lane >> 4;
         const int hdt = hd >> 4, ks_n = (hd + 31) >> 5;
@@ -102,7 +104,7 @@ struct WaveAttn {
             for (int ks = 0; ks < KS; ++ks) {
                 if (ks < ks_n) {
                     frag16 a;
-                    a.u = kp[(kt * ks_n + ks) * 64 + lane];
+                    a.r = kp[(kt * ks_n + ks) * 64 + lane];
 #pragma unroll
                     for (int t = 0; t < QTM; ++t)
                         if (t < qt) st[t][kt] = mfma_16x16x32(a, qf[t][ks], st[t][kt]);
@@ -162,7 +164,7 @@ struct WaveAttn {
 #pragma unroll
                 for (int s = 0; s < 2; ++s) {
                     frag16 b;
-                    b.u = vp[(d * 2 + s) * 64 + lane];
+                    b.r = vp[(d * 2 + s) * 64 + lane];
 #pragma unroll
                     for (int t = 0; t < QTM; ++t)
                         if (t < qt) o[t][d] = mfma_16x16x32(pf[t][s], b, o[t][d]);
@@ -231,8 +233,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(AttnArgs a) {
             pg = page_of(a, b, pi);
         }
         if (pg < 0) continue;
-        w.page(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride, a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride, pi, 1,
-               hd, a.scale, pos, los, lane);
+        w.page((const u32x4_t*)(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride),
+               (const u32x4_t*)(a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride), pi, 1, hd, a.scale, pos, los, lane);
     }
     w.finish_sums(1);
     // every wave leaves its (unnormalised) rows, maxima and sums in LDS
@@ -321,21 +323,31 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
     }
 }
 
-// ------------------------------------------------------------------ prefill: 16 positions x QT heads per wave
-// grid (position tile, kv head * head chunks, sequence); 4 waves per workgroup take 4
-// consecutive position tiles.  Slot j of tile t is position first + j of head chunk*QT + t.
+// ------------------------------------------------------------------ prefill: 64 positions x QT heads per workgroup
+// grid (block of positions, kv head * head chunks, sequence).  The four waves are hw heads
+// wide and 4/hw tiles of 16 positions deep; a wave takes QT heads of its tile (slot j of tile t
+// is position first + j of head chunk*hw*QT + (wave % hw)*QT + t).  All share the pages: a page's K and V tiles come into LDS once per workgroup, straight from global memory
+// (no registers in between), the next page while the current one is being used.
+typedef __attribute__((address_space(3))) u32x4_t lds_u32x4;
+
 template <int HDT, int QT>
-__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int qt_heads) {
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int qt_heads, int hw) {
+    extern __shared__ __attribute__((aligned(16))) uint4 page_lds[];      // [2][K tiles | V tiles][64]
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
     const int G = a.nh / a.nkv;
-    const int chunks = (G + qt_heads - 1) / qt_heads;
+    const int wg_heads = qt_heads * hw;                          // heads a workgroup covers
+    const int chunks = (G + wg_heads - 1) / wg_heads;
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
     const int b = blockIdx.z;
     const int t0 = a.cu[b], n_new = a.cu[b + 1] - t0;
-    const int tile0 = (blockIdx.x * 4 + wave) * 16;              // first step-token of this wave's tile
-    if (tile0 >= n_new) return;
-    const int qt = (G - chunk * qt_heads < qt_heads) ? G - chunk * qt_heads : qt_heads;
-    const int hd = a.hd, hdt = hd >> 4;
+    const int blk_len = (4 / hw) * 16;                           // positions a workgroup covers
+    const int blk0 = blockIdx.x * blk_len;
+    if (blk0 >= n_new) return;                                   // the whole workgroup leaves
+    const int tile0 = blk0 + (wave / hw) * 16;                   // first step-token of this wave's tile
+    const int head0 = chunk * wg_heads + (wave % hw) * qt_heads; // first head (within the group) of this wave
+    const int qt = (G - head0 < qt_heads) ? (G - head0 > 0 ? G - head0 : 0) : qt_heads;
+    const bool wave_on = tile0 < n_new && qt > 0;
+    const int hd = a.hd, hdt = hd >> 4, ks_n = (hd + 31) >> 5;
     const bool col_ok = tile0 + j < n_new;
     const int tok = t0 + (col_ok ? tile0 + j : n_new - 1);       // padding columns repeat the last token
     const int p = a.tok_pos[tok];
@@ -347,26 +359,56 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int 
     int pos[QT], los[QT];
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
-        const int head = kvh * G + chunk * qt_heads + t;
-        q_row[t] = (t < qt) ? a.q + (size_t)tok * a.ldq + (size_t)head * hd : nullptr;
+        const int head = kvh * G + head0 + t;
+        q_row[t] = (t < qt && wave_on) ? a.q + (size_t)tok * a.ldq + (size_t)head * hd : nullptr;
         pos[t] = p;
         los[t] = lo;
     }
     w.load_q(q_row, qt, hd, lane);
-    // pages from the first column's lower bound to the last column's position
-    const int lo_min = __shfl(lo, 0, 64), p_max = __shfl(p, 15, 64);
-    const size_t k_stride = (size_t)4 * ((hd + 31) >> 5) * 64, v_stride = (size_t)hdt * 2 * 64;
-    for (int pi = lo_min / AGAVE_PAGE; pi <= p_max / AGAVE_PAGE; ++pi) {
+    // this wave needs the pages from its first column's lower bound to its last column's position
+    const int my_first = __shfl(lo, 0, 64) / AGAVE_PAGE, my_last = __shfl(p, 15, 64) / AGAVE_PAGE;
+    // the workgroup: positions are consecutive within the step
+    const int p_blk0 = a.tok_pos[t0 + blk0];
+    const int blk_n = (n_new - blk0 < blk_len) ? n_new - blk0 : blk_len;
+    const int lo_blk = a.window > 0 ? (p_blk0 - a.window + 1 > 0 ? p_blk0 - a.window + 1 : 0) : 0;
+    const int page_first = lo_blk / AGAVE_PAGE, page_last = (p_blk0 + blk_n - 1) / AGAVE_PAGE;
+
+    const int n_k = 4 * ks_n, n_v = hdt * 2;                     // tiles (of 64 uint4) per page
+    const size_t k_stride = (size_t)n_k * 64, v_stride = (size_t)n_v * 64;
+    const int buf_tiles = n_k + n_v;
+    auto fetch = [&](int pi, int buf) {
         const long pg = page_of(a, b, pi);
-        if (pg < 0) continue;
-        w.page(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride, a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride, pi, qt,
-               hd, a.scale, pos, los, lane);
+        if (pg < 0) return;
+        const uint4* ksrc = a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride;
+        const uint4* vsrc = a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride;
+        for (int ti = wave; ti < buf_tiles; ti += 4) {
+            const uint4* src = (ti < n_k) ? ksrc + (size_t)ti * 64 : vsrc + (size_t)(ti - n_k) * 64;
+            uint4* dst = page_lds + ((size_t)buf * buf_tiles + ti) * 64;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + lane),
+                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+        }
+    };
+
+    fetch(page_first, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for (int pi = page_first; pi <= page_last; ++pi) {
+        const int buf = (pi - page_first) & 1;
+        if (pi < page_last) fetch(pi + 1, buf ^ 1);
+        if (wave_on && pi >= my_first && pi <= my_last && page_of(a, b, pi) >= 0) {
+            const lds_u32x4* kl = (const lds_u32x4*)(page_lds + (size_t)buf * buf_tiles * 64);
+            const lds_u32x4* vl = kl + (size_t)n_k * 64;
+            w.page(kl, vl, pi, qt, hd, a.scale, pos, los, lane);
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
     }
+    if (!wave_on) return;
     w.finish_sums(qt);
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
         if (t >= qt) continue;
-        const int head = kvh * G + chunk * qt_heads + t;
+        const int head = kvh * G + head0 + t;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int row = 4 * g + e;                            // slot (position) this lane's values belong to
@@ -442,14 +484,29 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
     AGAVE_CHECK(n_seqs <= 65535, "attn_prefill_mfma: %d sequences exceed the grid limit", n_seqs);
     if (N == 0) return 0;
     const int G = nh / nkv;
-    const int qt_cap = hd > 128 ? 1 : (hd > 64 ? 2 : QT_MAX);       // what fits the register file
+    const int qt_cap = hd > 128 ? 1 : (hd > 64 ? 2 : QT_MAX);       // heads per wave: what fits the register file
     const int qt_heads = G < qt_cap ? G : qt_cap;
-    const int chunks = (G + qt_heads - 1) / qt_heads;
+    // large heads: the other heads of the group go to other waves of the workgroup
+    int hw = 1;
+    if (hd > 128) hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
+    const int wg_heads = qt_heads * hw, blk_len = (4 / hw) * 16;
+    const int chunks = (G + wg_heads - 1) / wg_heads;
     AGAVE_CHECK(nkv * chunks <= 65535, "attn_prefill_mfma: too many head chunks");
-    dim3 grid((max_new + 63) / 64, nkv * chunks, n_seqs);
-    if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, 0, stream>>>(a, qt_heads);
-    else if (hd <= 128) attn_prefill_mfma_kernel<8, 2><<<grid, 256, 0, stream>>>(a, qt_heads);
-    else attn_prefill_mfma_kernel<16, 1><<<grid, 256, 0, stream>>>(a, qt_heads);
+    dim3 grid((max_new + blk_len - 1) / blk_len, nkv * chunks, n_seqs);
+    // two pages (K and V tiles) in LDS
+    const size_t lds = (size_t)2 * (4 * ((hd + 31) / 32) + (hd / 16) * 2) * 64 * sizeof(uint4);
+    static bool raised = false;
+    if (!raised) {
+        const int cap = 144 * 1024;
+        hipError_t e1 = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<4, QT_MAX>, hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+        hipError_t e2 = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<8, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+        hipError_t e3 = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<16, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, cap);
+        AGAVE_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "attn_prefill_mfma: cannot raise the LDS allowance");
+        raised = true;
+    }
+    if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
+    else if (hd <= 128) attn_prefill_mfma_kernel<8, 2><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
+    else attn_prefill_mfma_kernel<16, 1><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     AGAVE_LAUNCH_CHECK("attn_prefill_mfma");
     return 0;
 }

@@ -16,9 +16,11 @@
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 union frag16 {            // 16 bytes: one lane's share of an MFMA operand
     uint4 u;
+    u32x4_t r;
     bf16x8_t v;
     bf16 h[8];
 };
