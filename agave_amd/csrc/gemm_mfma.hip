@@ -14,6 +14,16 @@
 #include "common_impl.h"
 #include "mfma.h"
 
+// four consecutive outputs at once (the address is a multiple of four elements)
+template <typename T> __device__ __forceinline__ void store4(T* p, float4 v);
+template <> __device__ __forceinline__ void store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)f32_to_bf16(v.x).x | ((uint32_t)f32_to_bf16(v.y).x << 16);
+    u.y = (uint32_t)f32_to_bf16(v.z).x | ((uint32_t)f32_to_bf16(v.w).x << 16);
+    *reinterpret_cast<uint2*>(p) = u;
+}
+
 // ------------------------------------------------------------------ packing
 // mode 0: packed row p is source row p.
 // mode 1: the source is [gate (ff rows); up (ff rows)]; within a block of 16 packed rows, rows
@@ -282,121 +292,183 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
 
 
 // ------------------------------------------------------------------ tiled product (prefill)
-// A workgroup of four waves (2 x 2) computes 128 weight rows x 256 tokens; a wave 64 rows x 128
-// tokens as 4 x 8 MFMA tiles, so every weight tile it loads (straight from the packed layout,
-// coalesced, no LDS) meets eight token tiles and every token tile (staged through LDS, shared
-// by the workgroup) meets four weight tiles.  Two k-steps of 32 columns per stage, the next
-// stage's loads are in flight while the current one is multiplied.
+// A workgroup of four waves (2 x 2) computes WT*64 weight rows x 256 tokens; a wave WT x 4
+// tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16).  Both operands come into LDS straight from
+// global memory (no registers in between), KT k-steps of 32 columns per stage, in a ring of
+// NS buffers: the loads of NS-1 stages ahead are in flight while a stage is multiplied.
+// Weight tiles arrive in their packed order (one kilobyte per wave load; a 32-row operand is
+// read out of two packed 16-row tiles); token rows are stored with their 16-byte pieces
+// permuted so that the rows an MFMA operand reads fall into different banks.
+//   WT 2, KT 2, NS 3:  128 x 256 tiles, 144 KB of LDS - more workgroups for small products
+//   WT 4, KT 1, NS 4:  256 x 256 tiles, 128 KB of LDS - a third less traffic from L2 per flop
 // blockIdx.x walks the weight rows, so that workgroups sharing weight rows (ids a multiple of
 // the number of row tiles apart) tend to land on the same XCD and find them in its L2.
-#define TL_KT 2                       // k-steps per stage
-#define TL_ROW (TL_KT * 32 + 8)       // bf16 per staged token row (16 bytes of padding)
-#define TL_WM 8                       // token tiles per wave
-#define TL_WN 4                       // weight-row tiles per wave
+typedef __attribute__((address_space(3))) u32x4_t tl_lds_u32x4;
 
-template <int EPI, typename TC>
+template <int WT, int KT, int NS, int EPI, typename TC>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
                                                          const uint4* __restrict__ Wp, TC* __restrict__ Y, long ldy,
                                                          int M, int N, int K, int KB, int NB) {
-    __shared__ __attribute__((aligned(16))) bf16 xs[2][256][TL_ROW];
+    constexpr int CPR = KT * 4;                       // 16-byte pieces per staged token row
+    constexpr int RP = 16 / CPR;                      // token rows per 256 bytes of LDS
+    constexpr int WTILES = 4 * WT;                    // packed 16-row weight tiles per workgroup
+    constexpr int X_BYTES = 256 * KT * 64, W_BYTES = WTILES * KT * 1024;
+    constexpr int STAGE_BYTES = X_BYTES + W_BYTES;
+    constexpr int X_LOADS = X_BYTES / 1024 / 4, W_LOADS = W_BYTES / 1024 / 4;     // per wave and stage
+    constexpr int LOADS = X_LOADS + W_LOADS;
+    static_assert(LOADS * (NS - 2) < 64, "the load counter holds 6 bits");
+    extern __shared__ __attribute__((aligned(16))) unsigned char tl_lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int j = lane & 15, g = lane >> 4;
     const int wn = wave & 1, wm = wave >> 1;
-    const int nb0 = blockIdx.x * 8 + wn * TL_WN;          // first weight-row tile of this wave
+    const int nbw = blockIdx.x * WTILES;                  // first packed weight tile of this workgroup
     const int m0 = blockIdx.y * 256;                      // first token of this workgroup
-    const int n_stage = (KB + TL_KT - 1) / TL_KT;
+    const int n_stage = (KB + KT - 1) / KT;
+    const int i32 = lane & 31, kg = lane >> 5;
 
-    f32x4_t acc[TL_WN][TL_WM];
+    f32x16_t acc[WT][4];
 #pragma unroll
-    for (int a = 0; a < TL_WN; ++a)
+    for (int a = 0; a < WT; ++a)
 #pragma unroll
-        for (int b = 0; b < TL_WM; ++b) acc[a][b] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    frag16 wreg[TL_WN][TL_KT];
-    uint4 xreg[8];
-
-    auto load_stage = [&](int st) {
+    // this lane's part of the staging
+    const bf16* xsrc[X_LOADS];
+    int xcol[X_LOADS];
 #pragma unroll
-        for (int a = 0; a < TL_WN; ++a)
+    for (int i = 0; i < X_LOADS; ++i) {
+        const int o = ((wave * X_LOADS + i) * 64 + lane);              // 16-byte slot in the stage
+        const int row = o / CPR, pos = o % CPR;                        // LDS row and position this lane's piece lands in
+        const int piece = pos ^ ((row / RP) % CPR);                    // which 8 columns of that row it holds
+        int mrow = m0 + row;
+        if (mrow >= M) mrow = M - 1;                                   // rows past the end repeat the last one (never stored)
+        xcol[i] = piece * 8;
+        xsrc[i] = X + (size_t)mrow * ldx + piece * 8;
+    }
+    auto fetch = [&](int st) {
+        unsigned char* buf = tl_lds + (size_t)(st % NS) * STAGE_BYTES;
 #pragma unroll
-            for (int ks = 0; ks < TL_KT; ++ks) {
-                const int kb = st * TL_KT + ks;
-                if (kb < KB && nb0 + a < NB)
-                    wreg[a][ks].u = Wp[((size_t)(nb0 + a) * KB + kb) * 64 + lane];
-                else
-                    wreg[a][ks].u = uint4{0, 0, 0, 0};
-            }
+        for (int i = 0; i < X_LOADS; ++i) {
+            int k = st * (KT * 32);
+            if (k + xcol[i] >= K) k = -xcol[i];                        // past the last column: any valid address (weights are zero there)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xsrc[i] + k),
+                                             (__attribute__((address_space(3))) void*)(buf + (wave * X_LOADS + i) * 1024), 16, 0, 0);
+        }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int idx = threadIdx.x + 256 * i;        // 256 rows x 8 pieces of 8 columns
-            const int row = idx >> 3, piece = idx & 7;
-            const int k = st * (TL_KT * 32) + piece * 8;
-            if (m0 + row < M && k < K)
-                xreg[i] = *reinterpret_cast<const uint4*>(X + (size_t)(m0 + row) * ldx + k);
-            else
-                xreg[i] = uint4{0, 0, 0, 0};
+        for (int i = 0; i < W_LOADS; ++i) {
+            const int tt = wave * W_LOADS + i;                         // tile: row tile tt / KT, k-step tt % KT
+            int nb = nbw + tt / KT, kb = st * KT + tt % KT;
+            if (nb >= NB) nb = NB - 1;                                 // rows past the end: never stored
+            if (kb >= KB) kb = KB - 1;                                 // k-steps past the end: never multiplied
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Wp + ((size_t)nb * KB + kb) * 64 + lane),
+                                             (__attribute__((address_space(3))) void*)(buf + X_BYTES + tt * 1024), 16, 0, 0);
         }
     };
-    auto store_x = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int idx = threadIdx.x + 256 * i;
-            *reinterpret_cast<uint4*>(&xs[buf][idx >> 3][(idx & 7) * 8]) = xreg[i];
-        }
-    };
 
-    load_stage(0);
-    store_x(0);
-    __syncthreads();
+#pragma unroll
+    for (int s0 = 0; s0 < NS - 1; ++s0)
+        if (s0 < n_stage) fetch(s0);
     for (int st = 0; st < n_stage; ++st) {
-        const int buf = st & 1;
-        frag16 wcur[TL_WN][TL_KT];
+        // stage st has landed once at most the loads of the NS-2 stages after it are outstanding
+        const int ahead = (n_stage - 1 - st < NS - 2) ? n_stage - 1 - st : NS - 2;
+        if (ahead >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * LOADS) & 15) | (((2 * LOADS) >> 4) << 14));
+        else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS & 15) | ((LOADS >> 4) << 14));
+        else __builtin_amdgcn_s_waitcnt(0x0F70);
+        // a bare barrier: __syncthreads() would also wait for the loads still wanted in flight
+        __builtin_amdgcn_s_barrier();
+        if (st + NS - 1 < n_stage) fetch(st + NS - 1);
+        const unsigned char* buf = tl_lds + (size_t)(st % NS) * STAGE_BYTES;
 #pragma unroll
-        for (int a = 0; a < TL_WN; ++a)
+        for (int k16 = 0; k16 < KT * 2; ++k16) {
+            const int ks = k16 >> 1, h = k16 & 1;                      // k-step of 32 columns and its half
+            if (st * KT + ks >= KB) break;
+            // a 32-row weight operand is made of two packed 16-row tiles: rows 0..15 from the
+            // first, 16..31 from the second; the lane holding (row, columns 8*(2h+kg)..) there
+            frag16 wf[WT];
 #pragma unroll
-            for (int ks = 0; ks < TL_KT; ++ks) wcur[a][ks] = wreg[a][ks];
-        if (st + 1 < n_stage) load_stage(st + 1);
-#pragma unroll
-        for (int ks = 0; ks < TL_KT; ++ks)
-#pragma unroll
-            for (int b = 0; b < TL_WM; ++b) {
-                frag16 xb;
-                xb.u = *reinterpret_cast<const uint4*>(&xs[buf][(wm * TL_WM + b) * 16 + j][ks * 32 + g * 8]);
-#pragma unroll
-                for (int a = 0; a < TL_WN; ++a) acc[a][b] = mfma_16x16x32(wcur[a][ks], xb, acc[a][b]);
+            for (int a = 0; a < WT; ++a) {
+                const int nt = wn * (2 * WT) + 2 * a + (i32 >> 4);
+                wf[a].r = *(const tl_lds_u32x4*)(buf + X_BYTES + (nt * KT + ks) * 1024 + ((i32 & 15) + 16 * (2 * h + kg)) * 16);
             }
-        if (st + 1 < n_stage) store_x(buf ^ 1);
-        __syncthreads();
-    }
-
 #pragma unroll
-    for (int a = 0; a < TL_WN; ++a) {
-        if (nb0 + a >= NB) continue;
+            for (int b = 0; b < 4; ++b) {
+                const int row = (wm * 4 + b) * 32 + i32;
+                frag16 xb;
+                xb.r = *(const tl_lds_u32x4*)(buf + row * (CPR * 16) + (((k16 * 2 + kg) ^ ((row / RP) % CPR)) * 16));
 #pragma unroll
-        for (int b = 0; b < TL_WM; ++b) {
-            const int m = m0 + (wm * TL_WM + b) * 16 + j;
-            if (m >= M) continue;
-            const f32x4_t s = acc[a][b];
-            if (EPI == 0) {
-                const int n = (nb0 + a) * 16 + g * 4;
-                TC* dst = Y + (size_t)m * ldy + n;
-                if (n + 3 < N) {
-                    st(dst, s[0]);
-                    st(dst + 1, s[1]);
-                    st(dst + 2, s[2]);
-                    st(dst + 3, s[3]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (n + e < N) st(dst + e, s[e]);
-                }
-            } else {
-                const int n = (nb0 + a) * 8 + g * 2;
-                if (n < N) st(Y + (size_t)m * ldy + n, gelu_tanh_f(s[0]) * s[2]);
-                if (n + 1 < N) st(Y + (size_t)m * ldy + n + 1, gelu_tanh_f(s[1]) * s[3]);
+                for (int a = 0; a < WT; ++a) acc[a][b] = mfma_32x32x16(wf[a], xb, acc[a][b]);
             }
         }
     }
+
+    // D[i][j]: this lane holds token j = lane % 32 and rows i = 8*q + 4*kg + e (q, e = 0..3)
+#pragma unroll
+    for (int a = 0; a < WT; ++a) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int m = m0 + (wm * 4 + b) * 32 + i32;
+            if (m >= M) continue;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nb = nbw + wn * (2 * WT) + 2 * a + (q >> 1); // packed 16-row tile of these four rows
+                if (nb >= NB) continue;
+                const int r4 = ((2 * q + kg) & 3) * 4;                  // their first row inside that tile
+                const float s0 = acc[a][b][4 * q], s1 = acc[a][b][4 * q + 1], s2 = acc[a][b][4 * q + 2],
+                            s3 = acc[a][b][4 * q + 3];
+                if (EPI == 0) {
+                    const int n = nb * 16 + r4;
+                    TC* dst = Y + (size_t)m * ldy + n;
+                    if (n + 3 < N && (ldy & 3) == 0) {
+                        store4(dst, float4{s0, s1, s2, s3});
+                    } else {
+                        if (n < N) st(dst, s0);
+                        if (n + 1 < N) st(dst + 1, s1);
+                        if (n + 2 < N) st(dst + 2, s2);
+                        if (n + 3 < N) st(dst + 3, s3);
+                    }
+                } else {
+                    const int n = nb * 8 + (r4 >> 1);                   // N counts output columns (ff)
+                    const float v0 = gelu_tanh_f(s0) * s2, v1 = gelu_tanh_f(s1) * s3;
+                    if (n + 1 < N && (ldy & 1) == 0) {
+                        const uint32_t u = (uint32_t)f32_to_bf16(v0).x | ((uint32_t)f32_to_bf16(v1).x << 16);
+                        *reinterpret_cast<uint32_t*>(Y + (size_t)m * ldy + n) = u;
+                    } else {
+                        if (n < N) st(Y + (size_t)m * ldy + n, v0);
+                        if (n + 1 < N) st(Y + (size_t)m * ldy + n + 1, v1);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int WT, int KT, int NS, int EPI, typename TC>
+static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB, int NB,
+                        hipStream_t stream) {
+    constexpr int WTILES = 4 * WT;
+    const size_t lds = (size_t)NS * (256 * KT * 64 + WTILES * KT * 1024);
+    dim3 grid((NB + WTILES - 1) / WTILES, (M + 255) / 256);
+    AGAVE_CHECK(grid.y <= 65535, "gemm_tiled: M=%d exceeds the grid limit", M);
+    static bool raised = false;
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        AGAVE_CHECK(e == hipSuccess, "gemm_tiled: cannot raise the LDS allowance");
+        raised = true;
+    }
+    gemm_tiled_kernel<WT, KT, NS, EPI, TC><<<grid, 256, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
+                                                                      M, N, K, KB, NB);
+    return 0;
+}
+
+template <int EPI, typename TC>
+static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
+                          int NB, hipStream_t stream) {
+    // the larger tile once it still gives every compute unit two workgroups
+    const long big = (long)((NB + 15) / 16) * ((M + 255) / 256);
+    if (big >= 512) return launch_tiled<4, 1, 4, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    return launch_tiled<2, 2, 3, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
 }
 
 extern "C" int agave_gemm_tiled(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,
@@ -409,19 +481,16 @@ extern "C" int agave_gemm_tiled(const void* X, long ldx, const void* Wp, int dt_
     if (M == 0) return 0;
     const int KB = (K + 31) / 32;
     const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
-    dim3 grid((NB + 7) / 8, (M + 255) / 256);
-    AGAVE_CHECK(grid.y <= 65535, "gemm_tiled: M=%d exceeds the grid limit", M);
+    int rc;
     if (epilogue == 0) {
-        if (dt_y == AGAVE_BF16)
-            gemm_tiled_kernel<0, bf16><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (bf16*)Y, ldy, M, N, K, KB, NB);
-        else if (dt_y == AGAVE_F32)
-            gemm_tiled_kernel<0, float><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (float*)Y, ldy, M, N, K, KB, NB);
-        else
-            AGAVE_CHECK(false, "gemm_tiled: unknown output dtype %d", dt_y);
+        if (dt_y == AGAVE_BF16) rc = dispatch_tiled<0, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        else if (dt_y == AGAVE_F32) rc = dispatch_tiled<0, float>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        else AGAVE_CHECK(false, "gemm_tiled: unknown output dtype %d", dt_y);
     } else {
         AGAVE_CHECK(dt_y == AGAVE_BF16, "gemm_tiled: the GeGLU epilogue writes bfloat16");
-        gemm_tiled_kernel<1, bf16><<<grid, 256, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (bf16*)Y, ldy, M, N, K, KB, NB);
+        rc = dispatch_tiled<1, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     }
+    if (rc != 0) return rc;
     AGAVE_LAUNCH_CHECK("gemm_tiled");
     return 0;
 }

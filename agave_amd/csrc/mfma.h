@@ -28,3 +28,11 @@ union frag16 {            // 16 bytes: one lane's share of an MFMA operand
 __device__ __forceinline__ f32x4_t mfma_16x16x32(const frag16& a, const frag16& b, f32x4_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, c, 0, 0, 0);
 }
+
+// v_mfma_f32_32x32x16_bf16, D[32x32] += A[32x16] * B[16x32]:
+//   A[i][k] is held by lane i + 32*(k/8) as element k%8;  B[k][j] by lane j + 32*(k/8) as element k%8
+//   D[i][j] is held by lane j + 32*((i/4)%2) as element 4*(i/8) + i%4   (16 floats per lane)
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ f32x16_t mfma_32x32x16(const frag16& a, const frag16& b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
+}
