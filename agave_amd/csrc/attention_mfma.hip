@@ -285,6 +285,215 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(AttnArgs a) {
 }
 
 // out[t][head] = sum_s O_s * exp(m_s - m) / sum_s l_s * exp(m_s - m)
+// ------------------------------------------------------------------ decode, streamlined (head sizes 64, 128, 256)
+// The same decomposition as attn_decode_mfma_kernel, written for throughput: the unit of work
+// is half a page (32 keys: two K tiles per k-step and one V tile per 16 columns of d), the
+// loads of the next unit are issued as soon as the registers of the current one are free, the
+// output is rescaled only when a running maximum grows by more than 2^8 (otherwise the old
+// reference stays: probabilities are bounded by 2^8, which 32-bit sums and bfloat16 operands
+// hold without loss), and masks are applied only to units that touch the ends of the range.
+#define LAZY_LOG2 8.0f
+template <int HDT>
+__global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a) {
+    constexpr int KS = HDT / 2;
+    extern __shared__ float lds[];            // [4 waves][slots][hd] outputs, then [4][16][2] (max, sum)
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
+    const int G = a.nh / a.nkv;
+    const int chunks = (G + 15) / 16;
+    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int slots = (G - chunk * 16 < 16) ? G - chunk * 16 : 16;
+    const int t = blockIdx.z, split = blockIdx.x;
+    const int b = a.seq_is_token ? t : a.tok_seq[t];
+    const int col0 = split * a.pages_per_split + wave;
+    long pg0 = -1;
+    if (a.table_from_reach && col0 < a.width) pg0 = a.table[(size_t)b * a.width + col0];
+    const int p = a.tok_pos[t];
+    const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
+    const int first = lo / AGAVE_PAGE, last = p / AGAVE_PAGE;
+    const int page_lo = first + split * a.pages_per_split;
+    int page_hi = page_lo + a.pages_per_split - 1;
+    if (page_hi > last) page_hi = last;
+    constexpr int hd = HDT * 16;
+    const float scale2 = a.scale * 1.4426950408889634f;          // scores in units of log2
+
+    // queries of this chunk's heads: B operand of S^T = K Q^T
+    frag16 qf[KS];
+    {
+        const bool col_ok = j < slots;
+        const bf16* qrow = a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + j) * hd;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (col_ok) qf[ks].u = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * g);
+            else qf[ks].u = uint4{0, 0, 0, 0};
+        }
+    }
+    f32x4_t o[HDT];
+#pragma unroll
+    for (int d = 0; d < HDT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m_ref = -INFINITY, l = 0.f;
+
+    constexpr size_t k_stride = (size_t)4 * KS * 64, v_stride = (size_t)HDT * 2 * 64;   // uint4 per (page, kv head)
+    const int n_my = (page_hi >= page_lo + wave) ? (page_hi - page_lo - wave) / 4 + 1 : 0; // pages this wave takes
+    auto page_id = [&](int i) -> long {          // i-th page of this wave
+        const int pi = page_lo + wave + 4 * i;
+        long pg;
+        if (a.table_from_reach) {
+            const int col = pi - first;
+            pg = (i == 0) ? pg0 : (col < a.width ? a.table[(size_t)b * a.width + col] : -1);
+            if (pg >= a.n_pages) pg = -1;
+        } else {
+            pg = page_of(a, b, pi);
+        }
+        return pg;
+    };
+    frag16 kb[2][KS], vb[HDT];
+    const u32x4_t* kp = nullptr;
+    const u32x4_t* vp = nullptr;
+    auto load_k = [&](int half) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) kb[kt][ks].r = kp[((2 * half + kt) * KS + ks) * 64 + lane];
+    };
+    auto load_v = [&](int half) {
+#pragma unroll
+        for (int d = 0; d < HDT; ++d) vb[d].r = vp[(d * 2 + half) * 64 + lane];
+    };
+
+    // units: half pages, in order; the next unit's K and V are fetched while this one is used
+    int cur_page = 0;
+    long pg = n_my > 0 ? page_id(0) : -1;
+    bool have = n_my > 0 && pg >= 0;
+    if (have) {
+        kp = (const u32x4_t*)(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride);
+        vp = (const u32x4_t*)(a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride);
+        load_k(0);
+        load_v(0);
+    }
+    int half = 0;
+    while (have) {
+        const int pi = page_lo + wave + 4 * cur_page;
+        const int key0 = pi * AGAVE_PAGE + 32 * half;             // first key of this unit
+        // S^T for the unit's two key tiles
+        f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            st0 = mfma_16x16x32(kb[0][ks], qf[ks], st0);
+            st1 = mfma_16x16x32(kb[1][ks], qf[ks], st1);
+        }
+        // where the next unit lies, and its keys (the K registers are free now)
+        int n_half = half ^ 1, n_page = cur_page + (half == 1);
+        bool n_have = n_page < n_my;
+        const u32x4_t* nvp = vp;
+        if (n_have && half == 1) {
+            const long npg = page_id(n_page);
+            if (npg < 0) {
+                n_have = false;
+            } else {
+                kp = (const u32x4_t*)(a.k_pages + ((size_t)npg * a.nkv + kvh) * k_stride);
+                nvp = (const u32x4_t*)(a.v_pages + ((size_t)npg * a.nkv + kvh) * v_stride);
+            }
+        }
+        if (n_have) load_k(n_half);
+        // scores -> probabilities against the running reference
+        float s[8];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            s[e] = st0[e] * scale2;
+            s[4 + e] = st1[e] * scale2;
+        }
+        if (key0 < lo || key0 + 31 > p) {                          // a unit at an end of the range: mask
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int k0 = key0 + 4 * g + e, k1 = k0 + 16;
+                if (k0 > p || k0 < lo) s[e] = -INFINITY;
+                if (k1 > p || k1 < lo) s[4 + e] = -INFINITY;
+            }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        if (__any(mx > m_ref + LAZY_LOG2)) {                       // rare after the first unit
+            const float m_new = fmaxf(m_ref, mx);
+            const float f = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+            l *= f;
+            float f4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) f4[e] = __shfl(f, 4 * g + e, 64);
+#pragma unroll
+            for (int d = 0; d < HDT; ++d)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[d][e] *= f4[e];
+            m_ref = m_new;
+        }
+        const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
+        frag16 pf;
+        float sum = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float pe = __builtin_amdgcn_exp2f(s[e] - m_use);
+            sum += pe;
+            pf.v[e] = (__bf16)pe;
+        }
+        l += sum;
+        // O += P V, then the V registers are free for the next unit
+#pragma unroll
+        for (int d = 0; d < HDT; ++d) o[d] = mfma_16x16x32(pf, vb[d], o[d]);
+        vp = nvp;
+        if (n_have) load_v(n_half);
+        half = n_half;
+        cur_page = n_page;
+        have = n_have;
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+
+    // every wave leaves its (unnormalised) rows, references and sums in LDS
+    float* sm_o = lds;
+    float* sm_ml = lds + (size_t)4 * slots * hd;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int slot = 4 * g + e;
+        if (slot < slots) {
+            float* dst = sm_o + ((size_t)wave * slots + slot) * hd;
+#pragma unroll
+            for (int d = 0; d < HDT; ++d) dst[16 * d + j] = o[d][e];
+        }
+    }
+    if (lane < 16) {
+        sm_ml[(wave * 16 + lane) * 2 + 0] = m_ref;
+        sm_ml[(wave * 16 + lane) * 2 + 1] = l;
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < slots * hd; idx += 256) {
+        const int slot = idx / hd, d = idx % hd;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) mm = fmaxf(mm, sm_ml[(x * 16 + slot) * 2]);
+        float acc = 0.f, ll = 0.f;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+            const float mx = sm_ml[(x * 16 + slot) * 2];
+            if (mx != -INFINITY) {
+                const float f = __builtin_amdgcn_exp2f(mx - mm);
+                acc += sm_o[((size_t)x * slots + slot) * hd + d] * f;
+                ll += sm_ml[(x * 16 + slot) * 2 + 1] * f;
+            }
+        }
+        const int head = kvh * G + chunk * 16 + slot;
+        if (a.splits == 1) {
+            a.out[(size_t)t * a.ldo + (size_t)head * hd + d] = f32_to_bf16(ll > 0.f ? acc / ll : 0.f);
+        } else {
+            const size_t ps = ((size_t)t * a.nh + head) * a.splits + split;
+            a.part_o[ps * hd + d] = acc;
+            if (d == 0) {
+                a.part_ml[ps * 2 + 0] = mm * 0.6931471805599453f;    // the combine pass works in natural logarithms
+                a.part_ml[ps * 2 + 1] = ll;
+            }
+        }
+    }
+}
+
 #define COMBINE_MAX_SPLITS 256
 __global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                     bf16* __restrict__ out, long ldo, int nh, int hd, int splits) {
@@ -461,7 +670,16 @@ extern "C" int agave_attn_decode_mfma(const void* q, long ldq, void* out, long l
         hipError_t e3 = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
         AGAVE_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "attn_decode_mfma: cannot raise the LDS allowance");
     }
-    if (hd <= 64) attn_decode_mfma_kernel<4><<<grid, 256, lds, stream>>>(a);
+    if (lds > 48 * 1024) {
+        hipError_t e1 = hipFuncSetAttribute((const void*)attn_decode_fast_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        hipError_t e2 = hipFuncSetAttribute((const void*)attn_decode_fast_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        hipError_t e3 = hipFuncSetAttribute((const void*)attn_decode_fast_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+        AGAVE_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "attn_decode_mfma: cannot raise the LDS allowance");
+    }
+    if (hd == 64) attn_decode_fast_kernel<4><<<grid, 256, lds, stream>>>(a);
+    else if (hd == 128) attn_decode_fast_kernel<8><<<grid, 256, lds, stream>>>(a);
+    else if (hd == 256) attn_decode_fast_kernel<16><<<grid, 256, lds, stream>>>(a);
+    else if (hd <= 64) attn_decode_mfma_kernel<4><<<grid, 256, lds, stream>>>(a);
     else if (hd <= 128) attn_decode_mfma_kernel<8><<<grid, 256, lds, stream>>>(a);
     else attn_decode_mfma_kernel<16><<<grid, 256, lds, stream>>>(a);
     AGAVE_LAUNCH_CHECK("attn_decode_mfma");
