@@ -102,28 +102,35 @@ __device__ __forceinline__ float gelu_tanh_f(float x) {
     return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
 }
 
-#define SK_KS 4                    // k-steps (tiles of 32 columns) per chunk
-#define SK_ROW (SK_KS * 32 + 8)    // bf16 per staged X row: 128 columns + 16 bytes of padding
-
 // R: row blocks (of 16 weight rows) per workgroup; MT: tiles of 16 tokens; EPI 0: store, 1: GeGLU;
 // NW: waves per workgroup, which share the columns (few row blocks -> many waves each, so
 // that a small matrix still has enough loads in flight; the sums meet in LDS, never in memory).
+// A wave takes chunks of KS k-steps (tiles of 32 columns): 128 columns for up to 32 tokens, 64 beyond
+// (the registers that hold a chunk in flight grow with R and MT).  Every workgroup stages all of X
+// once, so with many tokens R grows: X then comes from L2 once per R row blocks.
 template <int R, int MT, int EPI, int NW, typename TC>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ X, long ldx,
                                                           const uint4* __restrict__ Wp, TC* __restrict__ Y,
                                                           long ldy, int M, int N, int K, int KB, int NB) {
-    // staged X: [wave][MT][16 rows][SK_ROW]; afterwards the same memory holds the waves' partial sums
-    constexpr int XS_WAVE = MT * 16 * SK_ROW;                       // bf16 elements
+    constexpr int KS = MT <= 2 ? 4 : 2;
+    constexpr int ROW = KS * 32 + 8;                                // bf16 per staged X row, 16 bytes of padding
+    constexpr int PIECES = KS * 4;                                  // 16-byte pieces per staged row
+    constexpr int RPI = 64 / PIECES;                                // rows one load instruction covers
+    constexpr int NI = 16 / RPI;                                    // load instructions per tile of 16 tokens
+    // staged X: [wave][MT][16 rows][ROW]; afterwards the same memory holds the waves' partial sums
+    constexpr int XS_WAVE = MT * 16 * ROW;                          // bf16 elements
     constexpr int RED_WAVE = R * MT * 64 * 4;                       // floats
     constexpr int LDS_BYTES = (NW * XS_WAVE * 2 > NW * RED_WAVE * 4) ? NW * XS_WAVE * 2 : NW * RED_WAVE * 4;
+    static_assert(LDS_BYTES <= 160 * 1024, "the staged tokens or the partial sums do not fit the LDS");
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
     bf16* xs = reinterpret_cast<bf16*>(smem);
     float* red = reinterpret_cast<float*>(smem);
 
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int j = lane & 15, g = lane >> 4;
+    const int xr = lane / PIECES, xp = lane % PIECES;               // staging: row within an instruction, piece
     const int nb0 = blockIdx.x * R;
-    const int n_chunks = (KB + SK_KS - 1) / SK_KS;
+    const int n_chunks = (KB + KS - 1) / KS;
     const int n_iter = (n_chunks + NW - 1) / NW;
 
     f32x4_t acc[R][MT];
@@ -132,8 +139,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[r][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    frag16 wreg[R][SK_KS];
-    uint4 xreg[MT][4];
+    frag16 wreg[R][KS];
+    uint4 xreg[MT][NI];
     bf16* my_xs = xs + wave * XS_WAVE;
 
     auto load_global = [&](int it) {
@@ -142,8 +149,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int ks = 0; ks < SK_KS; ++ks) {
-                const int kb = c * SK_KS + ks;
+            for (int ks = 0; ks < KS; ++ks) {
+                const int kb = c * KS + ks;
                 if (active && kb < KB && nb0 + r < NB)
                     wreg[r][ks].u = Wp[((size_t)(nb0 + r) * KB + kb) * 64 + lane];
                 else
@@ -152,9 +159,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int row = mt * 16 + 4 * i + g;              // 4 rows per instruction, 16 lanes a row
-                const int k = c * (SK_KS * 32) + j * 8;
+            for (int i = 0; i < NI; ++i) {
+                const int row = mt * 16 + RPI * i + xr;
+                const int k = c * (KS * 32) + xp * 8;
                 if (active && row < M && k < K)
                     xreg[mt][i] = *reinterpret_cast<const uint4*>(X + (size_t)row * ldx + k);
                 else
@@ -167,21 +174,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *reinterpret_cast<uint4*>(my_xs + (mt * 16 + 4 * i + g) * SK_ROW + j * 8) = xreg[mt][i];
-        frag16 wcur[R][SK_KS];
+            for (int i = 0; i < NI; ++i)
+                *reinterpret_cast<uint4*>(my_xs + (mt * 16 + RPI * i + xr) * ROW + xp * 8) = xreg[mt][i];
+        frag16 wcur[R][KS];
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int ks = 0; ks < SK_KS; ++ks) wcur[r][ks] = wreg[r][ks];
+            for (int ks = 0; ks < KS; ++ks) wcur[r][ks] = wreg[r][ks];
         if (it + 1 < n_iter) load_global(it + 1);
         __syncthreads();
 #pragma unroll
-        for (int ks = 0; ks < SK_KS; ++ks)
+        for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 frag16 xb;
-                xb.u = *reinterpret_cast<const uint4*>(my_xs + (mt * 16 + j) * SK_ROW + ks * 32 + g * 8);
+                xb.u = *reinterpret_cast<const uint4*>(my_xs + (mt * 16 + j) * ROW + ks * 32 + g * 8);
 #pragma unroll
                 for (int r = 0; r < R; ++r) acc[r][mt] = mfma_16x16x32(wcur[r][ks], xb, acc[r][mt]);
             }
@@ -218,6 +225,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     }
 }
 
+// A choice of R and NW forced from outside (0: the heuristics below); for measurements only.
+static int g_skinny_force_r = 0, g_skinny_force_nw = 0;
+extern "C" int agave_gemm_skinny_tune(int r, int nw) {
+    g_skinny_force_r = r;
+    g_skinny_force_nw = nw;
+    return 0;
+}
+
 template <int R, int MT, int EPI, int NW, typename TC>
 static void launch_skinny_nw(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                              int NB, hipStream_t stream) {
@@ -226,20 +241,28 @@ static void launch_skinny_nw(const void* X, long ldx, const void* Wp, void* Y, l
                                                                         ldy, M, N, K, KB, NB);
 }
 
+// Waves per workgroup: the fewest that put about 2048 waves on the chip (enough loads in
+// flight to cover the memory's latency), within what the registers and the LDS allow; more
+// waves than that only add to the merge of the sums and deal the chunks less evenly.
+static int skinny_waves(int groups, int n_chunks, int max_nw) {
+    if (g_skinny_force_nw) return g_skinny_force_nw <= max_nw ? g_skinny_force_nw : max_nw;
+    int nw = 4;
+    while (nw < max_nw && (long)groups * nw < 2048 && nw < n_chunks) nw *= 2;
+    return nw;
+}
+
 template <int R, int MT, int EPI, typename TC>
 static void launch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                           int NB, hipStream_t stream) {
-    // waves per workgroup: as many as the chunks of columns and the LDS allow while row blocks are few
-    const int n_chunks = (KB + SK_KS - 1) / SK_KS;
+    constexpr int KS = MT <= 2 ? 4 : 2;
+    constexpr int MAX_NW = (R * MT <= 2) ? 16 : (R * MT <= 8 ? 8 : 4);
+    const int n_chunks = (KB + KS - 1) / KS;
     const int groups = (NB + R - 1) / R;
-    int nw = groups >= 1536 ? 4 : (groups >= 640 ? 8 : 16);
-    if (MT >= 3 && nw > 4) nw = 4;
-    if (MT == 2 && nw > 8) nw = 8;
-    while (nw > 4 && nw > n_chunks) nw /= 2;
+    const int nw = skinny_waves(groups, n_chunks, MAX_NW);
     if (nw == 16) {
-        if constexpr (MT == 1) launch_skinny_nw<R, MT, EPI, 16, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        if constexpr (MAX_NW >= 16) launch_skinny_nw<R, MT, EPI, 16, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     } else if (nw == 8) {
-        if constexpr (MT <= 2) launch_skinny_nw<R, MT, EPI, 8, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        if constexpr (MAX_NW >= 8) launch_skinny_nw<R, MT, EPI, 8, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     } else {
         launch_skinny_nw<R, MT, EPI, 4, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     }
@@ -249,17 +272,30 @@ template <int EPI, typename TC>
 static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                            int NB, hipStream_t stream) {
     const int mt = (M + 15) / 16;
-    // two row blocks per workgroup once there are plenty of them, so that X is staged half as often
-    const bool wide = NB >= 4096;
+    // Row blocks per workgroup: every workgroup reads all of X, so the traffic from L2 is
+    // (1 + 16*MT/(16*R)) times the weights'; more row blocks as long as enough workgroups remain.
+    int r = 1;
+    if (mt == 1) r = NB >= 4096 ? 2 : 1;
+    else if (mt == 2) r = NB >= 4096 ? 4 : (NB >= 1024 ? 2 : 1);
+    else r = NB >= 1024 ? 4 : 1;
+    if (g_skinny_force_r) r = g_skinny_force_r;
+    if (mt <= 1 && r > 2) r = 2;
 #define SK_CASE(R_, MT_)                                                                        \
     launch_skinny<R_, MT_, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);              \
     break
-    switch (mt) {
-        case 1: if (wide) { SK_CASE(2, 1); } else { SK_CASE(1, 1); }
-        case 2: if (wide) { SK_CASE(2, 2); } else { SK_CASE(1, 2); }
-        case 3: if (wide) { SK_CASE(2, 3); } else { SK_CASE(1, 3); }
-        case 4: if (wide) { SK_CASE(2, 4); } else { SK_CASE(1, 4); }
-        default: AGAVE_CHECK(false, "gemm_skinny: M=%d exceeds 64", M);
+    switch (mt * 8 + r) {
+        case 1 * 8 + 1: SK_CASE(1, 1);
+        case 1 * 8 + 2: SK_CASE(2, 1);
+        case 2 * 8 + 1: SK_CASE(1, 2);
+        case 2 * 8 + 2: SK_CASE(2, 2);
+        case 2 * 8 + 4: SK_CASE(4, 2);
+        case 3 * 8 + 1: SK_CASE(1, 3);
+        case 3 * 8 + 2: SK_CASE(2, 3);
+        case 3 * 8 + 4: SK_CASE(4, 3);
+        case 4 * 8 + 1: SK_CASE(1, 4);
+        case 4 * 8 + 2: SK_CASE(2, 4);
+        case 4 * 8 + 4: SK_CASE(4, 4);
+        default: AGAVE_CHECK(false, "gemm_skinny: no kernel for %d tokens with %d row blocks a workgroup", M, r);
     }
 #undef SK_CASE
     return 0;
