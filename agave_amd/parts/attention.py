@@ -58,23 +58,33 @@ class Attention:
         n = x.shape[0]
         k_pages, v_pages, packed = step.cache.pages_of(memory)
         table, base = step.tables[step.cache.group_of_memory[memory]]
-        inv_freq, pos_scale = (None, 1.0)
         fused = getattr(self.position, "fused_rotation", None)
         qkv = self.qkv.forward(x, tag="qkv")
         q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
         if not writes:
             k = v = None            # a run that reads another run's cache appends nothing
+        q_out = ws.get("q_rot", n, self.qd, x.dtype)
+        qg, kg = (self.q_norm.gain if self.q_norm else None), (self.k_norm.gain if self.k_norm else None)
+        qe, ke = (self.q_norm.eps if self.q_norm else 0.0), (self.k_norm.eps if self.k_norm else 0.0)
         if fused is not None:
             inv_freq, pos_scale = fused()
+            kernels.qk_norm_rope_kv(q, k, v, q_out, qg, kg, qe, ke, inv_freq, pos_scale, step.tok_seq, step.tok_pos,
+                                    k_pages, v_pages, table, base, s.n_heads, s.n_kv_heads, s.head_dim, packed)
         else:
-            self.position.apply(q, k, step)
-        q_out = ws.get("q_rot", n, self.qd, x.dtype)
-        kernels.qk_norm_rope_kv(
-            q, k, v, q_out,
-            self.q_norm.gain if self.q_norm else None, self.k_norm.gain if self.k_norm else None,
-            self.q_norm.eps if self.q_norm else 0.0, self.k_norm.eps if self.k_norm else 0.0,
-            inv_freq, pos_scale, step.tok_seq, step.tok_pos, k_pages, v_pages, table, base,
-            s.n_heads, s.n_kv_heads, s.head_dim, packed)
+            # a position encoding the q/k kernel does not know: the norms, then the part's own
+            # ``apply`` on the normalised rows, then the cache write
+            kernels.qk_norm_rope_kv(q, None, None, q_out, qg, None, qe, 0.0, None, 1.0, step.tok_seq, step.tok_pos,
+                                    None, None, None, None, s.n_heads, 0, s.head_dim)
+            k_n = None
+            if k is not None:
+                k_n = ws.get("k_normed", n, self.kvd, x.dtype)
+                kernels.qk_norm_rope_kv(k, None, None, k_n, kg, None, ke, 0.0, None, 1.0, step.tok_seq, step.tok_pos,
+                                        None, None, None, None, s.n_kv_heads, 0, s.head_dim)
+            self.position.apply(q_out, k_n, step)
+            if k is not None:
+                kernels.qk_norm_rope_kv(None, k_n, v, None, None, None, 0.0, 0.0, None, 1.0, step.tok_seq,
+                                        step.tok_pos, k_pages, v_pages, table, base, 0, s.n_kv_heads, s.head_dim,
+                                        packed)
         ctx_out = ws.get("attn_ctx", n, self.qd, x.dtype)
         attn_ops.attention(q_out, ctx_out, k_pages, v_pages, table, base, step, s.n_heads, s.n_kv_heads,
                            s.head_dim, s.scale, s.window, packed)

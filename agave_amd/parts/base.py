@@ -10,7 +10,9 @@ Interfaces (duck-typed; the classes below document them):
 * norm:        ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, fields ``gain`` (float32
                on the device, any "+1" folded in) and ``eps``; the residual kernels take those.
 * position:    ``__init__(spec, env)``, ``fused_rotation() -> (inv_freq | None, pos_scale)`` when the
-               q/k kernel can apply it, else ``apply(q, k, step)`` on the projected rows.
+               q/k kernel can apply it (a rotation of pairs, or nothing), else ``apply(q, k, step)``:
+               in place on the normalised rows q [N, heads*head_dim] and k [N, kv_heads*head_dim]
+               (k is None in a run that appends nothing), positions in ``step.tok_pos``.
 * mixer:       ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, ``kv_need() -> GroupKey | None``,
                ``state_need() -> StateNeed | None``,
                ``forward(x[N, hidden], step, memory, writes) -> [N, hidden]``.

@@ -132,3 +132,37 @@ def test_graph_replays_equal_eager_steps(tiny, dtype):
             a.step([other], [U.random_tokens(5, v, i)], "last")
             torch.cuda.synchronize()
     assert len(a.graphs._graphs) >= 1
+
+
+def test_long_decoding(engine_of):
+    """A short prompt, then many tokens one by one: over page edges, past the window's reach (the
+    window groups give pages back while the sequence grows) and through many graph replays."""
+    eng, dtype, cfg, weights = engine_of
+    toks = U.random_tokens(190, cfg["vocab_size"], 80)
+    ref = U.plain_logits(cfg, weights, toks)
+    close(dtype)(U.run_tail(eng, toks, 183), ref, "long decoding")
+    for g in eng.cache.groups:
+        assert g.pool.n_free == g.pool.n_pages
+
+
+def test_prompt_in_pieces(engine_of):
+    """Steps of several tokens that start in the middle of a sequence (a prompt that enters in
+    pieces): pieces that end on a page's edge, one short of it and one past it, for two
+    sequences of unequal lengths at once."""
+    eng, dtype, cfg, weights = engine_of
+    v = cfg["vocab_size"]
+    reqs = [U.random_tokens(170, v, 90), U.random_tokens(131, v, 91)]
+    cuts = [(0, 63, 64, 129, 170), (0, 1, 65, 128, 131)]
+    slots = [eng.alloc_slot() for _ in reqs]
+    outs = [[], []]
+    for piece in range(4):
+        chunks = [r[c[piece]:c[piece + 1]] for r, c in zip(reqs, cuts)]
+        logits = eng.step(slots, chunks, "all").float().cpu()
+        o = 0
+        for i, ch in enumerate(chunks):
+            outs[i].append(logits[o:o + len(ch)].clone())
+            o += len(ch)
+    for s in slots:
+        eng.free_slot(s)
+    for i, r in enumerate(reqs):
+        close(dtype)(torch.cat(outs[i], 0), U.plain_logits(cfg, weights, r), f"request {i} in pieces")

@@ -1,0 +1,311 @@
+"""Parts that the framework does not have, defined here and registered from outside: a mixer
+with state of its own, a feed-forward with routing, another position encoding, and an
+architecture that arranges them with the built-in attention in a run order that names a
+layer twice and lets a layer read another layer's cache.  No file of the framework changes:
+the model is built from its folder by ``Engine.from_folder`` and stepped like any other.
+
+The toy parts compute with torch on the GPU (they are test fixtures, not product code); the
+framework's own parts beside them run their kernels.  Everything is compared with a plain
+whole-sequence statement of the same model below.
+"""
+import json
+import math
+import os
+from dataclasses import dataclass
+from typing import List, Optional
+
+import pytest
+import torch
+
+import engine_utils as U
+import plain_gemma3 as P
+
+pytestmark = pytest.mark.gpu
+
+HIDDEN, VOCAB, HEADS, KV, HD, INTER, EXPERTS, WINDOW = 96, 211, 4, 2, 32, 120, 3, 20
+EPS, THETA = 1e-5, 5000.0
+
+
+# ---------------------------------------------------------------- the toy parts
+def define_and_register():
+    from agave_amd.cache import StateNeed
+    from agave_amd.config import register_architecture
+    from agave_amd.config.registry import Architecture
+    from agave_amd.config.spec import (AttentionSpec, FeedForwardSpec, GatedFfnSpec, LayerSpec, MixerSpec, ModelSpec,
+                                       NormSpec, PositionSpec, RunEntry)
+    from agave_amd.parts import register
+    from agave_amd.weights.loader import TensorNeed
+
+    @dataclass(frozen=True)
+    class DecaySpec(MixerSpec):
+        hidden: int = 0
+        decay: str = ""
+        out_proj: str = ""
+
+    class DecayMixer:
+        """s_t = sigmoid(d) * s_{t-1} + x_t ;  y_t = W s_t.  The state s is kept per sequence."""
+
+        def __init__(self, spec, weights, env):
+            self.a = torch.sigmoid(weights.get(spec.decay).float().to(env.device))
+            self.w = weights.get(spec.out_proj).float().to(env.device)
+            self.spec, self.env = spec, env
+
+        @staticmethod
+        def tensor_needs(spec):
+            return [TensorNeed(spec.decay, (spec.hidden,)), TensorNeed(spec.out_proj, (spec.hidden, spec.hidden))]
+
+        def kv_need(self):
+            return None
+
+        def state_need(self):
+            return StateNeed((self.spec.hidden,), torch.float32)
+
+        def forward(self, x, step, memory, writes=True):
+            state = step.cache.state[memory]
+            xf = x.float()
+            if step.is_decode:                       # device indices only: the step may be a graph replay
+                idx = step.slots_dev.long()
+                s = self.a * state[idx] + xf
+                state[idx] = s
+                return (s @ self.w.T).to(x.dtype)
+            out = torch.empty_like(xf)
+            for i, slot in enumerate(step.slots):
+                s = state[slot].clone()
+                for t in range(step.cu[i], step.cu[i + 1]):
+                    s = self.a * s + xf[t]
+                    out[t] = s
+                state[slot] = s
+            return (out @ self.w.T).to(x.dtype)
+
+    @dataclass(frozen=True)
+    class TopOneSpec(FeedForwardSpec):
+        hidden: int = 0
+        intermediate: int = 0
+        experts: int = 0
+        router: str = ""
+        w_in: str = ""
+        w_out: str = ""
+
+    class TopOneFfn:
+        """Router logits in 32-bit; the token goes through the one expert with the largest logit,
+        weighted by how far its softmax weight lies above the second largest (so the output is
+        continuous where the choice changes, and rounding cannot make a large difference)."""
+
+        def __init__(self, spec, weights, env):
+            self.r = weights.get(spec.router).float().to(env.device)
+            self.w_in = weights.get(spec.w_in).float().to(env.device)
+            self.w_out = weights.get(spec.w_out).float().to(env.device)
+
+        @staticmethod
+        def tensor_needs(spec):
+            return [TensorNeed(spec.router, (spec.experts, spec.hidden)),
+                    TensorNeed(spec.w_in, (spec.experts, spec.intermediate, spec.hidden)),
+                    TensorNeed(spec.w_out, (spec.experts, spec.hidden, spec.intermediate))]
+
+        def forward(self, x, step):
+            xf = x.float()
+            logits = xf @ self.r.T
+            p = torch.softmax(logits, -1)
+            e = logits.argmax(-1)
+            hid = torch.nn.functional.gelu(torch.einsum("eih,nh->nei", self.w_in, xf), approximate="tanh")
+            y = torch.einsum("ehi,nei->neh", self.w_out, hid)
+            top2 = p.topk(2, -1).values
+            pick = torch.nn.functional.one_hot(e, logits.shape[-1]).float() * (top2[:, :1] - top2[:, 1:])
+            return torch.einsum("neh,ne->nh", y, pick).to(x.dtype)
+
+    class WobblePosition:
+        """Not a rotation: every element of q and k is multiplied by 1 + 0.3 cos(pos * f_i)."""
+
+        def __init__(self, spec, env):
+            i = torch.arange(spec.rotary_dim, dtype=torch.float32, device=env.device)
+            self.f = 0.05 + 0.01 * i
+
+        def apply(self, q, k, step):
+            pos = step.tok_pos.float()[:, None]
+            m = 1.0 + 0.3 * torch.cos(pos * self.f[None, :])          # [N, head_dim]
+            for t in (q, k):
+                if t is not None:
+                    n = t.shape[0]
+                    v = t.view(n, -1, m.shape[1]) if t.is_contiguous() else t.reshape(n, -1, m.shape[1])
+                    t.copy_((v.float() * m[:, None, :]).to(t.dtype).reshape(n, -1))
+
+    register("mixer", "toy_decay", DecayMixer)
+    register("ffn", "toy_top_one", TopOneFfn)
+    register("position", "toy_wobble", WobblePosition)
+
+    def norm(name):
+        return NormSpec("rmsnorm", HIDDEN, EPS, name, True)
+
+    def attention(prefix, window, position):
+        return AttentionSpec(kind="attention", hidden=HIDDEN, n_heads=HEADS, n_kv_heads=KV, head_dim=HD,
+                             scale=1.0 / math.sqrt(HD), window=window, position=position,
+                             q_norm=NormSpec("rmsnorm", HD, EPS, prefix + "qn", True),
+                             k_norm=NormSpec("rmsnorm", HD, EPS, prefix + "kn", True),
+                             q_proj=prefix + "q", k_proj=prefix + "k", v_proj=prefix + "v", o_proj=prefix + "o")
+
+    def dense(prefix):
+        return GatedFfnSpec(kind="gated_dense", hidden=HIDDEN, intermediate=INTER, activation="gelu_tanh",
+                            gate_proj=prefix + "g", up_proj=prefix + "u", down_proj=prefix + "d")
+
+    def layer(i, kind, mixer, ffn):
+        return LayerSpec(kind=kind, mixer=mixer, ffn=ffn, pre_mixer_norm=norm(f"l{i}.n0"),
+                         post_mixer_norm=norm(f"l{i}.n1"), pre_ffn_norm=norm(f"l{i}.n2"),
+                         post_ffn_norm=norm(f"l{i}.n3"))
+
+    def spec_of(cfg, names=None):
+        rope = PositionSpec("rope", HD, THETA, 1.0)
+        layers = [
+            layer(0, "prenorm", DecaySpec("toy_decay", HIDDEN, "l0.decay", "l0.w"),
+                  TopOneSpec("toy_top_one", HIDDEN, INTER, EXPERTS, "l0.router", "l0.w_in", "l0.w_out")),
+            layer(1, "sandwich", attention("l1.", WINDOW, PositionSpec("toy_wobble", HD)), dense("l1.")),
+            layer(2, "sandwich", attention("l2.", None, rope), dense("l2.")),
+            layer(3, "sandwich", attention("l3.", None, rope), dense("l3.")),
+        ]
+        order = [RunEntry(0, 0), RunEntry(1, 1), RunEntry(2, 2),
+                 RunEntry(0, 3),                       # layer 0 again, with a state of its own
+                 RunEntry(3, 2, writes=False)]         # layer 3 reads what layer 2 cached and appends nothing
+        return ModelSpec(architecture="ToyMixForCausalLM", vocab_size=VOCAB, hidden=HIDDEN, embed_weight="emb",
+                         embed_scale=1.0, layers=layers, order=order, final_norm=norm("final"), head_weight="head",
+                         max_context=cfg["max_position_embeddings"], eos_token_ids=())
+
+    register_architecture(Architecture("ToyMixForCausalLM", ("toy_mix",), lambda raw: dict(raw), spec_of))
+    return spec_of
+
+
+def toy_weights(seed):
+    from agave_amd.engine.model import tensor_needs
+    spec = define_and_register()({"max_position_embeddings": 512})
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for need in tensor_needs(spec):
+        std = 0.1 if len(need.shape) > 1 else 0.3
+        out[need.name] = (torch.randn(need.shape, generator=g) * std).bfloat16().float()
+    out["emb"] = (out["emb"] * 10).bfloat16().float()
+    return spec, out
+
+
+# ---------------------------------------------------------------- the same model, plainly
+def plain_toy(w, tokens) -> torch.Tensor:
+    W = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    pos = torch.arange(T, dtype=torch.float64)
+    h = W["emb"][torch.tensor(tokens)]
+
+    def n(x, name):
+        return P.rms_norm(x, W[name], EPS)
+
+    def decay(x):
+        a = torch.sigmoid(W["l0.decay"])
+        s = torch.zeros(HIDDEN, dtype=torch.float64)
+        out = []
+        for t in range(T):
+            s = a * s + x[t]
+            out.append(s)
+        return torch.stack(out) @ W["l0.w"].T
+
+    def top_one(x):
+        logits = x @ W["l0.router"].T
+        p = P.softmax_rows(logits)
+        out = torch.zeros_like(x)
+        for t in range(T):
+            e = int(logits[t].argmax())
+            second = max(float(p[t, j]) for j in range(EXPERTS) if j != e)
+            out[t] = (p[t, e] - second) * (W["l0.w_out"][e] @ P.gelu_tanh(W["l0.w_in"][e] @ x[t]))
+        return out
+
+    def qkv(pre, x, position):
+        q = n_heads(x @ W[pre + "q"].T, HEADS, pre + "qn")
+        k = n_heads(x @ W[pre + "k"].T, KV, pre + "kn")
+        v = (x @ W[pre + "v"].T).view(T, KV, HD)
+        if position == "rope":
+            ang = P.rope_angles(pos, HD, THETA, 1.0)
+            q, k = P.apply_rope(q, ang), P.apply_rope(k, ang)
+        else:
+            m = 1.0 + 0.3 * torch.cos(pos[:, None] * (0.05 + 0.01 * torch.arange(HD, dtype=torch.float64))[None, :])
+            q, k = q * m[:, None, :], k * m[:, None, :]
+        return q, k, v
+
+    def n_heads(x, heads, gain):
+        return P.rms_norm(x.view(T, heads, HD), W[gain], EPS)
+
+    def ffn(pre, x):
+        return P.geglu(x, W[pre + "g"], W[pre + "u"], W[pre + "d"])
+
+    scale = 1.0 / math.sqrt(HD)
+    # layer 0 (prenorm: a norm after the routed feed-forward would blow up the small outputs near a
+    # change of expert and make the model discontinuous there): decay mixer, routed feed-forward
+    h = h + decay(n(h, "l0.n0"))
+    h = h + top_one(n(h, "l0.n2"))
+    # layer 1 (sandwich): windowed attention with the wobble
+    q, k, v = qkv("l1.", n(h, "l1.n0"), "wobble")
+    h = h + n(P.attention_core(q, k, v, scale, WINDOW).reshape(T, -1) @ W["l1.o"].T, "l1.n1")
+    h = h + n(ffn("l1.", n(h, "l1.n2")), "l1.n3")
+    # layer 2 (sandwich): global attention; its keys and values are read again below
+    q, k2, v2 = qkv("l2.", n(h, "l2.n0"), "rope")
+    h = h + n(P.attention_core(q, k2, v2, scale, None).reshape(T, -1) @ W["l2.o"].T, "l2.n1")
+    h = h + n(ffn("l2.", n(h, "l2.n2")), "l2.n3")
+    # layer 0 once more, its state starting from zero again
+    h = h + decay(n(h, "l0.n0"))
+    h = h + top_one(n(h, "l0.n2"))
+    # layer 3: its own queries over layer 2's keys and values
+    q, _, _ = qkv("l3.", n(h, "l3.n0"), "rope")
+    h = h + n(P.attention_core(q, k2, v2, scale, None).reshape(T, -1) @ W["l3.o"].T, "l3.n1")
+    h = h + n(ffn("l3.", n(h, "l3.n2")), "l3.n3")
+    return n(h, "final") @ W["head"].T
+
+
+# ---------------------------------------------------------------- the tests
+@pytest.fixture(scope="module")
+def toy(tmp_path_factory):
+    from safetensors.torch import save_file
+    spec, w = toy_weights(5)
+    folder = str(tmp_path_factory.mktemp("toy"))
+    save_file({k: v.bfloat16().contiguous() for k, v in w.items()}, os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump({"architectures": ["ToyMixForCausalLM"], "model_type": "toy_mix", "max_position_embeddings": 512}, f)
+    return folder, w
+
+
+def close(got, ref, dtype, what):
+    scale = float(ref.abs().max())
+    err = (got.double() - ref).abs().max(dim=-1).values
+    tol = 3e-5 if dtype == "float32" else 0.04
+    assert float(err.max()) <= tol * scale, f"{what}: error {float(err.max()):.3e} of {scale:.3e} at row {int(err.argmax())}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_model_is_built_and_stepped(toy, dtype):
+    from agave_amd.engine import Engine
+    folder, w = toy
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=3, max_context=256)
+    assert set(eng.cache.state) == {0, 3}                       # the decay mixer's two runs, a state each
+    assert sorted(eng.cache.group_of_memory) == [1, 2]          # the two attention memories; layer 3 has none
+    assert len(eng.cache.groups) == 2                           # a window group and a group of all keys
+
+    toks = U.random_tokens(100, VOCAB, 1)
+    ref = plain_toy(w, toks)
+    close(U.run_whole(eng, toks), ref, dtype, "whole")
+    close(U.run_tail(eng, toks, 32), ref, dtype, "last 32 one by one (graph replays among them)")
+
+    # batches of unequal lengths, one after another: slots, pages and states are used again
+    for b, (lens, first) in enumerate([((50, 21, 80), (30, 21, 2)), ((70, 33), (69, 1)), ((90, 9, 40), (5, 9, 38))]):
+        reqs = [U.random_tokens(n, VOCAB, 10 * b + i) for i, n in enumerate(lens)]
+        outs = U.run_batched(eng, reqs, first)
+        for i, (r, o) in enumerate(zip(reqs, outs)):
+            close(o, plain_toy(w, r), dtype, f"batch {b} request {i}")
+    assert eng.cache.slots.n_free == eng.cache.max_slots
+
+
+def test_toy_model_generates(toy):
+    """Greedy generation through the entry point, against the plain model's own greedy loop."""
+    from agave_amd.engine import Engine
+    from agave_amd.sampling import SamplingParams
+    folder, w = toy
+    eng = Engine.from_folder(folder, dtype="float32", max_slots=2, max_context=128)
+    prompts = [U.random_tokens(7, VOCAB, 50), U.random_tokens(19, VOCAB, 51)]
+    res = eng.generate(prompts, SamplingParams(temperature=0.0, max_tokens=6))
+    for p, r in zip(prompts, res):
+        seq = list(p)
+        for _ in range(6):
+            seq.append(P.argmax_first(plain_toy(w, seq)[-1]))
+        assert list(r.tokens) == seq[len(p):]
