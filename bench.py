@@ -138,6 +138,8 @@ def main() -> int:
                     help="run fewer layers of the same sizes (reported in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="time only the 2048-token prefill and print its record (for profiles)")
     args = ap.parse_args()
     world = int(os.environ.get("WORLD_SIZE", "1"))
     if args.gpus != 1 or world != 1:
@@ -158,6 +160,13 @@ def main() -> int:
     engine = Engine.from_random(cfg, seed=0, dtype=args.dtype, max_slots=max_batch, max_context=CONTEXT,
                                 cache_tokens=cache_tokens, device="cuda:0")
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
+    if args.prefill_only:
+        pdt = run_prefill(engine, seed=2)
+        print(json.dumps({"prefill": {"value": round(PREFILL_LEN / pdt, 1), "tokens": PREFILL_LEN,
+                                      "ms": round(pdt * 1e3, 3),
+                                      "frac": round(prefill_flops(m, PREFILL_LEN) / pdt / PEAK_FLOPS[dkey], 4)}}),
+              flush=True)
+        return 0
 
     dt, contexts = run_decode(engine, args.batch, args.steps, args.warmup, seed=1)
     ms_step = dt / args.steps * 1e3
