@@ -107,8 +107,10 @@ __device__ __forceinline__ float gelu_tanh_f(float x) {
 // that a small matrix still has enough loads in flight; the sums meet in LDS, never in memory).
 // A wave takes chunks of KS k-steps (tiles of 32 columns): 128 columns for up to 32 tokens, 64 beyond
 // (the registers that hold a chunk in flight grow with R and MT).  Every workgroup stages all of X
-// once, so with many tokens R grows: X then comes from L2 once per R row blocks.
-template <int R, int MT, int EPI, int NW, typename TC>
+// once, so with many tokens R grows: X then comes from L2 once per R row blocks.  XR: rows of the
+// token tile that are loaded at all (4, 8 or 16 when there is one tile; a workgroup reads as many
+// bytes of X as of W when all 16 are loaded, so a step of 8 tokens should not load 16).
+template <int R, int MT, int EPI, int NW, typename TC, int XR>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ X, long ldx,
                                                           const uint4* __restrict__ Wp, TC* __restrict__ Y,
                                                           long ldy, int M, int N, int K, int KB, int NB) {
@@ -116,7 +118,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     constexpr int ROW = KS * 32 + 8;                                // bf16 per staged X row, 16 bytes of padding
     constexpr int PIECES = KS * 4;                                  // 16-byte pieces per staged row
     constexpr int RPI = 64 / PIECES;                                // rows one load instruction covers
-    constexpr int NI = 16 / RPI;                                    // load instructions per tile of 16 tokens
+    constexpr int NI = XR / RPI;                                    // load instructions per tile of 16 tokens
+    static_assert(XR == 16 || MT == 1, "only a single tile of tokens may be cut short");
+    static_assert(XR % RPI == 0 && XR <= 16, "rows of the tile must be whole load instructions");
     // staged X: [wave][MT][16 rows][ROW]; afterwards the same memory holds the waves' partial sums
     constexpr int XS_WAVE = MT * 16 * ROW;                          // bf16 elements
     constexpr int RED_WAVE = R * MT * 64 * 4;                       // floats
@@ -139,61 +143,92 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[r][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    frag16 wreg[R][KS];
-    uint4 xreg[MT][NI];
+    // S chunks are in flight per wave: the loads of chunk i+S are issued as soon as chunk i has
+    // been multiplied, long before they are waited for.
+    constexpr int S = (R * MT <= 2 && NW <= 8) ? 3 : 2;      // 16 waves leave 128 registers a lane
+    frag16 wreg[S][R][KS];
+    uint4 xreg[S][MT][NI];
     bf16* my_xs = xs + wave * XS_WAVE;
 
-    auto load_global = [&](int it) {
-        const int c = it * NW + wave;                // chunks are dealt to the waves in turn
-        const bool active = c < n_chunks;
+    // addresses that do not depend on the chunk; rows past the end repeat the last one (their
+    // results are never stored)
+    const uint4* wrow[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r)
+    for (int r = 0; r < R; ++r) wrow[r] = Wp + (size_t)(nb0 + r < NB ? nb0 + r : NB - 1) * KB * 64 + lane;
+    const bf16* xrow[MT][NI];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const int kb = c * KS + ks;
-                if (active && kb < KB && nb0 + r < NB)
-                    wreg[r][ks].u = Wp[((size_t)(nb0 + r) * KB + kb) * 64 + lane];
-                else
-                    wreg[r][ks].u = uint4{0, 0, 0, 0};
-            }
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const int row = mt * 16 + RPI * i + xr;
-                const int k = c * (KS * 32) + xp * 8;
-                if (active && row < M && k < K)
-                    xreg[mt][i] = *reinterpret_cast<const uint4*>(X + (size_t)row * ldx + k);
-                else
-                    xreg[mt][i] = uint4{0, 0, 0, 0};
-            }
-    };
+        for (int i = 0; i < NI; ++i) {
+            const int row = mt * 16 + RPI * i + xr;
+            xrow[mt][i] = X + (size_t)(row < M ? row : M - 1) * ldx;
+        }
 
-    load_global(0);
-    for (int it = 0; it < n_iter; ++it) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int i = 0; i < NI; ++i)
-                *reinterpret_cast<uint4*>(my_xs + (mt * 16 + RPI * i + xr) * ROW + xp * 8) = xreg[mt][i];
-        frag16 wcur[R][KS];
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) wcur[r][ks] = wreg[r][ks];
-        if (it + 1 < n_iter) load_global(it + 1);
-        __syncthreads();
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                frag16 xb;
-                xb.u = *reinterpret_cast<const uint4*>(my_xs + (mt * 16 + j) * ROW + ks * 32 + g * 8);
-#pragma unroll
-                for (int r = 0; r < R; ++r) acc[r][mt] = mfma_16x16x32(wcur[r][ks], xb, acc[r][mt]);
-            }
-        __syncthreads();
+    // Workgroups walk the columns from different starting chunks (and wrap around): row blocks lie
+    // a multiple of the memory channels' period apart for some K, and workgroups that move in step
+    // would then all read from the same few channels.
+    const int rot = blockIdx.x % n_chunks;
+    // Loads are issued without any condition around them (a chunk past the end repeats the last
+    // one and is not used): only then can a wait name the loads it needs and leave the younger
+    // ones in flight.
+#define SK_LOAD(ST, IT)                                                                          \
+    {                                                                                            \
+        int c_ = (IT) * NW + wave;                    /* chunks are dealt to the waves in turn */ \
+        c_ = (c_ < n_chunks ? c_ : n_chunks - 1) + rot;                                          \
+        c_ = c_ < n_chunks ? c_ : c_ - n_chunks;                                                 \
+        _Pragma("unroll") for (int r = 0; r < R; ++r)                                            \
+            _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                  \
+                const int kb = c_ * KS + ks;           /* past the last tile: any tile, X is zero there */ \
+                wreg[ST][r][ks].u = wrow[r][(size_t)(kb < KB ? kb : KB - 1) * 64];               \
+            }                                                                                    \
+        const int k_ = c_ * (KS * 32) + xp * 8;         /* past the last column: any piece, zeroed when used */ \
+        _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                        \
+            _Pragma("unroll") for (int i = 0; i < NI; ++i)                                       \
+                xreg[ST][mt][i] = *reinterpret_cast<const uint4*>(xrow[mt][i] + (k_ < K ? k_ : 0)); \
     }
+    // The staged rows are this wave's own and LDS serves a wave's accesses in order: no barrier.
+#define SK_USE(ST, IT)                                                                           \
+    if ((IT) * NW + wave < n_chunks) {                                                           \
+        const int pc_ = (IT) * NW + wave + rot;                                                  \
+        const bool in_ = (pc_ < n_chunks ? pc_ : pc_ - n_chunks) * (KS * 32) + xp * 8 < K;       \
+        _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                        \
+            _Pragma("unroll") for (int i = 0; i < NI; ++i)                                       \
+                *reinterpret_cast<uint4*>(my_xs + (mt * 16 + RPI * i + xr) * ROW + xp * 8) =     \
+                    in_ ? xreg[ST][mt][i] : uint4{0, 0, 0, 0};                                   \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks)                                        \
+            _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                  \
+                frag16 xb;                                                                       \
+                xb.u = *reinterpret_cast<const uint4*>(my_xs + (mt * 16 + j) * ROW + ks * 32 + g * 8); \
+                _Pragma("unroll") for (int r = 0; r < R; ++r)                                    \
+                    acc[r][mt] = mfma_16x16x32(wreg[ST][r][ks], xb, acc[r][mt]);                 \
+            }                                                                                    \
+    }
+
+    SK_LOAD(0, 0)
+    SK_LOAD(1, 1)
+    if constexpr (S == 3) SK_LOAD(2, 2)
+    int it = 0;
+    for (; it + 2 * S <= n_iter; it += S) {           // steady state: every load is of a chunk that exists
+        SK_USE(0, it)
+        SK_LOAD(0, it + S)
+        SK_USE(1, it + 1)
+        SK_LOAD(1, it + 1 + S)
+        if constexpr (S == 3) {
+            SK_USE(2, it + 2)
+            SK_LOAD(2, it + 2 + S)
+        }
+    }
+    // the last chunks: at most S - 1 more loads
+    SK_USE(0, it)
+    if (it + S < n_iter) SK_LOAD(0, it + S)
+    SK_USE(1, it + 1)
+    if (it + 1 + S < n_iter) SK_LOAD(1, it + 1 + S)
+    if constexpr (S == 3) SK_USE(2, it + 2)
+    SK_USE(0, it + S)
+    SK_USE(1, it + 1 + S)
+#undef SK_LOAD
+#undef SK_USE
+    __syncthreads();      // the staged rows give way to the partial sums
 
     // the waves' partial sums meet in LDS
 #pragma unroll
@@ -233,25 +268,25 @@ extern "C" int agave_gemm_skinny_tune(int r, int nw) {
     return 0;
 }
 
-template <int R, int MT, int EPI, int NW, typename TC>
+template <int R, int MT, int EPI, int NW, typename TC, int XR>
 static void launch_skinny_nw(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                              int NB, hipStream_t stream) {
     const int grid = (NB + R - 1) / R;
-    gemm_skinny_kernel<R, MT, EPI, NW, TC><<<grid, NW * 64, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y,
+    gemm_skinny_kernel<R, MT, EPI, NW, TC, XR><<<grid, NW * 64, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y,
                                                                         ldy, M, N, K, KB, NB);
 }
 
-// Waves per workgroup: the fewest that put about 2048 waves on the chip (enough loads in
-// flight to cover the memory's latency), within what the registers and the LDS allow; more
-// waves than that only add to the merge of the sums and deal the chunks less evenly.
+// Waves per workgroup: the fewest that put some 640 waves on the chip.  Every wave keeps two
+// or three chunks of loads in flight, which covers the memory's latency with few waves; more
+// waves only add to the merge of the sums and deal the chunks less evenly.
 static int skinny_waves(int groups, int n_chunks, int max_nw) {
     if (g_skinny_force_nw) return g_skinny_force_nw <= max_nw ? g_skinny_force_nw : max_nw;
     int nw = 4;
-    while (nw < max_nw && (long)groups * nw < 2048 && nw < n_chunks) nw *= 2;
+    while (nw < max_nw && (long)groups * nw < 640 && nw < n_chunks) nw *= 2;
     return nw;
 }
 
-template <int R, int MT, int EPI, typename TC>
+template <int R, int MT, int EPI, typename TC, int XR>
 static void launch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                           int NB, hipStream_t stream) {
     constexpr int KS = MT <= 2 ? 4 : 2;
@@ -260,11 +295,11 @@ static void launch_skinny(const void* X, long ldx, const void* Wp, void* Y, long
     const int groups = (NB + R - 1) / R;
     const int nw = skinny_waves(groups, n_chunks, MAX_NW);
     if (nw == 16) {
-        if constexpr (MAX_NW >= 16) launch_skinny_nw<R, MT, EPI, 16, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        if constexpr (MAX_NW >= 16) launch_skinny_nw<R, MT, EPI, 16, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     } else if (nw == 8) {
-        if constexpr (MAX_NW >= 8) launch_skinny_nw<R, MT, EPI, 8, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        if constexpr (MAX_NW >= 8) launch_skinny_nw<R, MT, EPI, 8, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     } else {
-        launch_skinny_nw<R, MT, EPI, 4, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        launch_skinny_nw<R, MT, EPI, 4, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     }
 }
 
@@ -281,11 +316,16 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
     if (g_skinny_force_r) r = g_skinny_force_r;
     if (mt <= 1 && r > 2) r = 2;
 #define SK_CASE(R_, MT_)                                                                        \
-    launch_skinny<R_, MT_, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);              \
+    launch_skinny<R_, MT_, EPI, TC, 16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);          \
+    break
+#define SK_CASE1(R_)                                                                            \
+    if (M <= 4) launch_skinny<R_, 1, EPI, TC, 4>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream); \
+    else if (M <= 8) launch_skinny<R_, 1, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream); \
+    else launch_skinny<R_, 1, EPI, TC, 16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);       \
     break
     switch (mt * 8 + r) {
-        case 1 * 8 + 1: SK_CASE(1, 1);
-        case 1 * 8 + 2: SK_CASE(2, 1);
+        case 1 * 8 + 1: SK_CASE1(1);
+        case 1 * 8 + 2: SK_CASE1(2);
         case 2 * 8 + 1: SK_CASE(1, 2);
         case 2 * 8 + 2: SK_CASE(2, 2);
         case 2 * 8 + 4: SK_CASE(4, 2);
@@ -297,6 +337,7 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
         case 4 * 8 + 4: SK_CASE(4, 4);
         default: AGAVE_CHECK(false, "gemm_skinny: no kernel for %d tokens with %d row blocks a workgroup", M, r);
     }
+#undef SK_CASE1
 #undef SK_CASE
     return 0;
 }
