@@ -20,6 +20,7 @@
 // after S^T = K * Q^T, so probabilities go into the P*V product without leaving their lane.
 #include "common_impl.h"
 #include "mfma.h"
+#include "qk_rope.h"
 #include <math.h>
 
 #define QT_MAX 4        // most q tiles (of 16 query slots) a wave takes
@@ -47,6 +48,21 @@ struct AttnArgs {
     int splits, pages_per_split;
     int seq_is_token;    // decode: sequence index == token index
     int table_from_reach; // decode: each table row starts at the first page its token reaches (base[b] == lo / 64)
+};
+
+// What the decode kernel needs to do the q/k head norm, the rotation and the cache write of
+// the step's own token itself (then AttnArgs::q holds the raw projection).
+struct QkFuse {
+    const bf16* k_raw;   // null: this run appends nothing
+    long ldk;
+    const bf16* v_raw;
+    long ldv;
+    const float* q_gain; // null: no norm
+    const float* k_gain;
+    float eps_q, eps_k;
+    const float* inv_freq;
+    int rot_half;
+    float pos_scale;
 };
 
 // One wave: QT tiles of 16 query slots against the pages [page_lo, page_hi] of one sequence
@@ -293,10 +309,16 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(AttnArgs a) {
 // reference stays: probabilities are bounded by 2^8, which 32-bit sums and bfloat16 operands
 // hold without loss), and masks are applied only to units that touch the ends of the range.
 #define LAZY_LOG2 8.0f
-template <int HDT>
-__global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a) {
+// FUSED: q arrives as the raw projection; the workgroup normalises and rotates its heads' queries
+// itself, and the workgroup whose range holds the token's own position does the same for the key,
+// writes key and value into their page and only then reads pages (its own stores are visible to
+// it after a workgroup barrier; no other workgroup of this launch reads that row, except those
+// of other head chunks of the same kv head, which write the same bytes themselves).
+template <int HDT, bool FUSED>
+__global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFuse f) {
     constexpr int KS = HDT / 2;
-    extern __shared__ float lds[];            // [4 waves][slots][hd] outputs, then [4][16][2] (max, sum)
+    extern __shared__ float lds[];            // [4 waves][slots][hd] outputs, then [4][16][2] (max, sum);
+                                              // FUSED: then [4][hd] floats and [16][hd] bf16 for the queries
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
     const int G = a.nh / a.nkv;
     const int chunks = (G + 15) / 16;
@@ -318,12 +340,54 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a) {
 
     // queries of this chunk's heads: B operand of S^T = K Q^T
     frag16 qf[KS];
-    {
+    if constexpr (!FUSED) {
         const bool col_ok = j < slots;
         const bf16* qrow = a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + j) * hd;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             if (col_ok) qf[ks].u = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * g);
+            else qf[ks].u = uint4{0, 0, 0, 0};
+        }
+    } else {
+        float* ybuf = lds + (size_t)4 * slots * hd + 4 * 16 * 2 + (size_t)wave * hd;
+        bf16* q_s = reinterpret_cast<bf16*>(lds + (size_t)4 * slots * hd + 4 * 16 * 2 + (size_t)4 * hd);
+        const float pf = (float)p * f.pos_scale;
+        // the token's own key and value go into the page of position p, by the workgroup that reads it
+        const bool writer = f.k_raw != nullptr && page_lo <= last && page_hi == last;
+        const int jobs = slots + (writer ? 1 : 0);
+        for (int job0 = 0; job0 < jobs; job0 += 4) {
+            const int job = job0 + wave;
+            const bool active = job < jobs, is_q = job < slots;
+            const bf16* src = is_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + (active ? job : 0)) * hd
+                                   : f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd;
+            qk_norm_rope_wave<bf16>(src, ybuf, is_q ? f.q_gain : f.k_gain, is_q ? f.eps_q : f.eps_k, f.inv_freq,
+                                    f.rot_half, pf, hd, lane, active);
+            if (active && is_q) {
+                for (int d = lane; d < hd; d += 64) q_s[job * hd + d] = f32_to_bf16(ybuf[d]);
+            } else if (active) {
+                long wpg;
+                if (a.table_from_reach) {
+                    const int col = last - first;
+                    wpg = col < a.width ? a.table[(size_t)b * a.width + col] : -1;
+                    if (wpg >= a.n_pages) wpg = -1;
+                } else {
+                    wpg = page_of(a, b, last);
+                }
+                if (wpg >= 0) {
+                    bf16* dk = (bf16*)(a.k_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)4 * KS * 64));
+                    bf16* dv = (bf16*)(a.v_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)HDT * 2 * 64));
+                    store_kv_row_packed<bf16>(dk, dv, ybuf, f.v_raw + (size_t)t * f.ldv + (size_t)kvh * hd,
+                                              p % AGAVE_PAGE, hd, lane);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        const bool col_ok = j < slots;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (col_ok) qf[ks].u = *reinterpret_cast<const uint4*>(q_s + j * hd + 32 * ks + 8 * g);
             else qf[ks].u = uint4{0, 0, 0, 0};
         }
     }
@@ -645,6 +709,52 @@ static int check_common(const char* who, const AttnArgs& a, int N) {
     return 0;
 }
 
+// FUSED: a.q is the raw q projection and f says how to normalise and rotate it (head sizes 64, 128, 256 only).
+template <bool FUSED>
+static int launch_decode(const AttnArgs& a, const QkFuse& f, int N, hipStream_t stream) {
+    const int nh = a.nh, nkv = a.nkv, hd = a.hd, splits = a.splits;
+    AGAVE_CHECK(splits >= 1 && splits <= COMBINE_MAX_SPLITS && a.pages_per_split >= 1, "attn_decode_mfma: bad split plan %d x %d", splits, a.pages_per_split);
+    AGAVE_CHECK(splits == 1 || (a.part_o && a.part_ml), "attn_decode_mfma: splits need the partial buffers");
+    AGAVE_CHECK(N <= 65535, "attn_decode_mfma: %d tokens exceed the grid limit", N);
+    if (N == 0) return 0;
+    const int G = nh / nkv;
+    dim3 grid(splits, nkv * ((G + 15) / 16), N);
+    const int slots = G < 16 ? G : 16;
+    size_t lds = ((size_t)4 * slots * hd + 4 * 16 * 2) * sizeof(float);
+    if (FUSED) lds += (size_t)4 * hd * sizeof(float) + (size_t)16 * hd * sizeof(bf16);
+    AGAVE_CHECK(lds <= 96 * 1024, "attn_decode_mfma: %zu bytes of LDS exceed what a workgroup may take", lds);
+    static bool raised = false;
+    if (!raised) {               // more than the default allowance of LDS for large groups of heads
+        const void* fns[] = {(const void*)attn_decode_mfma_kernel<4>, (const void*)attn_decode_mfma_kernel<8>,
+                             (const void*)attn_decode_mfma_kernel<16>,
+                             (const void*)attn_decode_fast_kernel<4, false>, (const void*)attn_decode_fast_kernel<8, false>,
+                             (const void*)attn_decode_fast_kernel<16, false>,
+                             (const void*)attn_decode_fast_kernel<4, true>, (const void*)attn_decode_fast_kernel<8, true>,
+                             (const void*)attn_decode_fast_kernel<16, true>};
+        for (const void* fn : fns)
+            AGAVE_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) == hipSuccess,
+                        "attn_decode_mfma: cannot raise the LDS allowance");
+        raised = true;
+    }
+    if (FUSED) {
+        AGAVE_CHECK(hd == 64 || hd == 128 || hd == 256, "attn_decode_fused: head_dim %d is not 64, 128 or 256", hd);
+        if (hd == 64) attn_decode_fast_kernel<4, true><<<grid, 256, lds, stream>>>(a, f);
+        else if (hd == 128) attn_decode_fast_kernel<8, true><<<grid, 256, lds, stream>>>(a, f);
+        else attn_decode_fast_kernel<16, true><<<grid, 256, lds, stream>>>(a, f);
+    } else if (hd == 64) attn_decode_fast_kernel<4, false><<<grid, 256, lds, stream>>>(a, f);
+    else if (hd == 128) attn_decode_fast_kernel<8, false><<<grid, 256, lds, stream>>>(a, f);
+    else if (hd == 256) attn_decode_fast_kernel<16, false><<<grid, 256, lds, stream>>>(a, f);
+    else if (hd <= 64) attn_decode_mfma_kernel<4><<<grid, 256, lds, stream>>>(a);
+    else if (hd <= 128) attn_decode_mfma_kernel<8><<<grid, 256, lds, stream>>>(a);
+    else attn_decode_mfma_kernel<16><<<grid, 256, lds, stream>>>(a);
+    AGAVE_LAUNCH_CHECK("attn_decode_mfma");
+    if (splits > 1) {
+        attn_combine_kernel<<<N * nh, hd >= 256 ? 256 : (hd >= 128 ? 128 : 64), 0, stream>>>(a.part_o, a.part_ml, a.out, a.ldo, nh, hd, splits);
+        AGAVE_LAUNCH_CHECK("attn_combine");
+    }
+    return 0;
+}
+
 extern "C" int agave_attn_decode_mfma(const void* q, long ldq, void* out, long ldo, float* part_o, float* part_ml,
                                       const void* k_pages, const void* v_pages, const int* table, int width,
                                       const int* base, int n_pages, const int* tok_seq, const int* tok_pos, int N,
@@ -655,39 +765,29 @@ extern "C" int agave_attn_decode_mfma(const void* q, long ldq, void* out, long l
                table, width, base, n_pages, tok_seq, tok_pos, nullptr, 0, nh, nkv, hd, scale, window, splits,
                pages_per_split, seq_is_token, table_from_reach};
     if (check_common("attn_decode_mfma", a, N)) return -1;
-    AGAVE_CHECK(splits >= 1 && splits <= COMBINE_MAX_SPLITS && pages_per_split >= 1, "attn_decode_mfma: bad split plan %d x %d", splits, pages_per_split);
-    AGAVE_CHECK(splits == 1 || (part_o && part_ml), "attn_decode_mfma: splits need the partial buffers");
-    AGAVE_CHECK(N <= 65535, "attn_decode_mfma: %d tokens exceed the grid limit", N);
-    if (N == 0) return 0;
-    const int G = nh / nkv;
-    dim3 grid(splits, nkv * ((G + 15) / 16), N);
-    const int slots = G < 16 ? G : 16;
-    const size_t lds = ((size_t)4 * slots * hd + 4 * 16 * 2) * sizeof(float);
-    AGAVE_CHECK(lds <= 96 * 1024, "attn_decode_mfma: %zu bytes of LDS exceed what a workgroup may take", lds);
-    if (lds > 48 * 1024) {       // more than the default allowance: ask for it (once per kernel would do)
-        hipError_t e1 = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        hipError_t e2 = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        hipError_t e3 = hipFuncSetAttribute((const void*)attn_decode_mfma_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        AGAVE_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "attn_decode_mfma: cannot raise the LDS allowance");
-    }
-    if (lds > 48 * 1024) {
-        hipError_t e1 = hipFuncSetAttribute((const void*)attn_decode_fast_kernel<4>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        hipError_t e2 = hipFuncSetAttribute((const void*)attn_decode_fast_kernel<8>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        hipError_t e3 = hipFuncSetAttribute((const void*)attn_decode_fast_kernel<16>, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
-        AGAVE_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "attn_decode_mfma: cannot raise the LDS allowance");
-    }
-    if (hd == 64) attn_decode_fast_kernel<4><<<grid, 256, lds, stream>>>(a);
-    else if (hd == 128) attn_decode_fast_kernel<8><<<grid, 256, lds, stream>>>(a);
-    else if (hd == 256) attn_decode_fast_kernel<16><<<grid, 256, lds, stream>>>(a);
-    else if (hd <= 64) attn_decode_mfma_kernel<4><<<grid, 256, lds, stream>>>(a);
-    else if (hd <= 128) attn_decode_mfma_kernel<8><<<grid, 256, lds, stream>>>(a);
-    else attn_decode_mfma_kernel<16><<<grid, 256, lds, stream>>>(a);
-    AGAVE_LAUNCH_CHECK("attn_decode_mfma");
-    if (splits > 1) {
-        attn_combine_kernel<<<N * nh, hd >= 256 ? 256 : (hd >= 128 ? 128 : 64), 0, stream>>>(part_o, part_ml, (bf16*)out, ldo, nh, hd, splits);
-        AGAVE_LAUNCH_CHECK("attn_combine");
-    }
-    return 0;
+    return launch_decode<false>(a, QkFuse{}, N, stream);
+}
+
+// Decode attention that first does the q/k head norm, the rotation and the cache write of each
+// sequence's new token (one token per sequence, positions tok_pos): q, k, v are the raw
+// projections; k and v null for a run that appends nothing.
+extern "C" int agave_attn_decode_fused(const void* q, long ldq, const void* k, long ldk, const void* v, long ldv,
+                                       const float* q_gain, const float* k_gain, float eps_q, float eps_k,
+                                       const float* inv_freq, int rot_half, float pos_scale, void* out, long ldo,
+                                       float* part_o, float* part_ml, void* k_pages, void* v_pages, const int* table,
+                                       int width, const int* base, int n_pages, const int* tok_seq,
+                                       const int* tok_pos, int N, int nh, int nkv, int hd, float scale, int window,
+                                       int splits, int pages_per_split, int seq_is_token, int table_from_reach,
+                                       hipStream_t stream) {
+    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
+               table, width, base, n_pages, tok_seq, tok_pos, nullptr, 0, nh, nkv, hd, scale, window, splits,
+               pages_per_split, seq_is_token, table_from_reach};
+    if (check_common("attn_decode_fused", a, N)) return -1;
+    AGAVE_CHECK((k == nullptr) == (v == nullptr), "attn_decode_fused: k and v come together");
+    AGAVE_CHECK(!k || (ldk >= (long)nkv * hd && ldv >= (long)nkv * hd), "attn_decode_fused: a k or v row stride is below nkv*hd");
+    AGAVE_CHECK(rot_half >= 0 && 2 * rot_half <= hd && (rot_half == 0 || inv_freq), "attn_decode_fused: bad rotation (rotary_dim %d, head_dim %d)", 2 * rot_half, hd);
+    QkFuse f{(const bf16*)k, ldk, (const bf16*)v, ldv, q_gain, k_gain, eps_q, eps_k, inv_freq, rot_half, pos_scale};
+    return launch_decode<true>(a, f, N, stream);
 }
 
 extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long ldo, const void* k_pages,

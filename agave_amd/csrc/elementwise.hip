@@ -7,6 +7,7 @@
 // src/backend/kernels/cpu/rope.zig:11-48 (split-half pairs), src/models/gemma3.zig:884-902
 // (position scaled before the angle), src/backend/kernels/cpu/activation.zig:69-113 (tanh GELU).
 #include "common_impl.h"
+#include "qk_rope.h"
 
 // ------------------------------------------------------------------ embedding
 template <typename T>
@@ -245,31 +246,8 @@ __global__ void qk_norm_rope_kv_kernel(const T* q, long ldq, const T* __restrict
     const float eps = is_q ? eps_q : eps_k;
     float* y = buf[wave];
 
-    float ss = 0.f;
-    if (active)
-        for (int d = lane; d < hd; d += 64) {
-            const float x = ld(src + d);
-            y[d] = x;
-            ss += x * x;
-        }
-    if (active && gain) {
-        ss = wave_sum(ss);
-        const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
-        for (int d = lane; d < hd; d += 64) y[d] = y[d] * inv * gain[d];
-    }
-    __syncthreads();
-
     const int p = active ? tok_pos[t] : 0;
-    const float pf = (float)p * pos_scale;
-    // rotation, in place in LDS: y[i], y[i + rot_half] <- rotated pair
-    for (int i = lane; active && i < rot_half; i += 64) {
-        const float a = y[i], b2 = y[i + rot_half];
-        float s, c;
-        sincosf(pf * inv_freq[i], &s, &c);
-        y[i] = a * c - b2 * s;
-        y[i + rot_half] = a * s + b2 * c;
-    }
-    __syncthreads();
+    qk_norm_rope_wave<T>(src, y, gain, eps, inv_freq, rot_half, (float)p * pos_scale, hd, lane, active);
     if (!active) return;
     if (is_q) {
         T* dst = q_out + (size_t)t * ldqo + (size_t)head * hd;
@@ -295,15 +273,7 @@ __global__ void qk_norm_rope_kv_kernel(const T* q, long ldq, const T* __restrict
         const int ks_n = (hd + 31) >> 5;
         T* dk = k_pages + ((size_t)pg * nkv + head) * (size_t)(AGAVE_PAGE * ks_n * 32);
         T* dv = v_pages + ((size_t)pg * nkv + head) * (size_t)hd * AGAVE_PAGE;
-        const int kt = row >> 4, ki = row & 15;
-        const int s2 = row >> 5, r32 = row & 31;
-        const int vg = (r32 & 15) >> 2, ve = (r32 & 3) + ((r32 >> 4) << 2);
-        for (int d = lane; d < hd; d += 64) {
-            const int ks = d >> 5, g = (d & 31) >> 3, e = d & 7;
-            st(dk + ((size_t)(kt * ks_n + ks) * 64 + ki + 16 * g) * 8 + e, y[d]);
-            const int dt = d >> 4, j = d & 15;
-            dv[((size_t)(dt * 2 + s2) * 64 + j + 16 * vg) * 8 + ve] = sv[d];
-        }
+        store_kv_row_packed<T>(dk, dv, y, sv, row, hd, lane);
     }
 }
 

@@ -1,0 +1,57 @@
+// Per-head RMSNorm and rotation of one q or k head by one wave, and the place of a cache row in
+// a page that is kept in the matrix cores' tile order.  Shared by the q/k kernel and by the
+// decode attention kernel that does this work itself, so that both leave the same bits.
+#pragma once
+#include "common.h"
+
+// y[0..hd) (LDS, 32-bit) <- rotate(src[0..hd) * rsqrt(mean(src^2) + eps) * gain).
+// gain may be null (no norm), rot_half 0 (no rotation).  pf: position times the position scale.
+// Every wave of the workgroup calls this together (it holds two workgroup barriers); a wave
+// without work passes active = false.
+template <typename T>
+__device__ __forceinline__ void qk_norm_rope_wave(const T* src, float* y, const float* __restrict__ gain, float eps,
+                                                  const float* __restrict__ inv_freq, int rot_half, float pf, int hd,
+                                                  int lane, bool active) {
+    float ss = 0.f;
+    if (active)
+        for (int d = lane; d < hd; d += 64) {
+            const float x = ld(src + d);
+            y[d] = x;
+            ss += x * x;
+        }
+    if (active && gain) {
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
+        for (int d = lane; d < hd; d += 64) y[d] = y[d] * inv * gain[d];
+    }
+    __syncthreads();
+    // rotation, in place in LDS: y[i], y[i + rot_half] <- rotated pair
+    for (int i = lane; active && i < rot_half; i += 64) {
+        const float a = y[i], b2 = y[i + rot_half];
+        float s, c;
+        sincosf(pf * inv_freq[i], &s, &c);
+        y[i] = a * c - b2 * s;
+        y[i + rot_half] = a * s + b2 * c;
+    }
+    __syncthreads();
+}
+
+// One wave writes a key row y[0..hd) (LDS) and a value row sv[0..hd) to row `row` of a page in tile
+// order: dk, dv are the page's K and V blocks of this kv head.
+//   K: tiles [row / 16][d / 32] of 64 lanes x 8: lane (row % 16) + 16 * ((d % 32) / 8), element d % 8
+//   V: tiles [d / 16][row / 32] of 64 lanes x 8: lane (d % 16) + 16 * vg, element ve, with the 32 keys
+//      of a half page in the order the score accumulators have them
+template <typename T>
+__device__ __forceinline__ void store_kv_row_packed(T* dk, T* dv, const float* y, const T* sv, int row, int hd,
+                                                    int lane) {
+    const int ks_n = (hd + 31) >> 5;
+    const int kt = row >> 4, ki = row & 15;
+    const int s2 = row >> 5, r32 = row & 31;
+    const int vg = (r32 & 15) >> 2, ve = (r32 & 3) + ((r32 >> 4) << 2);
+    for (int d = lane; d < hd; d += 64) {
+        const int ks = d >> 5, g = (d & 31) >> 3, e = d & 7;
+        st(dk + ((size_t)(kt * ks_n + ks) * 64 + ki + 16 * g) * 8 + e, y[d]);
+        const int dt = d >> 4, j = d & 15;
+        dv[((size_t)(dt * 2 + s2) * 64 + j + 16 * vg) * 8 + ve] = sv[d];
+    }
+}

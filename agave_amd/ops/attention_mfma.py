@@ -11,6 +11,8 @@ from .kernels import _F, _I, _L, _P
 kernels.register_signatures("attention_mfma", {
     "agave_attn_decode_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _I,
                                _I, _P],
+    "agave_attn_decode_fused": [_P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I,
+                                _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _P],
     "agave_attn_prefill_mfma": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
 })
 
@@ -59,3 +61,51 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
                      k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width, base.data_ptr(), n_pages,
                      step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), step.cu_dev.data_ptr(), step.n_seqs,
                      step.max_new, n, n_heads, n_kv, head_dim, scale, w, kernels.stream())
+
+
+FUSED_HEAD_DIMS = (64, 128, 256)
+
+
+def decode_fused(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], out: torch.Tensor,
+                 q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps_q: float, eps_k: float,
+                 inv_freq: Optional[torch.Tensor], pos_scale: float, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                 table: torch.Tensor, base: torch.Tensor, step, n_heads: int, n_kv: int, head_dim: int, scale: float,
+                 window: Optional[int]) -> None:
+    """A decode step's attention from the raw projections: the kernel normalises and rotates q and
+    k, writes k and v into their pages (``k`` None: nothing is appended) and attends."""
+    n = step.n_tokens
+    if not step.is_decode or head_dim not in FUSED_HEAD_DIMS:
+        raise ValueError("decode_fused: needs a decode step and a head size of 64, 128 or 256")
+    for name, t, cols in (("q", q, n_heads * head_dim), ("k", k, n_kv * head_dim), ("v", v, n_kv * head_dim),
+                          ("out", out, n_heads * head_dim)):
+        if t is None:
+            continue
+        if not t.is_cuda or t.dtype != torch.bfloat16 or t.shape != (n, cols) or t.stride(1) != 1:
+            raise ValueError(f"decode_fused: {name} must be bfloat16 [{n}, {cols}] on the GPU with contiguous rows")
+    if (k is None) != (v is None):
+        raise ValueError("decode_fused: k and v come together")
+    kernels._f32vec(q_gain, "q_gain", head_dim)
+    kernels._f32vec(k_gain, "k_gain", head_dim)
+    rot_half = 0
+    if inv_freq is not None:
+        rot_half = inv_freq.numel()
+        kernels._f32vec(inv_freq, "inv_freq", rot_half)
+    kernels._dev(q, k, v, out, q_gain, k_gain, inv_freq, k_pages, v_pages, table, base)
+    n_pages = kernels._check_pages(k_pages, v_pages, n_kv, head_dim, q.dtype, packed=True)
+    width = kernels._check_table(table, base, step.tok_seq)
+    span = step.page_span(window)
+    chunks = -(-(n_heads // n_kv) // 16)
+    splits, per = split_plan(span, n * n_kv * chunks)
+    part_o = part_ml = None
+    if splits > 1:
+        ws = step.workspace
+        part_o = ws.get("attn_part_o", n * n_heads * splits, head_dim, torch.float32)
+        part_ml = ws.get("attn_part_ml", n * n_heads * splits, 2, torch.float32)
+    library.call(kernels.lib("attention_mfma"), "agave_attn_decode_fused", q.data_ptr(), q.stride(0),
+                 kernels.ptr(k), k.stride(0) if k is not None else 0, kernels.ptr(v),
+                 v.stride(0) if v is not None else 0, kernels.ptr(q_gain), kernels.ptr(k_gain), eps_q, eps_k,
+                 kernels.ptr(inv_freq), rot_half, pos_scale, out.data_ptr(), out.stride(0), kernels.ptr(part_o),
+                 kernels.ptr(part_ml), k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width,
+                 base.data_ptr(), n_pages, step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), n, n_heads, n_kv,
+                 head_dim, scale, int(window or 0), splits, per, 1 if step.n_seqs == n else 0,
+                 1 if getattr(step, "tables_start_at_reach", False) else 0, kernels.stream())

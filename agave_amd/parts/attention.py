@@ -66,10 +66,12 @@ class Attention:
         q_out = ws.get("q_rot", n, self.qd, x.dtype)
         qg, kg = (self.q_norm.gain if self.q_norm else None), (self.k_norm.gain if self.k_norm else None)
         qe, ke = (self.q_norm.eps if self.q_norm else 0.0), (self.k_norm.eps if self.k_norm else 0.0)
+        ctx_out = ws.get("attn_ctx", n, self.qd, x.dtype)
         if fused is not None:
             inv_freq, pos_scale = fused()
-            kernels.qk_norm_rope_kv(q, k, v, q_out, qg, kg, qe, ke, inv_freq, pos_scale, step.tok_seq, step.tok_pos,
-                                    k_pages, v_pages, table, base, s.n_heads, s.n_kv_heads, s.head_dim, packed)
+            attn_ops.qk_attention(q, k, v, q_out, ctx_out, qg, kg, qe, ke, inv_freq, pos_scale, k_pages, v_pages,
+                                  table, base, step, s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, packed)
+            return self.o.forward(ctx_out, tag="attn_o")
         else:
             # a position encoding the q/k kernel does not know: the norms, then the part's own
             # ``apply`` on the normalised rows, then the cache write
@@ -85,7 +87,6 @@ class Attention:
                 kernels.qk_norm_rope_kv(None, k_n, v, None, None, None, 0.0, 0.0, None, 1.0, step.tok_seq,
                                         step.tok_pos, k_pages, v_pages, table, base, 0, s.n_kv_heads, s.head_dim,
                                         packed)
-        ctx_out = ws.get("attn_ctx", n, self.qd, x.dtype)
         attn_ops.attention(q_out, ctx_out, k_pages, v_pages, table, base, step, s.n_heads, s.n_kv_heads,
                            s.head_dim, s.scale, s.window, packed)
         return self.o.forward(ctx_out, tag="attn_o")

@@ -522,3 +522,56 @@ def test_embedding_from_a_packed_table(G):
     out = torch.empty(len(toks), 72, dtype=torch.float32, device=DEV)
     G.embed_scale_packed(_i32(toks), packed, math.sqrt(72.0), out, 300)
     assert torch.allclose(out.cpu().double(), P.embed(toks, table.double(), 72), atol=1e-6, rtol=1e-6)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,window,rot", [(8, 4, 256, 64, 128), (4, 2, 64, None, 16), (40, 2, 128, 1000, 64),
+                                                  (2, 2, 128, None, 0)])
+def test_attn_decode_fused_equals_the_two_kernels(K, nh, nkv, hd, window, rot):
+    """The decode kernel that normalises, rotates and caches the new token itself must leave the
+    same bits, in the output and in the cache pages, as the q/k kernel followed by the attention
+    kernel; appending nothing (k None) must leave the pages alone."""
+    from agave_amd.ops import attention as A
+    g = torch.Generator().manual_seed(11)
+    lens = [1, 64, 65, 300, 1500, 128]                  # positions at a page's first and last row among them
+    B = len(lens)
+    n_pages = sum((L + 63) // 64 for L in lens) + 1
+    width = max((L + 63) // 64 for L in lens)
+    perm = torch.randperm(n_pages, generator=g).tolist()
+    table = torch.full((B, width), -1, dtype=torch.int32)
+    for b, L in enumerate(lens):
+        for i in range((L + 63) // 64):
+            table[b, i] = perm.pop()
+    table, base = table.to(DEV), _i32([0] * B)
+    kp0 = torch.randn(n_pages, nkv, 64, hd, generator=g).bfloat16().to(DEV)      # older keys: any values
+    vp0 = torch.randn(n_pages, nkv, hd, 64, generator=g).bfloat16().to(DEV)
+    q = torch.randn(B, nh * hd, generator=g).bfloat16().to(DEV)
+    k = torch.randn(B, nkv * hd, generator=g).bfloat16().to(DEV)
+    v = torch.randn(B, nkv * hd, generator=g).bfloat16().to(DEV)
+    qg = (1 + 0.2 * torch.randn(hd, generator=g)).to(DEV)
+    kg = (1 + 0.2 * torch.randn(hd, generator=g)).to(DEV)
+    inv_freq = torch.exp(-torch.arange(rot).float() / max(rot, 1) * 5).to(DEV) if rot else None
+    step = _FakeStep(lens, lambda L: L - 1, window)
+    scale = 0.3 * (16 / hd) ** 0.5
+    outs = []
+    for fused in (True, False):
+        kp, vp = kp0.clone(), vp0.clone()
+        out = torch.full_like(q, float("nan"))
+        q_rot = torch.empty_like(q)
+        if fused:
+            A.qk_attention(q, k, v, q_rot, out, qg, kg, 1e-5, 2e-6, inv_freq, 0.5, kp, vp, table, base, step,
+                           nh, nkv, hd, scale, window, True)
+        else:
+            K.qk_norm_rope_kv(q, k, v, q_rot, qg, kg, 1e-5, 2e-6, inv_freq, 0.5, step.tok_seq, step.tok_pos, kp, vp,
+                              table, base, nh, nkv, hd, packed=True)
+            A.attention(q_rot, out, kp, vp, table, base, step, nh, nkv, hd, scale, window, True)
+        torch.cuda.synchronize()
+        outs.append((out, kp, vp))
+    assert torch.isfinite(outs[0][0].float()).all()
+    for a, b, what in zip(outs[0], outs[1], ("output", "K pages", "V pages")):
+        assert torch.equal(a, b), what
+    # a run that appends nothing: queries only, pages untouched
+    kp, vp = outs[1][1].clone(), outs[1][2].clone()
+    out = torch.full_like(q, float("nan"))
+    A.qk_attention(q, None, None, torch.empty_like(q), out, qg, kg, 1e-5, 2e-6, inv_freq, 0.5, kp, vp, table, base,
+                   step, nh, nkv, hd, scale, window, True)
+    assert torch.equal(out, outs[1][0]) and torch.equal(kp, outs[1][1]) and torch.equal(vp, outs[1][2])
