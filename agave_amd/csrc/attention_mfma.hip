@@ -348,48 +348,6 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
             if (col_ok) qf[ks].u = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * g);
             else qf[ks].u = uint4{0, 0, 0, 0};
         }
-    } else {
-        float* ybuf = lds + (size_t)4 * slots * hd + 4 * 16 * 2 + (size_t)wave * hd;
-        bf16* q_s = reinterpret_cast<bf16*>(lds + (size_t)4 * slots * hd + 4 * 16 * 2 + (size_t)4 * hd);
-        const float pf = (float)p * f.pos_scale;
-        // the token's own key and value go into the page of position p, by the workgroup that reads it
-        const bool writer = f.k_raw != nullptr && page_lo <= last && page_hi == last;
-        const int jobs = slots + (writer ? 1 : 0);
-        for (int job0 = 0; job0 < jobs; job0 += 4) {
-            const int job = job0 + wave;
-            const bool active = job < jobs, is_q = job < slots;
-            const bf16* src = is_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + (active ? job : 0)) * hd
-                                   : f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd;
-            qk_norm_rope_wave<bf16>(src, ybuf, is_q ? f.q_gain : f.k_gain, is_q ? f.eps_q : f.eps_k, f.inv_freq,
-                                    f.rot_half, pf, hd, lane, active);
-            if (active && is_q) {
-                for (int d = lane; d < hd; d += 64) q_s[job * hd + d] = f32_to_bf16(ybuf[d]);
-            } else if (active) {
-                long wpg;
-                if (a.table_from_reach) {
-                    const int col = last - first;
-                    wpg = col < a.width ? a.table[(size_t)b * a.width + col] : -1;
-                    if (wpg >= a.n_pages) wpg = -1;
-                } else {
-                    wpg = page_of(a, b, last);
-                }
-                if (wpg >= 0) {
-                    bf16* dk = (bf16*)(a.k_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)4 * KS * 64));
-                    bf16* dv = (bf16*)(a.v_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)HDT * 2 * 64));
-                    store_kv_row_packed<bf16>(dk, dv, ybuf, f.v_raw + (size_t)t * f.ldv + (size_t)kvh * hd,
-                                              p % AGAVE_PAGE, hd, lane);
-                }
-            }
-        }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __syncthreads();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-        const bool col_ok = j < slots;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            if (col_ok) qf[ks].u = *reinterpret_cast<const uint4*>(q_s + j * hd + 32 * ks + 8 * g);
-            else qf[ks].u = uint4{0, 0, 0, 0};
-        }
     }
     f32x4_t o[HDT];
 #pragma unroll
@@ -431,6 +389,58 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     if (have) {
         kp = (const u32x4_t*)(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride);
         vp = (const u32x4_t*)(a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride);
+    }
+    // FUSED: the token's own key and value go into the page of position p, by the workgroup that
+    // reads it; the wave whose first page that is waits with its loads until the row is there
+    const bool writer = FUSED && f.k_raw != nullptr && page_lo <= last && page_hi == last;
+    const bool early = !(writer && page_lo + wave == last);
+    if (have && early) {
+        load_k(0);
+        load_v(0);
+    }
+    if constexpr (FUSED) {
+        float* ybuf = lds + (size_t)4 * slots * hd + 4 * 16 * 2 + (size_t)wave * hd;
+        bf16* q_s = reinterpret_cast<bf16*>(lds + (size_t)4 * slots * hd + 4 * 16 * 2 + (size_t)4 * hd);
+        const float pf = (float)p * f.pos_scale;
+        // the token's own key and value go into the page of position p, by the workgroup that reads it
+        const int jobs = slots + (writer ? 1 : 0);
+        for (int job0 = 0; job0 < jobs; job0 += 4) {
+            const int job = job0 + wave;
+            const bool active = job < jobs, is_q = job < slots;
+            const bf16* src = is_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + (active ? job : 0)) * hd
+                                   : f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd;
+            qk_norm_rope_wave<bf16>(src, ybuf, is_q ? f.q_gain : f.k_gain, is_q ? f.eps_q : f.eps_k, f.inv_freq,
+                                    f.rot_half, pf, hd, lane, active);
+            if (active && is_q) {
+                for (int d = lane; d < hd; d += 64) q_s[job * hd + d] = f32_to_bf16(ybuf[d]);
+            } else if (active) {
+                long wpg;
+                if (a.table_from_reach) {
+                    const int col = last - first;
+                    wpg = col < a.width ? a.table[(size_t)b * a.width + col] : -1;
+                    if (wpg >= a.n_pages) wpg = -1;
+                } else {
+                    wpg = page_of(a, b, last);
+                }
+                if (wpg >= 0) {
+                    bf16* dk = (bf16*)(a.k_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)4 * KS * 64));
+                    bf16* dv = (bf16*)(a.v_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)HDT * 2 * 64));
+                    store_kv_row_packed<bf16>(dk, dv, ybuf, f.v_raw + (size_t)t * f.ldv + (size_t)kvh * hd,
+                                              p % AGAVE_PAGE, hd, lane);
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        const bool col_ok = j < slots;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (col_ok) qf[ks].u = *reinterpret_cast<const uint4*>(q_s + j * hd + 32 * ks + 8 * g);
+            else qf[ks].u = uint4{0, 0, 0, 0};
+        }
+    }
+    if (have && !early) {
         load_k(0);
         load_v(0);
     }
