@@ -369,8 +369,12 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
 
 
 // ------------------------------------------------------------------ tiled product (prefill)
-// A workgroup of four waves (2 x 2) computes WT*64 weight rows x 256 tokens; a wave WT x 4
-// tiles of 32 x 32 (v_mfma_f32_32x32x16_bf16).  Both operands come into LDS straight from
+// A workgroup computes WT*64 weight rows x 256 tokens in tiles of 32 x 32
+// (v_mfma_f32_32x32x16_bf16): four waves (2 x 2, a wave WT x 4 tiles) or eight (2 x 4, a wave
+// WT x 2 tiles).  Eight waves are two per SIMD: while one waits for a stage of loads or at the
+// barrier the other multiplies, which a single wave per SIMD cannot hide (a third of its time
+// was waiting); they read a half more from LDS per flop, which the LDS has to spare.
+// Both operands come into LDS straight from
 // global memory (no registers in between), KT k-steps of 32 columns per stage, in a ring of
 // NS buffers: the loads of NS-1 stages ahead are in flight while a stage is multiplied.
 // Weight tiles arrive in their packed order (one kilobyte per wave load; a 32-row operand is
@@ -382,8 +386,8 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
 // the number of row tiles apart) tend to land on the same XCD and find them in its L2.
 typedef __attribute__((address_space(3))) u32x4_t tl_lds_u32x4;
 
-template <int WT, int KT, int NS, int EPI, typename TC>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
+template <int WT, int KT, int NS, int EPI, typename TC, int NWV>
+__global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
                                                          const uint4* __restrict__ Wp, TC* __restrict__ Y, long ldy,
                                                          int M, int N, int K, int KB, int NB) {
     constexpr int CPR = KT * 4;                       // 16-byte pieces per staged token row
@@ -391,7 +395,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     constexpr int WTILES = 4 * WT;                    // packed 16-row weight tiles per workgroup
     constexpr int X_BYTES = 256 * KT * 64, W_BYTES = WTILES * KT * 1024;
     constexpr int STAGE_BYTES = X_BYTES + W_BYTES;
-    constexpr int X_LOADS = X_BYTES / 1024 / 4, W_LOADS = W_BYTES / 1024 / 4;     // per wave and stage
+    constexpr int XB = 16 / NWV;                      // 32-token tiles per wave: 4 (four waves, 2 x 2) or 2 (eight, 2 x 4)
+    constexpr int X_LOADS = X_BYTES / 1024 / NWV, W_LOADS = W_BYTES / 1024 / NWV;     // per wave and stage
+    static_assert(NWV == 4 || NWV == 8, "four or eight waves");
+    static_assert(X_LOADS * NWV * 1024 == X_BYTES && W_LOADS * NWV * 1024 == W_BYTES, "whole loads per wave");
     constexpr int LOADS = X_LOADS + W_LOADS;
     static_assert(LOADS * (NS - 2) < 64, "the load counter holds 6 bits");
     extern __shared__ __attribute__((aligned(16))) unsigned char tl_lds[];
@@ -402,11 +409,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     const int n_stage = (KB + KT - 1) / KT;
     const int i32 = lane & 31, kg = lane >> 5;
 
-    f32x16_t acc[WT][4];
+    f32x16_t acc[WT][XB];
 #pragma unroll
     for (int a = 0; a < WT; ++a)
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
+        for (int b = 0; b < XB; ++b)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
@@ -469,8 +476,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
                 wf[a].r = *(const tl_lds_u32x4*)(buf + X_BYTES + (nt * KT + ks) * 1024 + ((i32 & 15) + 16 * (2 * h + kg)) * 16);
             }
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                const int row = (wm * 4 + b) * 32 + i32;
+            for (int b = 0; b < XB; ++b) {
+                const int row = (wm * XB + b) * 32 + i32;
                 frag16 xb;
                 xb.r = *(const tl_lds_u32x4*)(buf + row * (CPR * 16) + (((k16 * 2 + kg) ^ ((row / RP) % CPR)) * 16));
 #pragma unroll
@@ -483,8 +490,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
 #pragma unroll
     for (int a = 0; a < WT; ++a) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const int m = m0 + (wm * 4 + b) * 32 + i32;
+        for (int b = 0; b < XB; ++b) {
+            const int m = m0 + (wm * XB + b) * 32 + i32;
             if (m >= M) continue;
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
@@ -520,7 +527,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
     }
 }
 
-template <int WT, int KT, int NS, int EPI, typename TC>
+template <int WT, int KT, int NS, int EPI, typename TC, int NWV>
 static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB, int NB,
                         hipStream_t stream) {
     constexpr int WTILES = 4 * WT;
@@ -529,13 +536,20 @@ static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long l
     AGAVE_CHECK(grid.y <= 65535, "gemm_tiled: M=%d exceeds the grid limit", M);
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         AGAVE_CHECK(e == hipSuccess, "gemm_tiled: cannot raise the LDS allowance");
         raised = true;
     }
-    gemm_tiled_kernel<WT, KT, NS, EPI, TC><<<grid, 256, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
+    gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
                                                                       M, N, K, KB, NB);
+    return 0;
+}
+
+// A configuration forced from outside (0: the rule below); for measurements only.
+static int g_tiled_force = 0;
+extern "C" int agave_gemm_tiled_tune(int which) {
+    g_tiled_force = which;
     return 0;
 }
 
@@ -544,8 +558,12 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
                           int NB, hipStream_t stream) {
     // the larger tile once it still gives every compute unit two workgroups
     const long big = (long)((NB + 15) / 16) * ((M + 255) / 256);
-    if (big >= 512) return launch_tiled<4, 1, 4, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-    return launch_tiled<2, 2, 3, EPI, TC>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    if (g_tiled_force == 1) return launch_tiled<4, 1, 4, EPI, TC, 4>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    if (g_tiled_force == 2) return launch_tiled<2, 2, 3, EPI, TC, 4>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    if (g_tiled_force == 3) return launch_tiled<4, 1, 4, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    if (g_tiled_force == 4) return launch_tiled<2, 2, 3, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    if (big >= 512) return launch_tiled<4, 1, 4, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    return launch_tiled<2, 2, 3, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
 }
 
 extern "C" int agave_gemm_tiled(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,
