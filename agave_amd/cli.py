@@ -48,6 +48,7 @@ def build_parser() -> argparse.ArgumentParser:
                     help="prefill chunk size in tokens; 0 = whole prompts in one step [default: 0]")
     ap.add_argument("--json", action="store_true", help="output results as JSON (implies --quiet)")
     ap.add_argument("--model-info", action="store_true", help="print model metadata and exit (supports --json)")
+    ap.add_argument("--profile", action="store_true", help="profile per-op timing (lowers throughput)")
     ap.add_argument("-q", "--quiet", action="store_true", help="suppress stats (raw output only)")
     ap.add_argument("-V", "--verbose", action="store_true", help="show technical details")
     ap.add_argument("-v", "--version", action="store_true", help="print version and exit")
@@ -138,9 +139,18 @@ def main(argv: Optional[List[str]] = None) -> int:
                             ignore_eos=args.ignore_eos)
     stats = GenerationStats()
     engine.prefill_chunk = max(0, args.prefill_batch_size)
+    if args.profile:
+        engine.enable_profiling()
     results = engine.generate(prompts, params, stats=stats)
+    table = engine.profile_table() if args.profile else None
+    if table is not None and not args.json:
+        whole = sum(r[2] for r in table) or 1.0
+        print(f"{'op':32s} {'calls':>8s} {'ms':>10s} {'%':>6s}", file=sys.stderr)
+        for name, calls, ms in table:
+            print(f"{name:32s} {calls:8d} {ms:10.3f} {100 * ms / whole:6.1f}", file=sys.stderr)
     if args.json:
-        print(json.dumps({
+        extra = {"profile": [{"op": n, "calls": c, "ms": round(ms, 3)} for n, c, ms in table]} if table else {}
+        print(json.dumps({**extra,
             "outputs": [{"request": r.request, "tokens": r.tokens, "finish_reason": r.finish_reason,
                          "prompt_tokens": r.prompt_tokens} for r in results],
             "tokens": stats.tokens, "tok_per_sec": round(stats.tok_per_sec, 2),

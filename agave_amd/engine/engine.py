@@ -127,6 +127,21 @@ class Engine:
     def kv_seq_len(self, slot: int) -> int:
         return self.cache.length(slot)
 
+    def enable_profiling(self, on: bool = True) -> None:
+        """Time every kernel call by class (``profile_table``).  Steps run eagerly meanwhile, with
+        two events around each call, so throughput drops (the reference's ``--profile``,
+        ``src/main.zig:381, 1516``)."""
+        from ..ops import library
+        library.profile.enabled = bool(on)
+        library.profile.reset()
+        self._graphs_before_profiling = getattr(self, "_graphs_before_profiling", self.use_graphs)
+        self.use_graphs = False if on else self._graphs_before_profiling
+
+    def profile_table(self):
+        """(op, calls, total ms) rows by falling time."""
+        from ..ops import library
+        return library.profile.table()
+
     # ------------------------------------------------------------------ slots and steps
     def alloc_slot(self) -> int:
         return self.cache.alloc_slot()

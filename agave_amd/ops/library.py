@@ -188,8 +188,45 @@ def loaded_paths() -> List[str]:
     return [lib._name for lib in _loaded.values()]
 
 
+class OpProfile:
+    """Wall time per class of op, from a pair of HIP events around every call
+    (the reference's ``--profile``: ``src/perf.zig:28-131``).  Steps must run
+    eagerly while it is on: events are not recorded into graphs."""
+
+    def __init__(self):
+        self.enabled = False
+        self.label: Optional[str] = None       # set by a part for its next calls (a product's role)
+        self._records: List[tuple] = []
+
+    def reset(self) -> None:
+        self._records = []
+
+    def table(self) -> List[tuple]:
+        """(op, calls, total ms) by falling total; waits for the device."""
+        import torch
+        torch.cuda.synchronize()
+        total: Dict[str, List[float]] = {}
+        for name, e0, e1 in self._records:
+            t = total.setdefault(name, [0, 0.0])
+            t[0] += 1
+            t[1] += e0.elapsed_time(e1)
+        return sorted(((k, int(v[0]), v[1]) for k, v in total.items()), key=lambda r: -r[2])
+
+
+profile = OpProfile()
+
+
 def call(lib: ctypes.CDLL, fn: str, *args) -> None:
     """Call an entry point; a non-zero return raises with the library's message."""
-    rc = getattr(lib, fn)(*args)
+    if profile.enabled:
+        import torch
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        rc = getattr(lib, fn)(*args)
+        e1.record()
+        name = fn[6:] if fn.startswith("agave_") else fn
+        profile._records.append((f"{name}:{profile.label}" if profile.label else name, e0, e1))
+    else:
+        rc = getattr(lib, fn)(*args)
     if rc != 0:
         raise KernelLibraryError(f"{fn}: {lib.agave_last_error().decode(errors='replace')}")

@@ -48,16 +48,20 @@ class Linear:
         n = x.shape[0]
         if out is None:
             out = self.env.workspace.get(tag or self.name, n, self.out_features, out_dtype or x.dtype)
-        from ..ops import gemm
+        from ..ops import gemm, library
         if self.interleave_ff:
             raise RuntimeError(f"{self.name}: a weight packed for GeGLU only serves forward_geglu")
+        library.profile.label = self.name
         gemm.linear(x, self, out)
+        library.profile.label = None
         return out
 
     def forward_geglu(self, x: torch.Tensor, out: torch.Tensor) -> bool:
         """out = gelu_tanh(gate x) * (up x) in one kernel, if the weight was packed for it."""
         if not self.interleave_ff:
             return False
-        from ..ops import gemm_mfma
+        from ..ops import gemm_mfma, library
+        library.profile.label = self.name
         gemm_mfma.product(x, self.packed, out, self.interleave_ff, epilogue=1)
+        library.profile.label = None
         return True

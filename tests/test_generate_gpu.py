@@ -115,6 +115,27 @@ def test_command_line_json(model_a):
     assert meta["architecture"] == "Gemma3ForCausalLM" and meta["n_layers"] == 4 and meta["vocab_size"] == 512
 
 
+def test_profile_option_times_every_class_of_op_without_changing_tokens(model_a):
+    """--profile (src/main.zig:381): per-op wall time; the tokens are those of an unprofiled run."""
+    cfg, w, folder = model_a
+    prompt = [2] + U.random_tokens(9, 512, 111)
+    out = subprocess.run([sys.executable, "-m", "agave_amd", folder, " ".join(map(str, prompt)), "-n", "6",
+                          "--dtype", "bfloat16", "--json", "--ignore-eos", "--ctx-size", "64", "--profile"],
+                         capture_output=True, text=True, cwd=ROOT, timeout=600)
+    assert out.returncode == 0, out.stderr[-2000:]
+    rec = json.loads(out.stdout.strip().splitlines()[-1])
+    ops = {r["op"]: r for r in rec["profile"]}
+    for part in ("qkv", "attn_o", "gate_up", "ffn_down", "lm_head"):
+        assert any(name.endswith(":" + part) for name in ops), (part, sorted(ops))
+    assert any(name.startswith("residual_norm") for name in ops) and any("attn" in name for name in ops)
+    # per step two norms a layer, and at the model's end the last branch's add and the final norm
+    assert ops["residual_norm"]["calls"] == 6 * (2 * 4 + 2) and all(r["ms"] >= 0 for r in rec["profile"])
+    plain = subprocess.run([sys.executable, "-m", "agave_amd", folder, " ".join(map(str, prompt)), "-n", "6",
+                            "--dtype", "bfloat16", "--json", "--ignore-eos", "--ctx-size", "64"],
+                           capture_output=True, text=True, cwd=ROOT, timeout=600)
+    assert json.loads(plain.stdout.strip().splitlines()[-1])["outputs"][0]["tokens"] == rec["outputs"][0]["tokens"]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_tool_whole_tail_and_batches(model_b, dtype, tmp_path):
     """bin/trace_run as a user calls it: the same requests whole, with the last 32 tokens one by
