@@ -4,7 +4,7 @@
 
 A "step" is one decode step of the whole batch: planning on the host, every kernel of the
 model, sampling (greedy) and the copy of the new token ids back to the host.  The default run
-has the layer sizes of BASELINE.json's configs[2], a batch of 8, prompts of 1,024 tokens and
+has the layer sizes of the published Gemma 3 4B text configuration, a batch of 8, prompts of 1,024 tokens and
 256 decoded tokens per sequence (W warm-up steps, then K timed ones).  One JSON line is
 printed: ``value`` is decoded tokens a second; ``prefill`` is one 2,048-token prompt;
 ``roofline`` prices the decode step by the bytes it has to read (every weight once, and the
@@ -24,7 +24,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0            # MI355X HBM3E, published
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
-# BASELINE.json configs[2]: Gemma 3 4B text decoder
+# Gemma 3 4B text decoder, as its config.json gives it
 GEMMA3_4B = dict(
     architectures=["Gemma3ForCausalLM"], model_type="gemma3_text", vocab_size=262208, hidden_size=2560,
     num_hidden_layers=34, num_attention_heads=8, num_key_value_heads=4, head_dim=256,

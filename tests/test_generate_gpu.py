@@ -41,7 +41,7 @@ def plain_greedy(cfg, w, prompt, n, stops=()):
 
 
 def test_greedy_generation_through_the_entry_point(model_a):
-    """BASELINE's Tiny A run: prompts of 5 / 19 / 40 tokens, 8 greedy steps each, context 64."""
+    """The Tiny A run: prompts of 5 / 19 / 40 tokens, 8 greedy steps each, context 64."""
     from agave_amd import Engine, SamplingParams
     cfg, w, folder = model_a
     eng = Engine.from_folder(folder, dtype="float32", max_slots=3, max_context=64)
@@ -73,7 +73,7 @@ def test_stop_ids_and_context_end_generation(model_a):
 
 
 def test_temperature_sampling_is_seeded_and_independent_of_batch_mates(model_b):
-    """BASELINE's Tiny B run: prompts of 1 / 7 / 13 / 30 / 57 tokens, 12 steps at temperature 0.8."""
+    """The Tiny B run: prompts of 1 / 7 / 13 / 30 / 57 tokens, 12 steps at temperature 0.8."""
     from agave_amd import Engine, SamplingParams
     cfg, w, folder = model_b
     eng = Engine.from_folder(folder, dtype="float32", max_slots=5, max_context=96)
