@@ -706,6 +706,163 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int 
     }
 }
 
+// ------------------------------------------------------------------ prefill, streamlined (head sizes 64, 128, 256)
+// The same frame as attn_prefill_mfma_kernel (a workgroup's waves share each page through LDS,
+// two pages in flight), with the decode kernel's inner loop: half pages as units, head size
+// fixed at compile time, probabilities against a running reference that is renewed only when a
+// maximum outgrows it by 2^8, exp2, and masks only on units that touch the diagonal or the
+// window's edge; units that no column of the tile can see are skipped.  A wave takes 16
+// positions of one head; hw heads of a group sit side by side in a workgroup.
+template <int HDT>
+__global__ __launch_bounds__(256) void attn_prefill_fast_kernel(AttnArgs a, int hw) {
+    constexpr int KS = HDT / 2, hd = HDT * 16;
+    constexpr int n_k = 4 * KS, n_v = HDT * 2, buf_tiles = n_k + n_v;         // tiles (of 64 uint4) per page
+    extern __shared__ __attribute__((aligned(16))) uint4 page_lds[];          // [2][K tiles | V tiles][64]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
+    const int G = a.nh / a.nkv;
+    const int chunks = (G + hw - 1) / hw;
+    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
+    const int b = blockIdx.z;
+    const int t0 = a.cu[b], n_new = a.cu[b + 1] - t0;
+    const int blk_len = (4 / hw) * 16;                           // positions a workgroup covers
+    const int blk0 = blockIdx.x * blk_len;
+    if (blk0 >= n_new) return;                                   // the whole workgroup leaves
+    const int tile0 = blk0 + (wave / hw) * 16;                   // first step-token of this wave's tile
+    const int gh = chunk * hw + wave % hw;                       // this wave's head within the group
+    const bool wave_on = tile0 < n_new && gh < G;
+    const bool col_ok = tile0 + j < n_new;
+    const int tok = t0 + (col_ok ? tile0 + j : n_new - 1);       // padding columns repeat the last token
+    const int p = a.tok_pos[tok];
+    const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
+    const float scale2 = a.scale * 1.4426950408889634f;          // scores in units of log2
+
+    frag16 qf[KS];
+    {
+        const bf16* qrow = a.q + (size_t)tok * a.ldq + (size_t)(kvh * G + (gh < G ? gh : 0)) * hd;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (wave_on) qf[ks].u = *reinterpret_cast<const uint4*>(qrow + 32 * ks + 8 * g);
+            else qf[ks].u = uint4{0, 0, 0, 0};
+        }
+    }
+    f32x4_t o[HDT];
+#pragma unroll
+    for (int d = 0; d < HDT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m_ref = -INFINITY, l = 0.f;
+
+    // positions rise along the tile's columns: the first column has the lowest bounds, the last the highest
+    const int p_min = __shfl(p, 0, 64), p_max = __shfl(p, 15, 64);
+    const int lo_min = __shfl(lo, 0, 64), lo_max = __shfl(lo, 15, 64);
+    const int my_first = lo_min / AGAVE_PAGE, my_last = p_max / AGAVE_PAGE;
+    // the workgroup: positions are consecutive within the step
+    const int p_blk0 = a.tok_pos[t0 + blk0];
+    const int blk_n = (n_new - blk0 < blk_len) ? n_new - blk0 : blk_len;
+    const int lo_blk = a.window > 0 ? (p_blk0 - a.window + 1 > 0 ? p_blk0 - a.window + 1 : 0) : 0;
+    const int page_first = lo_blk / AGAVE_PAGE, page_last = (p_blk0 + blk_n - 1) / AGAVE_PAGE;
+
+    constexpr size_t k_stride = (size_t)n_k * 64, v_stride = (size_t)n_v * 64;
+    auto fetch = [&](int pi, int buf) {
+        const long pg = page_of(a, b, pi);
+        if (pg < 0) return;
+        const uint4* ksrc = a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride;
+        const uint4* vsrc = a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride;
+        for (int ti = wave; ti < buf_tiles; ti += 4) {
+            const uint4* src = (ti < n_k) ? ksrc + (size_t)ti * 64 : vsrc + (size_t)(ti - n_k) * 64;
+            uint4* dst = page_lds + ((size_t)buf * buf_tiles + ti) * 64;
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + lane),
+                                             (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+        }
+    };
+
+    fetch(page_first, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for (int pi = page_first; pi <= page_last; ++pi) {
+        const int buf = (pi - page_first) & 1;
+        if (pi < page_last) fetch(pi + 1, buf ^ 1);
+        if (wave_on && pi >= my_first && pi <= my_last && page_of(a, b, pi) >= 0) {
+            const lds_u32x4* kl = (const lds_u32x4*)(page_lds + (size_t)buf * buf_tiles * 64);
+            const lds_u32x4* vl = kl + (size_t)n_k * 64;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const int key0 = pi * AGAVE_PAGE + 32 * half;
+                if (key0 > p_max || key0 + 31 < lo_min) continue;              // no column sees this unit
+                f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0;
+#pragma unroll
+                for (int ks = 0; ks < KS; ++ks) {
+                    frag16 k0, k1;
+                    k0.r = kl[((2 * half) * KS + ks) * 64 + lane];
+                    k1.r = kl[((2 * half + 1) * KS + ks) * 64 + lane];
+                    st0 = mfma_16x16x32(k0, qf[ks], st0);
+                    st1 = mfma_16x16x32(k1, qf[ks], st1);
+                }
+                float s[8];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    s[e] = st0[e] * scale2;
+                    s[4 + e] = st1[e] * scale2;
+                }
+                if (key0 + 31 > p_min || key0 < lo_max) {                      // the diagonal or the window's edge
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int k0 = key0 + 4 * g + e, k1 = k0 + 16;
+                        if (k0 > p || k0 < lo) s[e] = -INFINITY;
+                        if (k1 > p || k1 < lo) s[4 + e] = -INFINITY;
+                    }
+                }
+                float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                if (__any(mx > m_ref + LAZY_LOG2)) {
+                    const float m_new = fmaxf(m_ref, mx);
+                    const float f = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+                    l *= f;
+                    float f4[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) f4[e] = __shfl(f, 4 * g + e, 64);
+#pragma unroll
+                    for (int d = 0; d < HDT; ++d)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[d][e] *= f4[e];
+                    m_ref = m_new;
+                }
+                const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
+                frag16 pf;
+                float sum = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float pe = __builtin_amdgcn_exp2f(s[e] - m_use);
+                    sum += pe;
+                    pf.v[e] = (__bf16)pe;
+                }
+                l += sum;
+#pragma unroll
+                for (int d = 0; d < HDT; ++d) {
+                    frag16 vb;
+                    vb.r = vl[(d * 2 + half) * 64 + lane];
+                    o[d] = mfma_16x16x32(pf, vb, o[d]);
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
+    if (!wave_on) return;
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const int head = kvh * G + gh;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int row = 4 * g + e;                                // slot (position) this lane's values belong to
+        const float lr = __shfl(l, row, 64);
+        if (tile0 + row >= n_new) continue;
+        const float inv = lr > 0.f ? 1.0f / lr : 0.f;
+        bf16* dst = a.out + (size_t)(t0 + tile0 + row) * a.ldo + (size_t)head * hd;
+#pragma unroll
+        for (int d = 0; d < HDT; ++d) dst[16 * d + j] = f32_to_bf16(o[d][e] * inv);
+    }
+}
+
 // ------------------------------------------------------------------ host side
 static int check_common(const char* who, const AttnArgs& a, int N) {
     AGAVE_CHECK(N >= 0 && a.nh > 0 && a.nkv > 0 && a.hd > 0, "%s: bad sizes N=%d nh=%d nkv=%d hd=%d", who, N, a.nh, a.nkv, a.hd);
@@ -812,11 +969,12 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
     AGAVE_CHECK(n_seqs <= 65535, "attn_prefill_mfma: %d sequences exceed the grid limit", n_seqs);
     if (N == 0) return 0;
     const int G = nh / nkv;
-    const int qt_cap = hd > 128 ? 1 : (hd > 64 ? 2 : QT_MAX);       // heads per wave: what fits the register file
+    const bool fast = hd == 64 || hd == 128 || hd == 256;
+    const int qt_cap = fast ? 1 : (hd > 128 ? 1 : (hd > 64 ? 2 : QT_MAX));   // heads per wave: what fits the register file
     const int qt_heads = G < qt_cap ? G : qt_cap;
-    // large heads: the other heads of the group go to other waves of the workgroup
+    // the other heads of the group go to other waves of the workgroup
     int hw = 1;
-    if (hd > 128) hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
+    if (fast || hd > 128) hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
     const int wg_heads = qt_heads * hw, blk_len = (4 / hw) * 16;
     const int chunks = (G + wg_heads - 1) / wg_heads;
     AGAVE_CHECK(nkv * chunks <= 65535, "attn_prefill_mfma: too many head chunks");
@@ -826,12 +984,18 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
     static bool raised = false;
     if (!raised) {
         const int cap = 144 * 1024;
-        hipError_t e1 = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<4, QT_MAX>, hipFuncAttributeMaxDynamicSharedMemorySize, cap);
-        hipError_t e2 = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<8, 2>, hipFuncAttributeMaxDynamicSharedMemorySize, cap);
-        hipError_t e3 = hipFuncSetAttribute((const void*)attn_prefill_mfma_kernel<16, 1>, hipFuncAttributeMaxDynamicSharedMemorySize, cap);
-        AGAVE_CHECK(e1 == hipSuccess && e2 == hipSuccess && e3 == hipSuccess, "attn_prefill_mfma: cannot raise the LDS allowance");
+        const void* fns[] = {(const void*)attn_prefill_mfma_kernel<4, QT_MAX>, (const void*)attn_prefill_mfma_kernel<8, 2>,
+                             (const void*)attn_prefill_mfma_kernel<16, 1>, (const void*)attn_prefill_fast_kernel<4>,
+                             (const void*)attn_prefill_fast_kernel<8>, (const void*)attn_prefill_fast_kernel<16>};
+        for (const void* fn : fns)
+            AGAVE_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, cap) == hipSuccess,
+                        "attn_prefill_mfma: cannot raise the LDS allowance");
         raised = true;
     }
+    if (hd == 64) attn_prefill_fast_kernel<4><<<grid, 256, lds, stream>>>(a, hw);
+    else if (hd == 128) attn_prefill_fast_kernel<8><<<grid, 256, lds, stream>>>(a, hw);
+    else if (hd == 256) attn_prefill_fast_kernel<16><<<grid, 256, lds, stream>>>(a, hw);
+    else
     if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else if (hd <= 128) attn_prefill_mfma_kernel<8, 2><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else attn_prefill_mfma_kernel<16, 1><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
