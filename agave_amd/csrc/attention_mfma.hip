@@ -712,9 +712,11 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int 
 // fixed at compile time, probabilities against a running reference that is renewed only when a
 // maximum outgrows it by 2^8, exp2, and masks only on units that touch the diagonal or the
 // window's edge; units that no column of the tile can see are skipped.  A wave takes 16
-// positions of one head; hw heads of a group sit side by side in a workgroup.
-template <int HDT>
-__global__ __launch_bounds__(256) void attn_prefill_fast_kernel(AttnArgs a, int hw) {
+// positions of one head; hw heads of a group sit side by side in a workgroup of NWV waves (4 or
+// 8: a page fetched into LDS then serves 64 positions instead of 32, which halves the traffic
+// from L2 that bounds this kernel, and two waves share a SIMD).
+template <int HDT, int NWV>
+__global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a, int hw) {
     constexpr int KS = HDT / 2, hd = HDT * 16;
     constexpr int n_k = 4 * KS, n_v = HDT * 2, buf_tiles = n_k + n_v;         // tiles (of 64 uint4) per page
     extern __shared__ __attribute__((aligned(16))) uint4 page_lds[];          // [2][K tiles | V tiles][64]
@@ -724,7 +726,7 @@ __global__ __launch_bounds__(256) void attn_prefill_fast_kernel(AttnArgs a, int 
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
     const int b = blockIdx.z;
     const int t0 = a.cu[b], n_new = a.cu[b + 1] - t0;
-    const int blk_len = (4 / hw) * 16;                           // positions a workgroup covers
+    const int blk_len = (NWV / hw) * 16;                         // positions a workgroup covers
     const int blk0 = blockIdx.x * blk_len;
     if (blk0 >= n_new) return;                                   // the whole workgroup leaves
     const int tile0 = blk0 + (wave / hw) * 16;                   // first step-token of this wave's tile
@@ -766,7 +768,7 @@ __global__ __launch_bounds__(256) void attn_prefill_fast_kernel(AttnArgs a, int 
         if (pg < 0) return;
         const uint4* ksrc = a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride;
         const uint4* vsrc = a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride;
-        for (int ti = wave; ti < buf_tiles; ti += 4) {
+        for (int ti = wave; ti < buf_tiles; ti += NWV) {
             const uint4* src = (ti < n_k) ? ksrc + (size_t)ti * 64 : vsrc + (size_t)(ti - n_k) * 64;
             uint4* dst = page_lds + ((size_t)buf * buf_tiles + ti) * 64;
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + lane),
@@ -975,7 +977,9 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
     // the other heads of the group go to other waves of the workgroup
     int hw = 1;
     if (fast || hd > 128) hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
-    const int wg_heads = qt_heads * hw, blk_len = (4 / hw) * 16;
+    // the streamlined kernel takes eight waves once a sequence brings enough tokens for them
+    const int nwv = (fast && max_new > 32) ? 8 : 4;
+    const int wg_heads = qt_heads * hw, blk_len = (nwv / hw) * 16;
     const int chunks = (G + wg_heads - 1) / wg_heads;
     AGAVE_CHECK(nkv * chunks <= 65535, "attn_prefill_mfma: too many head chunks");
     dim3 grid((max_new + blk_len - 1) / blk_len, nkv * chunks, n_seqs);
@@ -985,18 +989,24 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
     if (!raised) {
         const int cap = 144 * 1024;
         const void* fns[] = {(const void*)attn_prefill_mfma_kernel<4, QT_MAX>, (const void*)attn_prefill_mfma_kernel<8, 2>,
-                             (const void*)attn_prefill_mfma_kernel<16, 1>, (const void*)attn_prefill_fast_kernel<4>,
-                             (const void*)attn_prefill_fast_kernel<8>, (const void*)attn_prefill_fast_kernel<16>};
+                             (const void*)attn_prefill_mfma_kernel<16, 1>,
+                             (const void*)attn_prefill_fast_kernel<4, 4>, (const void*)attn_prefill_fast_kernel<8, 4>,
+                             (const void*)attn_prefill_fast_kernel<16, 4>, (const void*)attn_prefill_fast_kernel<4, 8>,
+                             (const void*)attn_prefill_fast_kernel<8, 8>, (const void*)attn_prefill_fast_kernel<16, 8>};
         for (const void* fn : fns)
             AGAVE_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, cap) == hipSuccess,
                         "attn_prefill_mfma: cannot raise the LDS allowance");
         raised = true;
     }
-    if (hd == 64) attn_prefill_fast_kernel<4><<<grid, 256, lds, stream>>>(a, hw);
-    else if (hd == 128) attn_prefill_fast_kernel<8><<<grid, 256, lds, stream>>>(a, hw);
-    else if (hd == 256) attn_prefill_fast_kernel<16><<<grid, 256, lds, stream>>>(a, hw);
-    else
-    if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
+    if (fast && nwv == 8) {
+        if (hd == 64) attn_prefill_fast_kernel<4, 8><<<grid, 512, lds, stream>>>(a, hw);
+        else if (hd == 128) attn_prefill_fast_kernel<8, 8><<<grid, 512, lds, stream>>>(a, hw);
+        else attn_prefill_fast_kernel<16, 8><<<grid, 512, lds, stream>>>(a, hw);
+    } else if (fast) {
+        if (hd == 64) attn_prefill_fast_kernel<4, 4><<<grid, 256, lds, stream>>>(a, hw);
+        else if (hd == 128) attn_prefill_fast_kernel<8, 4><<<grid, 256, lds, stream>>>(a, hw);
+        else attn_prefill_fast_kernel<16, 4><<<grid, 256, lds, stream>>>(a, hw);
+    } else if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else if (hd <= 128) attn_prefill_mfma_kernel<8, 2><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else attn_prefill_mfma_kernel<16, 1><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     AGAVE_LAUNCH_CHECK("attn_prefill_mfma");
