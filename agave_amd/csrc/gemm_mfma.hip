@@ -401,6 +401,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
     static_assert(X_LOADS * NWV * 1024 == X_BYTES && W_LOADS * NWV * 1024 == W_BYTES, "whole loads per wave");
     constexpr int LOADS = X_LOADS + W_LOADS;
     static_assert(LOADS * (NS - 2) < 64, "the load counter holds 6 bits");
+    static_assert(NS >= 2 && NS <= 5, "the waits below name up to three stages in flight behind the awaited one");
     extern __shared__ __attribute__((aligned(16))) unsigned char tl_lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wn = wave & 1, wm = wave >> 1;
@@ -456,7 +457,8 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
     for (int st = 0; st < n_stage; ++st) {
         // stage st has landed once at most the loads of the NS-2 stages after it are outstanding
         const int ahead = (n_stage - 1 - st < NS - 2) ? n_stage - 1 - st : NS - 2;
-        if (ahead >= 2) __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * LOADS) & 15) | (((2 * LOADS) >> 4) << 14));
+        if (ahead >= 3) __builtin_amdgcn_s_waitcnt(0x0F70 | ((3 * LOADS) & 15) | (((3 * LOADS) >> 4) << 14));
+        else if (ahead == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * LOADS) & 15) | (((2 * LOADS) >> 4) << 14));
         else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS & 15) | ((LOADS >> 4) << 14));
         else __builtin_amdgcn_s_waitcnt(0x0F70);
         // a bare barrier: __syncthreads() would also wait for the loads still wanted in flight
