@@ -33,6 +33,14 @@ GEMMA3_4B = dict(
     rms_norm_eps=1e-6, tie_word_embeddings=True, hidden_activation="gelu_pytorch_tanh",
     max_position_embeddings=131072, bos_token_id=2, eos_token_id=1)
 
+# the larger published sizes of the same architecture, for --model (not the default run)
+GEMMA3_12B = dict(GEMMA3_4B, hidden_size=3840, num_hidden_layers=48, num_attention_heads=16, num_key_value_heads=8,
+                  intermediate_size=15360)
+GEMMA3_27B = dict(GEMMA3_4B, hidden_size=5376, num_hidden_layers=62, num_attention_heads=32, num_key_value_heads=16,
+                  head_dim=128, query_pre_attn_scalar=168, intermediate_size=21504)
+MODELS = {"4b": ("gemma3-4b-text", GEMMA3_4B), "12b": ("gemma3-12b-text", GEMMA3_12B),
+          "27b": ("gemma3-27b-text", GEMMA3_27B)}
+
 PROMPT_LEN, DECODE_LEN, CONTEXT, PREFILL_LEN = 1024, 256, 4096, 2048
 
 
@@ -134,7 +142,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=240)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=GEMMA3_4B["num_hidden_layers"],
+    ap.add_argument("--model", default="4b", choices=sorted(MODELS),
+                    help="layer sizes: Gemma 3 4B (the default run), 12B or 27B")
+    ap.add_argument("--layers", type=int, default=0,
                     help="run fewer layers of the same sizes (reported in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
@@ -152,7 +162,10 @@ def main() -> int:
     import torch
     from agave_amd.engine import Engine
 
-    cfg = dict(GEMMA3_4B, num_hidden_layers=args.layers)
+    model_name, full = MODELS[args.model]
+    if args.layers <= 0:
+        args.layers = full["num_hidden_layers"]
+    cfg = dict(full, num_hidden_layers=args.layers)
     m = model_numbers(cfg, args.layers)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     per_seq = -(-(PROMPT_LEN + DECODE_LEN + 64) // 64) * 64
@@ -174,11 +187,11 @@ def main() -> int:
     need = decode_step_bytes(m, contexts)
     achieved = need / (ms_step * 1e-3) / 1e9
     out = {
-        "metric": "decode tok/s, Gemma3-4B bf16, batch 8, 1024-token prompts + 256 decoded",
+        "metric": f"decode tok/s, Gemma3-{args.model.upper()} {dkey}, batch {args.batch}, 1024-token prompts + 256 decoded",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dkey, "data": "synthetic: uniform-random token ids, random N(0,0.02) weights",
-        "config": {"model": "gemma3-4b-text", "layers": args.layers, "layers_of_config": GEMMA3_4B["num_hidden_layers"],
+        "config": {"model": model_name, "layers": args.layers, "layers_of_config": full["num_hidden_layers"],
                    "hidden": m["e"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                    "head_dim": cfg["head_dim"], "intermediate": m["ff"], "vocab": m["v"],
                    "sliding_window": m["window"], "sliding_pattern": cfg["sliding_window_pattern"],
