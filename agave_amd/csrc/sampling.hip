@@ -349,3 +349,23 @@ extern "C" int agave_repeat_penalty(float* logits, long ld, const int* ids, cons
     AGAVE_LAUNCH_CHECK("repeat_penalty");
     return 0;
 }
+
+
+// ------------------------------------------------------------------ sampled tokens feed the next step
+// dst[i] = src[map[i]]: the tokens a step sampled become the next step's input on the device, so
+// that the host can launch that step before it has read them.
+__global__ void gather_tokens_kernel(const int* __restrict__ src, const int* __restrict__ map, int* __restrict__ dst,
+                                     int n, int n_src) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int k = map[i];
+    dst[i] = (k >= 0 && k < n_src) ? src[k] : 0;
+}
+
+extern "C" int agave_gather_tokens(const int* src, const int* map, int* dst, int n, int n_src, hipStream_t stream) {
+    AGAVE_CHECK(n >= 0 && n_src >= 0 && (n == 0 || (src && map && dst)), "gather_tokens: bad sizes or null buffer");
+    if (n == 0) return 0;
+    gather_tokens_kernel<<<(n + 255) / 256, 256, 0, stream>>>(src, map, dst, n, n_src);
+    AGAVE_LAUNCH_CHECK("gather_tokens");
+    return 0;
+}

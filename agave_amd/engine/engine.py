@@ -153,14 +153,22 @@ class Engine:
         """Run ``tokens[i]`` as the next tokens of the sequence in ``slots[i]``.  Returns the
         float32 logits [wanted, vocab] on the GPU in the order of the sequences and of their
         wanted places (valid until the next step), or None if nothing is wanted."""
-        step = self.planner.plan(slots, tokens, want, decode_widths=self._decode_widths if self.use_graphs else None)
+        return self._run(slots, tokens, want)[0]
+
+    def _run(self, slots, tokens, want, carry=None, floats=None):
+        """Plan, run and commit one step; (logits, step)."""
+        step = self.planner.plan(slots, tokens, want, decode_widths=self._decode_widths if self.use_graphs else None,
+                                 carry=carry, floats=floats)
+        if carry is not None:
+            from ..ops import sampling as sample_ops
+            sample_ops.gather_tokens(self._sampled_all(), step.carry_dev, step.tokens)
         if self.use_graphs and step.is_decode and step.n_want == step.n_tokens:
             step.fixed_span = span_bucket(step.page_span(None))
             logits = self.graphs.run(step)
         else:
             logits = self.model.forward(step)
         self.planner.commit(step)
-        return logits
+        return logits, step
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.device)
@@ -170,10 +178,31 @@ class Engine:
     def max_slots(self) -> int:
         return self.cache.max_slots
 
+    def _sampled_all(self) -> torch.Tensor:
+        """Where every step leaves its sampled tokens (one per sequence, in the step's order)."""
+        return self.workspace.get("sampled", self.max_slots, 1, torch.int32).view(-1)
+
     def step_sample(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], rows) -> List[int]:
         """One step, then one token per sequence drawn from its last logits on the GPU.
         ``rows``: one :class:`RowSampling` per sequence."""
+        return self.finish_step(self.launch_step(slots, tokens, rows))
+
+    def launch_step(self, slots: Sequence[int], tokens: Optional[Sequence[Sequence[int]]], rows,
+                    carry: Optional[Sequence[int]] = None):
+        """Enqueue a step and the sampling of one token per sequence, without waiting for the
+        GPU; :meth:`finish_step` returns the tokens.  ``carry`` (with ``tokens`` None): sequence i
+        of this step continues with the token that row ``carry[i]`` of the step launched before
+        sampled; it is taken on the device, so this step can be launched before that one has
+        been read back, and the host's work on a step hides behind the GPU's on the one before."""
+        import numpy as np
         from ..ops import sampling as sample_ops
+        b = len(slots)
+        if carry is not None:
+            if tokens is not None:
+                raise ValueError("launch_step: either tokens or carry")
+            if any(r.repeat_penalty != 1.0 for r in rows):
+                raise ValueError("launch_step: the repeat penalty needs the tokens on the host; no carry")
+            tokens = [[0]] * b
         chunk = int(self.prefill_chunk or 0)
         if chunk > 0 and max(len(t) for t in tokens) > chunk:
             # the reference feeds a prompt in chunks (src/models/gemma3.zig:385-391); only the
@@ -184,8 +213,9 @@ class Engine:
                 self.step([slots[i] for i in idx], [tokens[i][:chunk] for i in idx], "none")
                 for i in idx:
                     tokens[i] = tokens[i][chunk:]
-        logits = self.step(slots, tokens, "last")
-        b = len(slots)
+        params = np.asarray([[r.temperature, float(min(r.top_k, 1 << 20)), r.top_p, r.u] for r in rows],
+                            dtype=np.float32)
+        logits, step = self._run(slots, tokens, "last", carry=carry, floats=params)
         if any(r.repeat_penalty != 1.0 and r.generated for r in rows):
             cu = [0]
             flat: List[int] = []
@@ -197,13 +227,26 @@ class Engine:
             cu_t = torch.tensor(cu, dtype=torch.int32, device=self.device)
             pen = torch.tensor([r.repeat_penalty for r in rows], dtype=torch.float32, device=self.device)
             sample_ops.repeat_penalty(logits, ids, cu_t, pen)
-        params = torch.tensor([[r.temperature, float(min(r.top_k, 1 << 20)), r.top_p, r.u] for r in rows],
-                              dtype=torch.float32, device=self.device)
         work = self.workspace.get("sample_work", b, self.spec.vocab_size, torch.float32)
-        out = self.workspace.get("sampled", b, 1, torch.int32).view(-1)
+        out = self._sampled_all()[:b]
         scratch = self.workspace.get("sample_scratch", b, 128, torch.float32).view(-1)
-        sample_ops.sample(logits, work, params, out, scratch)
-        return out.cpu().tolist()
+        sample_ops.sample(logits, work, step.floats_dev.view(b, 4), out, scratch)
+        self._result_turn = 1 - getattr(self, "_result_turn", 0)
+        hosts = getattr(self, "_result_hosts", None)
+        if hosts is None:
+            hosts = self._result_hosts = [torch.empty(self.max_slots, dtype=torch.int32, pin_memory=True)
+                                          for _ in range(2)]
+        host = hosts[self._result_turn]
+        host[:b].copy_(out, non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        return host, done, b
+
+    def finish_step(self, handle) -> List[int]:
+        """The tokens of a step that :meth:`launch_step` enqueued (waits for it)."""
+        host, done, b = handle
+        done.synchronize()
+        return host[:b].tolist()
 
     def generate(self, prompts, params=None, max_batch: Optional[int] = None, stats=None):
         """Generate for every prompt (lists of token ids); see :func:`agave_amd.engine.generate.generate`."""

@@ -11,6 +11,13 @@ equal tokens" (``src/main.zig:2400-2407``) changes outputs and is not taken over
 The loop's decisions need no GPU: it talks to a *backend* with ``max_context``, ``max_slots``,
 ``alloc_slot()``, ``free_slot(slot)`` and ``step_sample(slots, tokens, rows) -> token ids``;
 the engine is one, the tests use a fake.
+
+A backend that also has ``launch_step(slots, tokens | None, rows, carry)`` and
+``finish_step(handle)`` is driven one step ahead: the next step is launched, with its tokens
+taken on the device from what the running step samples, before the running step's tokens are
+read.  The host's work then hides behind the GPU's.  A sequence that turns out to have
+stopped has run one step too many; that step's token for it is dropped and its slot is given
+back once the step has ended.  Nothing a request gets depends on this.
 """
 from __future__ import annotations
 
@@ -87,6 +94,21 @@ def generate(backend, prompts: Sequence[Sequence[int]],
         u = float(rngs[i].random(dtype=np.float32)) if p.temperature > 0 else 0.0
         return RowSampling(p.temperature, p.top_k, p.top_p, p.repeat_penalty, u, results[i].tokens)
 
+    ahead = hasattr(backend, "launch_step") and all(p.repeat_penalty == 1.0 for p in plist)
+
+    def settle(i: int, tok: int) -> None:
+        """Book the token request i drew; sets its finish reason if it ends here."""
+        r = results[i]
+        if tok in stops[i]:
+            r.finish_reason = "stop"                      # the end token is not emitted
+        else:
+            r.tokens.append(tok)
+            stats.tokens += 1
+            if len(r.tokens) >= plist[i].max_tokens:
+                r.finish_reason = "length"
+            elif r.prompt_tokens + len(r.tokens) > backend.max_context:
+                r.finish_reason = "context"               # no room to feed this token
+
     while queue:
         batch, queue = queue[:max_batch], queue[max_batch:]
         stats.batches += 1
@@ -95,36 +117,62 @@ def generate(backend, prompts: Sequence[Sequence[int]],
         feed = [list(prompts[i]) for i in live]
         first = True
         try:
-            while live:
-                t0 = time.perf_counter()
-                sampled = backend.step_sample([slots[i] for i in live], feed, [row(i) for i in live])
+            if not ahead:
+                while live:
+                    t0 = time.perf_counter()
+                    sampled = backend.step_sample([slots[i] for i in live], feed, [row(i) for i in live])
+                    ms = (time.perf_counter() - t0) * 1e3
+                    if first:
+                        stats.prefill_tokens += sum(len(f) for f in feed)
+                        stats.prefill_ms += ms
+                    else:
+                        stats.gen_ms += ms
+                        stats.decode_tokens += len(live)
+                    first = False
+                    nxt = []
+                    for i, tok in zip(live, sampled):
+                        settle(i, int(tok))
+                        if results[i].finish_reason:
+                            backend.free_slot(slots.pop(i))               # given back at once
+                        else:
+                            nxt.append(i)
+                    live = nxt
+                    feed = [[results[i].tokens[-1]] for i in live]
+                continue
+            # one step ahead: `running` is the step under way over the requests `live`, some of which
+            # may have ended with the token before (this is then their step too many)
+            t0 = time.perf_counter()
+            running = backend.launch_step([slots[i] for i in live], feed, [row(i) for i in live], None)
+            stats.prefill_tokens += sum(len(f) for f in feed)
+            while True:
+                # who goes on unless the running step draws an end token: known beforehand
+                on = [i for i in live if not results[i].finish_reason
+                      and len(results[i].tokens) + 1 < plist[i].max_tokens
+                      and results[i].prompt_tokens + len(results[i].tokens) + 1 <= backend.max_context]
+                following = None
+                if on:
+                    following = backend.launch_step([slots[i] for i in on], None, [row(i) for i in on],
+                                                    [live.index(i) for i in on])
+                sampled = backend.finish_step(running)
                 ms = (time.perf_counter() - t0) * 1e3
+                t0 = time.perf_counter()
                 if first:
-                    stats.prefill_tokens += sum(len(f) for f in feed)
                     stats.prefill_ms += ms
                 else:
                     stats.gen_ms += ms
-                    stats.decode_tokens += len(live)
-                first = False
-                nxt = []
                 for i, tok in zip(live, sampled):
-                    tok = int(tok)
-                    r = results[i]
-                    if tok in stops[i]:
-                        r.finish_reason = "stop"                      # the end token is not emitted
-                    else:
-                        r.tokens.append(tok)
-                        stats.tokens += 1
-                        if len(r.tokens) >= plist[i].max_tokens:
-                            r.finish_reason = "length"
-                        elif r.prompt_tokens + len(r.tokens) > backend.max_context:
-                            r.finish_reason = "context"               # no room to feed this token
-                    if r.finish_reason:
-                        backend.free_slot(slots.pop(i))               # given back at once
-                    else:
-                        nxt.append(i)
-                live = nxt
-                feed = [[results[i].tokens[-1]] for i in live]
+                    if results[i].finish_reason:
+                        backend.free_slot(slots.pop(i))       # ended a step ago; no step uses its slot now
+                        continue
+                    settle(i, int(tok))
+                    if not first:
+                        stats.decode_tokens += 1
+                    if results[i].finish_reason and i not in on:
+                        backend.free_slot(slots.pop(i))       # not part of the step that is under way
+                first = False
+                if following is None:
+                    break
+                live, running = on, following
         finally:
             for s in slots.values():
                 backend.free_slot(s)

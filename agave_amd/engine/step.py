@@ -54,6 +54,8 @@ class Step:
     workspace: object = None
     fixed_span: Optional[int] = None    # a captured decode graph plans its splits for this many pages
     tables_start_at_reach: bool = False  # decode: column 0 of every table row is the first page the token reaches
+    carry_dev: Optional[torch.Tensor] = None    # int32 [B]: rows of the previous step's sample that these tokens are
+    floats_dev: Optional[torch.Tensor] = None   # float32 payload that travelled with the step (sampling parameters)
 
     def page_span(self, window: Optional[int]) -> int:
         """Most pages any sequence's last token of this step reaches back over."""
@@ -104,25 +106,36 @@ class StepPlanner:
         self.workspace = workspace
         self.vocab_size = vocab_size
         self.device = device
-        self._host: Optional[torch.Tensor] = None
+        self._hosts: List[Optional[torch.Tensor]] = [None, None]   # two pinned buffers in turn: a step may be
+        self._copied: List[Optional[torch.cuda.Event]] = [None, None]  # planned while the one before still waits
+        self._turn = 0
         self._dev: Optional[torch.Tensor] = None
-        self._copied = None          # event: the last upload has left the host buffer
         self.fixed_width: Optional[List[int]] = None   # table widths pinned for graph capture
         self.buffer_generation = 0   # changes when the device buffer of the step's description moves
 
-    def _buffers(self, n: int) -> None:
-        if self._host is None or self._host.numel() < n:
-            cap = max(n, 4096) if self._host is None else max(n, 2 * self._host.numel())
-            if self._copied is not None:
-                self._copied.synchronize()
-            self._host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
-            self._dev = torch.empty(cap, dtype=torch.int32, device=self.device)
+    def _buffers(self, n: int) -> torch.Tensor:
+        """The pinned host buffer of this turn, at least ``n`` int32 long, free to be written."""
+        self._turn ^= 1
+        t = self._turn
+        if self._copied[t] is not None:
+            self._copied[t].synchronize()          # its last upload has left it
+        host = self._hosts[t]
+        if host is None or host.numel() < n:
+            cap = max(n, 4096) if host is None else max(n, 2 * host.numel())
+            self._hosts[t] = host = torch.empty(cap, dtype=torch.int32, pin_memory=True)
+        if self._dev is None or self._dev.numel() < host.numel():
+            self._dev = torch.empty(host.numel(), dtype=torch.int32, device=self.device)
             self.buffer_generation += 1
+        return host
 
     def plan(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want = "last",
-             decode_widths: Optional[List[int]] = None) -> Step:
+             decode_widths: Optional[List[int]] = None, carry: Optional[Sequence[int]] = None,
+             floats: Optional[np.ndarray] = None) -> Step:
         """``decode_widths``: table widths to use if this turns out to be a decode step (one token per
-        sequence), so that all decode steps of a batch size have the same layout on the device."""
+        sequence), so that all decode steps of a batch size have the same layout on the device.
+        ``carry``: one index per sequence into what the previous step sampled (the tokens given
+        are placeholders then); ``floats``: float32 values that travel in the same upload.  Both
+        lie behind everything else, so they do not move what a recorded graph reads."""
         if len(slots) != len(tokens) or len(slots) == 0:
             raise StepError("a step needs as many token lists as slots, and at least one")
         n_new = [len(t) for t in tokens]
@@ -147,11 +160,13 @@ class StepPlanner:
             if fixed is not None and w <= fixed[gi]:
                 w = fixed[gi]
             widths.append(w)
-        total = 3 * n + 3 * b + 1 + len(want_rows) + sum(b + b * w for w in widths)
-        self._buffers(total)
-        if self._copied is not None:
-            self._copied.synchronize()
-        host = self._host.numpy()
+        n_carry = len(carry) if carry is not None else 0
+        n_floats = int(floats.size) if floats is not None else 0
+        if carry is not None and n_carry != b:
+            raise StepError("carry needs one index per sequence")
+        total = 3 * n + 3 * b + 1 + len(want_rows) + sum(b + b * w for w in widths) + n_carry + n_floats
+        host_t = self._buffers(total)
+        host = host_t.numpy()
         off = 0
 
         def put(values, count) -> Tuple[int, int]:
@@ -175,10 +190,14 @@ class StepPlanner:
             for i, r in enumerate(p.rows):
                 tab[i, :len(r)] = r
             s_tables.append((put(tab.reshape(-1), b * w), s_base, w))
+        s_carry = put(np.asarray(carry, dtype=np.int32), n_carry) if carry is not None else None
+        s_floats = None
+        if floats is not None:
+            s_floats = put(np.ascontiguousarray(floats, dtype=np.float32).reshape(-1).view(np.int32), n_floats)
         assert off == total
-        self._dev[:total].copy_(self._host[:total], non_blocking=True)
-        self._copied = torch.cuda.Event()
-        self._copied.record()
+        self._dev[:total].copy_(host_t[:total], non_blocking=True)
+        self._copied[self._turn] = torch.cuda.Event()
+        self._copied[self._turn].record()
         d = self._dev
 
         def view(span):
@@ -190,7 +209,9 @@ class StepPlanner:
             tokens=view(s_tok), tok_seq=view(s_seq), tok_pos=view(s_pos), slots_dev=view(s_slots),
             pos0_dev=view(s_pos0), cu_dev=view(s_cu), want_rows=view(s_want),
             tables=[(view(t).view(b, w), view(sb)) for t, sb, w in s_tables], cache=self.cache,
-            workspace=self.workspace, tables_start_at_reach=(max(n_new) == 1))
+            workspace=self.workspace, tables_start_at_reach=(max(n_new) == 1),
+            carry_dev=view(s_carry) if s_carry is not None else None,
+            floats_dev=view(s_floats).view(torch.float32) if s_floats is not None else None)
 
     def commit(self, step: Step) -> None:
         self.cache.commit_step(step.slots, step.n_new)

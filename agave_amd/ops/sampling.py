@@ -9,6 +9,7 @@ from .kernels import _I, _L, _P
 kernels.register_signatures("sampling", {
     "agave_sample": [_P, _L, _P, _L, _P, _P, _I, _I, _P, _P],
     "agave_repeat_penalty": [_P, _L, _P, _P, _P, _I, _I, _P],
+    "agave_gather_tokens": [_P, _P, _P, _I, _I, _P],
 })
 
 
@@ -53,3 +54,14 @@ def repeat_penalty(logits: torch.Tensor, ids: torch.Tensor, cu: torch.Tensor, pe
         raise TypeError(f"repeat_penalty: penalty must be {b} float32 on the GPU")
     library.call(kernels.lib("sampling"), "agave_repeat_penalty", logits.data_ptr(), ld, ids.data_ptr(),
                  cu.data_ptr(), penalty.data_ptr(), b, v, kernels.stream())
+
+
+def gather_tokens(src: torch.Tensor, index: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst[i] = src[index[i]] (int32, on the GPU): what a step sampled becomes the next step's tokens."""
+    for t, what in ((src, "src"), (index, "index"), (dst, "dst")):
+        if t.dtype != torch.int32 or not t.is_contiguous() or not t.is_cuda:
+            raise TypeError(f"gather_tokens: {what} must be contiguous int32 on the GPU")
+    if index.numel() != dst.numel():
+        raise ValueError("gather_tokens: one index per destination")
+    library.call(kernels.lib("sampling"), "agave_gather_tokens", src.data_ptr(), index.data_ptr(), dst.data_ptr(),
+                 dst.numel(), src.numel(), kernels.stream())

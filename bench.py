@@ -3,7 +3,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A "step" is one decode step of the whole batch: planning on the host, every kernel of the
-model, sampling (greedy) and the copy of the new token ids back to the host.  The default run
+model, sampling (greedy) and the copy of the new token ids back to the host; as in generation,
+a step is launched while the host still waits for the tokens of the step before.  The default run
 has the layer sizes of the published Gemma 3 4B text configuration, a batch of 8, prompts of 1,024 tokens and
 256 decoded tokens per sequence (W warm-up steps, then K timed ones).  One JSON line is
 printed: ``value`` is decoded tokens a second; ``prefill`` is one 2,048-token prompt;
@@ -103,9 +104,16 @@ def run_decode(engine, batch: int, steps: int, warmup: int, seed: int):
         for _ in range(warmup):
             toks = engine.step_sample(slots, [[t] for t in toks], rows)
         torch.cuda.synchronize()
+        # the timed steps run as generation runs them: each is launched, its tokens taken on the
+        # device from the step before, while the host still waits for that step's tokens
+        carry = list(range(batch))
         t0 = time.perf_counter()
-        for _ in range(steps):
-            toks = engine.step_sample(slots, [[t] for t in toks], rows)
+        running = engine.launch_step(slots, [[t] for t in toks], rows)
+        for _ in range(steps - 1):
+            following = engine.launch_step(slots, None, rows, carry)
+            toks = engine.finish_step(running)
+            running = following
+        toks = engine.finish_step(running)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         first_ctx = PROMPT_LEN + warmup + 1          # keys the first timed step attends to

@@ -175,3 +175,36 @@ def test_trace_tool_whole_tail_and_batches(model_b, dtype, tmp_path):
             check(got, U.plain_logits(cfg, w, r), f"batch {bi} request {ri}")
     # a step that wants nothing writes no file
     assert not os.path.exists(str(tmp_path / "none" / "0.f32"))
+
+
+def test_steps_launched_ahead_give_the_tokens_of_steps_run_one_by_one(model_b):
+    """launch_step with tokens carried on the device (also for a shrinking subset of the rows, in
+    another order) against step_sample fed from the host."""
+    from agave_amd.engine import Engine
+    from agave_amd.engine.generate import RowSampling
+    cfg, w, folder = model_b
+    a = Engine.from_folder(folder, dtype="float32", max_slots=4, max_context=96)
+    b = Engine.from_folder(folder, dtype="float32", max_slots=4, max_context=96)
+    prompts = [U.random_tokens(n, cfg["vocab_size"], 300 + i) for i, n in enumerate((9, 1, 30, 14))]
+    rows = lambda k: [RowSampling(0.0, 0, 1.0, 1.0, 0.0, []) for _ in range(k)]
+    sa = [a.alloc_slot() for _ in prompts]
+    sb = [b.alloc_slot() for _ in prompts]
+    keep = [[0, 1, 2, 3], [0, 1, 2, 3], [3, 0, 2], [3, 0, 2], [2, 3], [2], [2]]     # rows of the first step, per step
+    # one by one, from the host
+    toks = a.step_sample(sa, prompts, rows(4))
+    ref = [list(toks)]
+    cur = list(range(4))
+    for k in keep:
+        toks = a.step_sample([sa[i] for i in k], [[toks[cur.index(i)]] for i in k], rows(len(k)))
+        cur = k
+        ref.append(list(toks))
+    # launched ahead, tokens carried on the device
+    got = []
+    running = b.launch_step(sb, prompts, rows(4))
+    cur = list(range(4))
+    for k in keep:
+        following = b.launch_step([sb[i] for i in k], None, rows(len(k)), [cur.index(i) for i in k])
+        got.append(b.finish_step(running))
+        running, cur = following, k
+    got.append(b.finish_step(running))
+    assert got == ref

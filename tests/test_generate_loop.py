@@ -99,3 +99,72 @@ def test_sampling_params_are_checked():
                 dict(repeat_penalty=0)):
         with pytest.raises(ValueError):
             SamplingParams(**bad)
+
+
+class AheadBackend(FakeBackend):
+    """The same model with ``launch_step`` / ``finish_step``: a launched step's tokens may come from
+    what the step before it sampled (``carry``), which the backend keeps as the device would."""
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        self.sampled: List[int] = []
+        self.in_flight = 0
+        self.max_in_flight = 0
+        self.busy = set()                # slots of launched, unfinished steps
+
+    def free_slot(self, s):
+        assert s not in self.busy, "slot freed while a launched step still uses it"
+        super().free_slot(s)
+
+    def launch_step(self, slots, tokens, rows, carry=None):
+        if carry is not None:
+            assert tokens is None and len(carry) == len(slots)
+            tokens = [[self.sampled[k]] for k in carry]
+        self.sampled = self.step_sample(slots, tokens, rows)
+        self.in_flight += 1
+        self.max_in_flight = max(self.max_in_flight, self.in_flight)
+        self.busy |= set(slots)
+        return (list(self.sampled), list(slots))
+
+    def finish_step(self, handle):
+        toks, slots = handle
+        self.in_flight -= 1
+        self.busy -= set(slots)
+        return toks
+
+
+@pytest.mark.parametrize("prompts,params,eos", [
+    ([[10, 11], [40], [5]], SamplingParams(max_tokens=8), [13, 44]),
+    ([[1, 2, 3], [9], [30, 31]], SamplingParams(max_tokens=3, ignore_eos=True), [5]),
+    ([[i] for i in range(7)], SamplingParams(max_tokens=5), [4, 9]),
+    ([[1, 2, 3, 4], [2]], SamplingParams(max_tokens=50), []),
+    ([[3]], SamplingParams(max_tokens=1), []),
+])
+def test_one_step_ahead_gives_the_same_results_and_loses_no_slot(prompts, params, eos):
+    plain, ahead = FakeBackend(max_slots=3, max_context=9), AheadBackend(max_slots=3, max_context=9)
+    sa, sb = GenerationStats(), GenerationStats()
+    a = generate(plain, prompts, params, eos_ids=eos, stats=sa)
+    b = generate(ahead, prompts, params, eos_ids=eos, stats=sb)
+    assert [(r.tokens, r.finish_reason) for r in a] == [(r.tokens, r.finish_reason) for r in b]
+    assert (sa.tokens, sa.prefill_tokens, sa.decode_tokens, sa.batches) == (sb.tokens, sb.prefill_tokens, sb.decode_tokens, sb.batches)
+    assert ahead.length == {} and sorted(ahead.free) == [0, 1, 2] and ahead.in_flight == 0
+    assert ahead.max_in_flight <= 2
+    if len(prompts) > 1 or params.max_tokens > 1:
+        assert ahead.max_in_flight == 2                         # it does run ahead
+
+
+def test_one_step_ahead_keeps_each_request_stream_of_draws():
+    p = SamplingParams(max_tokens=4, temperature=0.8, seed=3)
+    a, b = FakeBackend(max_slots=3), AheadBackend(max_slots=3)
+    generate(a, [[1], [2], [3]], p, eos_ids=[4])                # request 1 stops early: one step too many
+    generate(b, [[1], [2], [3]], p, eos_ids=[4])
+    for sl in (0, 1, 2):
+        ua = [s["u"][s["slots"].index(sl)] for s in a.steps if sl in s["slots"]]
+        ub = [s["u"][s["slots"].index(sl)] for s in b.steps if sl in s["slots"]]
+        assert ub[:len(ua)] == ua and len(ub) - len(ua) in (0, 1)
+
+
+def test_repeat_penalty_is_not_run_ahead():
+    be = AheadBackend(max_slots=1)
+    generate(be, [[7, 8]], SamplingParams(max_tokens=3, repeat_penalty=1.3))
+    assert be.max_in_flight == 0 and [s["gen"][0] for s in be.steps] == [[], [9], [9, 10]]
