@@ -29,8 +29,12 @@ class Linear:
             if env.dtype == torch.float32 and w.dtype != torch.float32:
                 w = w.to(torch.float32)
             ws.append(w)
-        if len({w.dtype for w in ws}) != 1 or len({w.shape[1] for w in ws}) != 1:
-            raise ValueError(f"{name}: stacked weights must agree in element type and input size")
+        if len({w.shape[1] for w in ws}) != 1:
+            raise ValueError(f"{name}: stacked weights must agree in input size")
+        if len({w.dtype for w in ws}) != 1:
+            # a stack of matrices stored in different widths is held in 32-bit (what is stored in
+            # 32-bit stays so; widening the others loses nothing)
+            ws = [w.to(torch.float32) for w in ws]
         dev = [w.to(env.device) for w in ws]
         self.weight = dev[0].contiguous() if len(dev) == 1 else torch.cat(dev, dim=0).contiguous()
         self.out_features, self.in_features = self.weight.shape

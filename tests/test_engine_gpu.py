@@ -166,3 +166,31 @@ def test_prompt_in_pieces(engine_of):
         eng.free_slot(s)
     for i, r in enumerate(reqs):
         close(dtype)(torch.cat(outs[i], 0), U.plain_logits(cfg, weights, r), f"request {i} in pieces")
+
+
+def test_tensors_stored_in_32_bit_stay_so_in_a_bfloat16_engine(tmp_path):
+    """A checkpoint that stores some matrices and the table in 32-bit (values that bfloat16 cannot
+    hold): the bfloat16 engine keeps them in 32-bit and still gives the plain logits."""
+    from safetensors.torch import save_file
+    import json, os
+    from agave_amd.engine import Engine
+    cfg = P.tiny_config("B")
+    weights = P.random_weights(cfg, 7, bf16_exact=False)
+    kept32 = [k for k in weights if k.endswith(("embed_tokens.weight", "q_proj.weight", "down_proj.weight",
+                                                "input_layernorm.weight"))]
+    assert kept32 and any((weights[k].bfloat16().float() != weights[k].float()).any() for k in kept32)
+    stored = {k: (v.float() if k in kept32 else v.bfloat16()).contiguous() for k, v in weights.items()}
+    folder = str(tmp_path / "mixed")
+    os.makedirs(folder)
+    save_file(stored, os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    eng = Engine.from_folder(folder, dtype="bfloat16", max_slots=2, max_context=128)
+    toks = U.random_tokens(70, cfg["vocab_size"], 5)
+    as_stored = {k: v.double() for k, v in stored.items()}
+    ref = U.plain_logits(cfg, as_stored, toks)
+    bf16_close(U.run_whole(eng, toks), ref, "mixed storage, whole")
+    bf16_close(U.run_tail(eng, toks, 20), ref, "mixed storage, tail")
+    # the 32-bit values took part: rounding them to bfloat16 first gives visibly other logits than the engine's
+    attn0 = eng.model.blocks[0].mixer
+    assert attn0.qkv.packed is None and attn0.qkv.weight.dtype == torch.float32
