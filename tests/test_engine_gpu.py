@@ -194,3 +194,47 @@ def test_tensors_stored_in_32_bit_stay_so_in_a_bfloat16_engine(tmp_path):
     # the 32-bit values took part: rounding them to bfloat16 first gives visibly other logits than the engine's
     attn0 = eng.model.blocks[0].mixer
     assert attn0.qkv.packed is None and attn0.qkv.weight.dtype == torch.float32
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "float32"), ("B", "bfloat16")])
+def test_random_schedules_of_ragged_steps(tmp_path, which, dtype):
+    """Forty steps whose make-up is drawn at random: some sequences bring many tokens and others one
+    in the same step, sequences start and end at any time, slots and pages are used again, and pieces
+    end anywhere relative to page edges and the window.  Every logit row is checked."""
+    import random
+    from agave_amd.engine import Engine
+    cfg = P.tiny_config(which)
+    weights = P.random_weights(cfg, 3)
+    folder = U.write_model(str(tmp_path / "m"), cfg, weights)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=4, max_context=200)
+    rnd = random.Random(17)
+    live = {}                       # slot -> [tokens, reference logits, fed so far]
+    started = 0
+    for it in range(40):
+        while len(live) < 4 and (started < 3 or rnd.random() < 0.5):
+            n = rnd.choice([1, 2, 63, 64, 65, 100, 130, 190])
+            toks = U.random_tokens(n, cfg["vocab_size"], 1000 + started)
+            live[eng.alloc_slot()] = [toks, U.plain_logits(cfg, weights, toks), 0]
+            started += 1
+        chosen = [s for s in live if rnd.random() < 0.8] or list(live)[:1]
+        chunks = []
+        for s in chosen:
+            toks, _, fed = live[s]
+            room = len(toks) - fed
+            k = 1 if rnd.random() < 0.4 else rnd.choice([1, 3, 31, 64, 70])
+            chunks.append(toks[fed:fed + min(k, room)])
+        logits = eng.step(chosen, chunks, "all").float().cpu()
+        o = 0
+        for s, ch in zip(chosen, chunks):
+            toks, ref, fed = live[s]
+            close(dtype)(logits[o:o + len(ch)], ref[fed:fed + len(ch)], f"step {it}, slot {s}, positions {fed}..{fed + len(ch) - 1}")
+            o += len(ch)
+            live[s][2] = fed + len(ch)
+            if live[s][2] == len(toks):
+                eng.free_slot(s)
+                del live[s]
+    for s in list(live):
+        eng.free_slot(s)
+    assert eng.cache.slots.n_free == eng.cache.max_slots
+    for g in eng.cache.groups:
+        assert g.pool.n_free == g.pool.n_pages
