@@ -177,7 +177,10 @@ static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, co
         (out && (ldo % 4 != 0 || (uintptr_t)out % align != 0)) || (uintptr_t)h % 16 != 0 ||
         (post_gain && (uintptr_t)post_gain % 16 != 0) || (pre_gain && (uintptr_t)pre_gain % 16 != 0))
         return false;
-    const int threads = e <= 1024 ? 64 * ((e / 4 + 63) / 64) : (e <= 4096 ? 256 : 1024);
+    // few rows (decode steps): as many threads per row as it has float4, so that every thread's
+    // loads are one round trip; many rows: 256 threads with several float4 each
+    const int threads = (e <= 1024 || (n_rows <= 64 && e <= 4096)) ? 64 * ((e / 4 + 63) / 64)
+                                                                    : (e <= 4096 ? 256 : 1024);
     const int vpt = (e / 4 + threads - 1) / threads;
 #define RN_FAST(V)                                                                                                    \
     residual_norm_fast_kernel<T, V><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, post_gain, post_eps,   \
