@@ -575,6 +575,15 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
     __shared__ float red[16];
     const int t = blockIdx.x / nh, head = blockIdx.x % nh;
     const size_t slot0 = ((size_t)t * nh + head) * splits;
+    // the first splits' partial outputs are requested before anything is waited for (one column
+    // per thread when the block is as wide as the head)
+    constexpr int PRE = 8;
+    float pre[PRE];
+    {
+        const int d = threadIdx.x < hd ? threadIdx.x : 0;
+#pragma unroll
+        for (int sp = 0; sp < PRE; ++sp) pre[sp] = sp < splits ? part_o[(slot0 + sp) * hd + d] : 0.f;
+    }
     // every split's maximum and sum are fetched at once, one split per thread
     float ms[COMBINE_MAX_SPLITS / 64], ls[COMBINE_MAX_SPLITS / 64];
     float m = -INFINITY;
@@ -600,8 +609,11 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
     for (int d = threadIdx.x; d < hd; d += blockDim.x) {
         float acc = 0.f;
         const float* po = part_o + slot0 * hd + d;
-#pragma unroll 8
-        for (int sp = 0; sp < splits; ++sp) acc += po[(size_t)sp * hd] * wgt[sp];
+        const bool first = d == (int)threadIdx.x;          // the columns whose first splits are in registers
+#pragma unroll
+        for (int sp = 0; sp < PRE; ++sp)
+            if (sp < splits) acc += (first ? pre[sp] : po[(size_t)sp * hd]) * wgt[sp];
+        for (int sp = PRE; sp < splits; ++sp) acc += po[(size_t)sp * hd] * wgt[sp];
         out[(size_t)t * ldo + (size_t)head * hd + d] = f32_to_bf16(acc * inv);
     }
 }
