@@ -409,6 +409,12 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
             const bool active = job < jobs, is_q = job < slots;
             const bf16* src = is_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + (active ? job : 0)) * hd
                                    : f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd;
+            bf16 vreg[QK_ROPE_HD_MAX / 64];                      // the value row, requested along with the key's
+#pragma unroll
+            for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) {
+                const int d = lane + 64 * k;
+                vreg[k] = (active && !is_q && d < hd) ? f.v_raw[(size_t)t * f.ldv + (size_t)kvh * hd + d] : bf16{0};
+            }
             qk_norm_rope_wave<bf16>(src, ybuf, is_q ? f.q_gain : f.k_gain, is_q ? f.eps_q : f.eps_k, f.inv_freq,
                                     f.rot_half, pf, hd, lane, active);
             if (active && is_q) {
@@ -425,8 +431,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
                 if (wpg >= 0) {
                     bf16* dk = (bf16*)(a.k_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)4 * KS * 64));
                     bf16* dv = (bf16*)(a.v_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)HDT * 2 * 64));
-                    store_kv_row_packed<bf16>(dk, dv, ybuf, f.v_raw + (size_t)t * f.ldv + (size_t)kvh * hd,
-                                              p % AGAVE_PAGE, hd, lane);
+                    store_kv_row_packed_regs<bf16>(dk, dv, ybuf, vreg, p % AGAVE_PAGE, hd, lane);
                 }
             }
         }

@@ -8,30 +8,50 @@
 // gain may be null (no norm), rot_half 0 (no rotation).  pf: position times the position scale.
 // Every wave of the workgroup calls this together (it holds two workgroup barriers); a wave
 // without work passes active = false.
+#define QK_ROPE_HD_MAX 512
 template <typename T>
 __device__ __forceinline__ void qk_norm_rope_wave(const T* src, float* y, const float* __restrict__ gain, float eps,
                                                   const float* __restrict__ inv_freq, int rot_half, float pf, int hd,
                                                   int lane, bool active) {
+    // everything this needs from memory is requested at once: the row, the gains, the frequencies
+    constexpr int NV = QK_ROPE_HD_MAX / 64;
+    float xv[NV], gv[NV], fv[NV / 2];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int d = lane + 64 * k;
+        xv[k] = (active && d < hd) ? ld(src + d) : 0.f;
+        gv[k] = (active && gain && d < hd) ? gain[d] : 1.f;
+    }
+#pragma unroll
+    for (int k = 0; k < NV / 2; ++k) {
+        const int i = lane + 64 * k;
+        fv[k] = (active && i < rot_half) ? inv_freq[i] : 0.f;
+    }
     float ss = 0.f;
-    if (active)
-        for (int d = lane; d < hd; d += 64) {
-            const float x = ld(src + d);
-            y[d] = x;
-            ss += x * x;
-        }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) ss += xv[k] * xv[k];
+    float inv = 1.0f;
     if (active && gain) {
         ss = wave_sum(ss);
-        const float inv = 1.0f / sqrtf(ss / (float)hd + eps);
-        for (int d = lane; d < hd; d += 64) y[d] = y[d] * inv * gain[d];
+        inv = 1.0f / sqrtf(ss / (float)hd + eps);
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        const int d = lane + 64 * k;
+        if (active && d < hd) y[d] = gain ? xv[k] * inv * gv[k] : xv[k];
     }
     __syncthreads();
     // rotation, in place in LDS: y[i], y[i + rot_half] <- rotated pair
-    for (int i = lane; active && i < rot_half; i += 64) {
-        const float a = y[i], b2 = y[i + rot_half];
-        float s, c;
-        sincosf(pf * inv_freq[i], &s, &c);
-        y[i] = a * c - b2 * s;
-        y[i + rot_half] = a * s + b2 * c;
+#pragma unroll
+    for (int k = 0; k < NV / 2; ++k) {
+        const int i = lane + 64 * k;
+        if (active && i < rot_half) {
+            const float a = y[i], b2 = y[i + rot_half];
+            float s, c;
+            sincosf(pf * fv[k], &s, &c);
+            y[i] = a * c - b2 * s;
+            y[i + rot_half] = a * s + b2 * c;
+        }
     }
     __syncthreads();
 }
@@ -53,5 +73,26 @@ __device__ __forceinline__ void store_kv_row_packed(T* dk, T* dv, const float* y
         st(dk + ((size_t)(kt * ks_n + ks) * 64 + ki + 16 * g) * 8 + e, y[d]);
         const int dt = d >> 4, j = d & 15;
         dv[((size_t)(dt * 2 + s2) * 64 + j + 16 * vg) * 8 + ve] = sv[d];
+    }
+}
+
+// The same with the value row already in registers: vreg[k] is element lane + 64 k.
+template <typename T>
+__device__ __forceinline__ void store_kv_row_packed_regs(T* dk, T* dv, const float* y,
+                                                         const T (&vreg)[QK_ROPE_HD_MAX / 64], int row, int hd,
+                                                         int lane) {
+    const int ks_n = (hd + 31) >> 5;
+    const int kt = row >> 4, ki = row & 15;
+    const int s2 = row >> 5, r32 = row & 31;
+    const int vg = (r32 & 15) >> 2, ve = (r32 & 3) + ((r32 >> 4) << 2);
+#pragma unroll
+    for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) {
+        const int d = lane + 64 * k;
+        if (d < hd) {
+            const int ks = d >> 5, g = (d & 31) >> 3, e = d & 7;
+            st(dk + ((size_t)(kt * ks_n + ks) * 64 + ki + 16 * g) * 8 + e, y[d]);
+            const int dt = d >> 4, j = d & 15;
+            dv[((size_t)(dt * 2 + s2) * 64 + j + 16 * vg) * 8 + ve] = vreg[k];
+        }
     }
 }
