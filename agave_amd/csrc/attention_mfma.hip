@@ -356,12 +356,30 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
 
     constexpr size_t k_stride = (size_t)4 * KS * 64, v_stride = (size_t)HDT * 2 * 64;   // uint4 per (page, kv head)
     const int n_my = (page_hi >= page_lo + wave) ? (page_hi - page_lo - wave) / 4 + 1 : 0; // pages this wave takes
+    // the ids of this wave's first pages are fetched together, ahead of any use: a lookup in the
+    // loop would stand between every two pages
+    constexpr int PG_AHEAD = 8;
+    int pg_pre[PG_AHEAD];
+#pragma unroll
+    for (int i = 1; i < PG_AHEAD; ++i) {
+        const int col = page_lo + wave + 4 * i - first;
+        pg_pre[i] = (a.table_from_reach && i < n_my && col < a.width) ? a.table[(size_t)b * a.width + col] : -1;
+    }
     auto page_id = [&](int i) -> long {          // i-th page of this wave
         const int pi = page_lo + wave + 4 * i;
         long pg;
         if (a.table_from_reach) {
             const int col = pi - first;
-            pg = (i == 0) ? pg0 : (col < a.width ? a.table[(size_t)b * a.width + col] : -1);
+            if (i == 0) {
+                pg = pg0;
+            } else if (i < PG_AHEAD) {
+                pg = -1;
+#pragma unroll
+                for (int k = 1; k < PG_AHEAD; ++k)
+                    if (k == i) pg = pg_pre[k];
+            } else {
+                pg = col < a.width ? a.table[(size_t)b * a.width + col] : -1;
+            }
             if (pg >= a.n_pages) pg = -1;
         } else {
             pg = page_of(a, b, pi);
