@@ -325,6 +325,23 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
     const int slots = (G - chunk * 16 < 16) ? G - chunk * 16 : 16;
     const int t = blockIdx.z, split = blockIdx.x;
+    // FUSED: the first rows of the q/k work are requested before anything else (wave w takes query
+    // head w of the chunk; the wave after the last head takes the key and value rows, in case
+    // this workgroup turns out to be the one that writes them)
+    QkRow row0;
+    bf16 vreg0[QK_ROPE_HD_MAX / 64];
+    const bool row0_q = FUSED && wave < slots, row0_k = FUSED && wave == slots && f.k_raw != nullptr;
+    if constexpr (FUSED) {
+        constexpr int hd0 = HDT * 16;
+        const bf16* src0 = row0_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + wave) * hd0
+                                  : (row0_k ? f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd0 : a.q);
+        row0 = qk_row_load<bf16>(src0, row0_q ? f.q_gain : f.k_gain, f.inv_freq, f.rot_half, hd0, lane, row0_q || row0_k);
+#pragma unroll
+        for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) {
+            const int d = lane + 64 * k;
+            vreg0[k] = (row0_k && d < hd0) ? f.v_raw[(size_t)t * f.ldv + (size_t)kvh * hd0 + d] : bf16{0};
+        }
+    }
     const int b = a.seq_is_token ? t : a.tok_seq[t];
     const int col0 = split * a.pages_per_split + wave;
     long pg0 = -1;
@@ -425,16 +442,24 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
         for (int job0 = 0; job0 < jobs; job0 += 4) {
             const int job = job0 + wave;
             const bool active = job < jobs, is_q = job < slots;
-            const bf16* src = is_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + (active ? job : 0)) * hd
-                                   : f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd;
-            bf16 vreg[QK_ROPE_HD_MAX / 64];                      // the value row, requested along with the key's
+            QkRow row;
+            bf16 vreg[QK_ROPE_HD_MAX / 64];
+            if (job0 == 0) {                       // requested at the kernel's start
+                row = row0;
 #pragma unroll
-            for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) {
-                const int d = lane + 64 * k;
-                vreg[k] = (active && !is_q && d < hd) ? f.v_raw[(size_t)t * f.ldv + (size_t)kvh * hd + d] : bf16{0};
+                for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) vreg[k] = vreg0[k];
+            } else {
+                const bf16* src = is_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + (active ? job : 0)) * hd
+                                       : f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd;
+                row = qk_row_load<bf16>(src, is_q ? f.q_gain : f.k_gain, f.inv_freq, f.rot_half, hd, lane, active);
+#pragma unroll
+                for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) {
+                    const int d = lane + 64 * k;
+                    vreg[k] = (active && !is_q && d < hd) ? f.v_raw[(size_t)t * f.ldv + (size_t)kvh * hd + d] : bf16{0};
+                }
             }
-            qk_norm_rope_wave<bf16>(src, ybuf, is_q ? f.q_gain : f.k_gain, is_q ? f.eps_q : f.eps_k, f.inv_freq,
-                                    f.rot_half, pf, hd, lane, active);
+            qk_row_finish(row, ybuf, (is_q ? f.q_gain : f.k_gain) != nullptr, is_q ? f.eps_q : f.eps_k, f.rot_half, pf,
+                          hd, lane, active);
             if (active && is_q) {
                 for (int d = lane; d < hd; d += 64) q_s[job * hd + d] = f32_to_bf16(ybuf[d]);
             } else if (active) {

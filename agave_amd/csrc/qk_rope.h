@@ -4,41 +4,53 @@
 #pragma once
 #include "common.h"
 
-// y[0..hd) (LDS, 32-bit) <- rotate(src[0..hd) * rsqrt(mean(src^2) + eps) * gain).
-// gain may be null (no norm), rot_half 0 (no rotation).  pf: position times the position scale.
-// Every wave of the workgroup calls this together (it holds two workgroup barriers); a wave
-// without work passes active = false.
 #define QK_ROPE_HD_MAX 512
+// What one wave holds of a head's row between asking memory for it and using it: lane l has the
+// elements l, l + 64, ... with their gains, and the frequencies of the pairs l, l + 64, ...
+struct QkRow {
+    float xv[QK_ROPE_HD_MAX / 64], gv[QK_ROPE_HD_MAX / 64], fv[QK_ROPE_HD_MAX / 128];
+};
+
+// Requests the row, the gains and the frequencies; nothing is waited for here, so a kernel can
+// call this first and let the loads travel while it finds out the position.
 template <typename T>
-__device__ __forceinline__ void qk_norm_rope_wave(const T* src, float* y, const float* __restrict__ gain, float eps,
-                                                  const float* __restrict__ inv_freq, int rot_half, float pf, int hd,
-                                                  int lane, bool active) {
-    // everything this needs from memory is requested at once: the row, the gains, the frequencies
-    constexpr int NV = QK_ROPE_HD_MAX / 64;
-    float xv[NV], gv[NV], fv[NV / 2];
+__device__ __forceinline__ QkRow qk_row_load(const T* src, const float* __restrict__ gain,
+                                             const float* __restrict__ inv_freq, int rot_half, int hd, int lane,
+                                             bool active) {
+    QkRow r;
 #pragma unroll
-    for (int k = 0; k < NV; ++k) {
+    for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) {
         const int d = lane + 64 * k;
-        xv[k] = (active && d < hd) ? ld(src + d) : 0.f;
-        gv[k] = (active && gain && d < hd) ? gain[d] : 1.f;
+        r.xv[k] = (active && d < hd) ? ld(src + d) : 0.f;
+        r.gv[k] = (active && gain && d < hd) ? gain[d] : 1.f;
     }
 #pragma unroll
-    for (int k = 0; k < NV / 2; ++k) {
+    for (int k = 0; k < QK_ROPE_HD_MAX / 128; ++k) {
         const int i = lane + 64 * k;
-        fv[k] = (active && i < rot_half) ? inv_freq[i] : 0.f;
+        r.fv[k] = (active && i < rot_half) ? inv_freq[i] : 0.f;
     }
+    return r;
+}
+
+// y[0..hd) (LDS, 32-bit) <- rotate(row * rsqrt(mean(row^2) + eps) * gain) for the row that qk_row_load
+// fetched.  has_gain false: no norm; rot_half 0: no rotation.  pf: position times the position
+// scale.  Every wave of the workgroup calls this together (it holds two workgroup barriers); a
+// wave without work passes active = false.
+__device__ __forceinline__ void qk_row_finish(const QkRow& r, float* y, bool has_gain, float eps, int rot_half,
+                                              float pf, int hd, int lane, bool active) {
+    constexpr int NV = QK_ROPE_HD_MAX / 64;
     float ss = 0.f;
 #pragma unroll
-    for (int k = 0; k < NV; ++k) ss += xv[k] * xv[k];
+    for (int k = 0; k < NV; ++k) ss += r.xv[k] * r.xv[k];
     float inv = 1.0f;
-    if (active && gain) {
+    if (active && has_gain) {
         ss = wave_sum(ss);
         inv = 1.0f / sqrtf(ss / (float)hd + eps);
     }
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         const int d = lane + 64 * k;
-        if (active && d < hd) y[d] = gain ? xv[k] * inv * gv[k] : xv[k];
+        if (active && d < hd) y[d] = has_gain ? r.xv[k] * inv * r.gv[k] : r.xv[k];
     }
     __syncthreads();
     // rotation, in place in LDS: y[i], y[i + rot_half] <- rotated pair
@@ -48,12 +60,21 @@ __device__ __forceinline__ void qk_norm_rope_wave(const T* src, float* y, const 
         if (active && i < rot_half) {
             const float a = y[i], b2 = y[i + rot_half];
             float s, c;
-            sincosf(pf * fv[k], &s, &c);
+            sincosf(pf * r.fv[k], &s, &c);
             y[i] = a * c - b2 * s;
             y[i + rot_half] = a * s + b2 * c;
         }
     }
     __syncthreads();
+}
+
+// Both at once.
+template <typename T>
+__device__ __forceinline__ void qk_norm_rope_wave(const T* src, float* y, const float* __restrict__ gain, float eps,
+                                                  const float* __restrict__ inv_freq, int rot_half, float pf, int hd,
+                                                  int lane, bool active) {
+    const QkRow r = qk_row_load<T>(src, gain, inv_freq, rot_half, hd, lane, active);
+    qk_row_finish(r, y, gain != nullptr, eps, rot_half, pf, hd, lane, active);
 }
 
 // One wave writes a key row y[0..hd) (LDS) and a value row sv[0..hd) to row `row` of a page in tile
