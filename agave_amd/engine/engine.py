@@ -61,6 +61,13 @@ class Engine:
         self.spec = spec
         self.config = config
         torch.cuda.set_device(self.device)
+        # what this element type needs is compiled now, side by side, rather than one library
+        # after the other as the first step meets them (a fresh checkout's first run)
+        from ..ops import library
+        needed = ["elementwise", "gemm", "attention_plain", "sampling"]
+        if self.dtype == torch.bfloat16:
+            needed += ["gemm_mfma", "attention_mfma"]
+        library.ensure_built(needed)
         self.workspace = Workspace(self.device)
         self.env = BuildEnv(self.dtype, self.device, self.workspace)
         self.model = Model(spec, weights, self.env)
