@@ -260,14 +260,6 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     }
 }
 
-// A choice of R and NW forced from outside (0: the heuristics below); for measurements only.
-static int g_skinny_force_r = 0, g_skinny_force_nw = 0;
-extern "C" int agave_gemm_skinny_tune(int r, int nw) {
-    g_skinny_force_r = r;
-    g_skinny_force_nw = nw;
-    return 0;
-}
-
 template <int R, int MT, int EPI, int NW, typename TC, int XR>
 static void launch_skinny_nw(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                              int NB, hipStream_t stream) {
@@ -280,7 +272,6 @@ static void launch_skinny_nw(const void* X, long ldx, const void* Wp, void* Y, l
 // or three chunks of loads in flight, which covers the memory's latency with few waves; more
 // waves only add to the merge of the sums and deal the chunks less evenly.
 static int skinny_waves(int groups, int n_chunks, int max_nw) {
-    if (g_skinny_force_nw) return g_skinny_force_nw <= max_nw ? g_skinny_force_nw : max_nw;
     int nw = 4;
     while (nw < max_nw && (long)groups * nw < 640 && nw < n_chunks) nw *= 2;
     return nw;
@@ -313,8 +304,6 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
     if (mt == 1) r = NB >= 4096 ? 2 : 1;
     else if (mt == 2) r = NB >= 4096 ? 4 : (NB >= 1024 ? 2 : 1);
     else r = NB >= 1024 ? 4 : 1;
-    if (g_skinny_force_r) r = g_skinny_force_r;
-    if (mt <= 1 && r > 2) r = 2;
 #define SK_CASE(R_, MT_)                                                                        \
     launch_skinny<R_, MT_, EPI, TC, 16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);          \
     break
@@ -330,10 +319,8 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
         case 2 * 8 + 2: SK_CASE(2, 2);
         case 2 * 8 + 4: SK_CASE(4, 2);
         case 3 * 8 + 1: SK_CASE(1, 3);
-        case 3 * 8 + 2: SK_CASE(2, 3);
         case 3 * 8 + 4: SK_CASE(4, 3);
         case 4 * 8 + 1: SK_CASE(1, 4);
-        case 4 * 8 + 2: SK_CASE(2, 4);
         case 4 * 8 + 4: SK_CASE(4, 4);
         default: AGAVE_CHECK(false, "gemm_skinny: no kernel for %d tokens with %d row blocks a workgroup", M, r);
     }
@@ -548,22 +535,11 @@ static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long l
     return 0;
 }
 
-// A configuration forced from outside (0: the rule below); for measurements only.
-static int g_tiled_force = 0;
-extern "C" int agave_gemm_tiled_tune(int which) {
-    g_tiled_force = which;
-    return 0;
-}
-
 template <int EPI, typename TC>
 static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                           int NB, hipStream_t stream) {
     // the larger tile once it still gives every compute unit two workgroups
     const long big = (long)((NB + 15) / 16) * ((M + 255) / 256);
-    if (g_tiled_force == 1) return launch_tiled<4, 1, 4, EPI, TC, 4>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-    if (g_tiled_force == 2) return launch_tiled<2, 2, 3, EPI, TC, 4>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-    if (g_tiled_force == 3) return launch_tiled<4, 1, 4, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-    if (g_tiled_force == 4) return launch_tiled<2, 2, 3, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     if (big >= 512) return launch_tiled<4, 1, 4, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     return launch_tiled<2, 2, 3, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
 }
