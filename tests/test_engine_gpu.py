@@ -23,9 +23,12 @@ def bf16_close(got: torch.Tensor, ref: torch.Tensor, what: str):
     assert float(err.max()) < 0.04, f"{what}: relative error {float(err.max()):.4f} at position {worst}"
 
 
-def f32_close(got: torch.Tensor, ref: torch.Tensor, what: str):
+def f32_close(got: torch.Tensor, ref: torch.Tensor, what: str, longer_sums: float = 1.0):
+    """``longer_sums``: how many times longer the model's dot products are than the tiny
+    configurations' (a few hundred terms); the rounding error of a 32-bit sum grows with the
+    root of its length."""
     diff = (got.double() - ref).abs()
-    tol = F32_ATOL + F32_RTOL * ref.abs()
+    tol = (F32_ATOL + F32_RTOL * ref.abs()) * longer_sums ** 0.5
     bad = (diff > tol).any(dim=-1)
     if bad.any():
         first = int(torch.nonzero(bad)[0])
@@ -238,3 +241,33 @@ def test_random_schedules_of_ragged_steps(tmp_path, which, dtype):
     assert eng.cache.slots.n_free == eng.cache.max_slots
     for g in eng.cache.groups:
         assert g.pool.n_free == g.pool.n_pages
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_layers_of_the_benchmark_sizes(tmp_path, dtype):
+    """Two layers with the 4B model's own sizes (width 2560, 8 query and 4 kv heads of 256, 10240
+    inner columns, window 1024, the second layer global with its scaled rope) and a small
+    vocabulary: a prompt that ends just short of the window's reach, then steps across it."""
+    from agave_amd.engine import Engine
+    cfg = dict(P.tiny_config("A"), vocab_size=1536, hidden_size=2560, num_hidden_layers=2, num_attention_heads=8,
+               num_key_value_heads=4, head_dim=256, query_pre_attn_scalar=256, intermediate_size=10240,
+               sliding_window=1024, sliding_window_pattern=2, rope_theta=1e6, rope_local_base_freq=1e4,
+               rope_scaling={"rope_type": "linear", "factor": 8.0}, rms_norm_eps=1e-6,
+               max_position_embeddings=4096)
+    cfg.pop("layer_types", None)
+    weights = P.random_weights(cfg, 11)
+    folder = U.write_model(str(tmp_path / "m"), cfg, weights)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=2, max_context=1152)
+    toks = U.random_tokens(1060, cfg["vocab_size"], 12)
+    n_prompt = 1015
+    ref = U.plain_logits(cfg, weights, toks)
+    slot = eng.alloc_slot()
+    got = [eng.step([slot], [toks[:n_prompt]], [[0, 1, 511, 1013, 1014]]).float().cpu().clone()]
+    for t in toks[n_prompt:]:
+        got.append(eng.step([slot], [[t]], "last").float().cpu().clone())
+    eng.free_slot(slot)
+    rows = [0, 1, 511, 1013, 1014] + list(range(n_prompt, len(toks)))
+    if dtype == "float32":
+        f32_close(torch.cat(got, 0), ref[rows], "benchmark-sized layers", longer_sums=10240 / 320)
+    else:
+        bf16_close(torch.cat(got, 0), ref[rows], "benchmark-sized layers")
