@@ -243,31 +243,41 @@ def test_random_schedules_of_ragged_steps(tmp_path, which, dtype):
         assert g.pool.n_free == g.pool.n_pages
 
 
+BIG_LAYERS = {
+    # the 4B model's layers: width 2560, 8 query and 4 kv heads of 256, 10240 inner columns, window 1024
+    "4b": (dict(hidden_size=2560, num_attention_heads=8, num_key_value_heads=4, head_dim=256, query_pre_attn_scalar=256,
+                intermediate_size=10240, sliding_window=1024), 1060, 1015),
+    # the 27B model's: width 5376, 32 query and 16 kv heads of 128, a scale that is not the head size;
+    # a shorter window so that the plain implementation stays quick
+    "27b": (dict(hidden_size=5376, num_attention_heads=32, num_key_value_heads=16, head_dim=128,
+                 query_pre_attn_scalar=168, intermediate_size=21504, sliding_window=256), 300, 250),
+}
+
+
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
-def test_layers_of_the_benchmark_sizes(tmp_path, dtype):
-    """Two layers with the 4B model's own sizes (width 2560, 8 query and 4 kv heads of 256, 10240
-    inner columns, window 1024, the second layer global with its scaled rope) and a small
-    vocabulary: a prompt that ends just short of the window's reach, then steps across it."""
+@pytest.mark.parametrize("size", sorted(BIG_LAYERS))
+def test_layers_of_the_published_sizes(tmp_path, dtype, size):
+    """Two layers with a published model's own sizes (the second one global with its scaled rope) and
+    a small vocabulary: a prompt that ends just short of the window's reach, then steps across it."""
     from agave_amd.engine import Engine
-    cfg = dict(P.tiny_config("A"), vocab_size=1536, hidden_size=2560, num_hidden_layers=2, num_attention_heads=8,
-               num_key_value_heads=4, head_dim=256, query_pre_attn_scalar=256, intermediate_size=10240,
-               sliding_window=1024, sliding_window_pattern=2, rope_theta=1e6, rope_local_base_freq=1e4,
-               rope_scaling={"rope_type": "linear", "factor": 8.0}, rms_norm_eps=1e-6,
-               max_position_embeddings=4096)
+    sizes, n_all, n_prompt = BIG_LAYERS[size]
+    cfg = dict(P.tiny_config("A"), vocab_size=1536, num_hidden_layers=2, sliding_window_pattern=2, rope_theta=1e6,
+               rope_local_base_freq=1e4, rope_scaling={"rope_type": "linear", "factor": 8.0}, rms_norm_eps=1e-6,
+               max_position_embeddings=4096, **sizes)
     cfg.pop("layer_types", None)
     weights = P.random_weights(cfg, 11)
     folder = U.write_model(str(tmp_path / "m"), cfg, weights)
     eng = Engine.from_folder(folder, dtype=dtype, max_slots=2, max_context=1152)
-    toks = U.random_tokens(1060, cfg["vocab_size"], 12)
-    n_prompt = 1015
+    toks = U.random_tokens(n_all, cfg["vocab_size"], 12)
     ref = U.plain_logits(cfg, weights, toks)
+    first = [0, 1, n_prompt // 2, n_prompt - 2, n_prompt - 1]
     slot = eng.alloc_slot()
-    got = [eng.step([slot], [toks[:n_prompt]], [[0, 1, 511, 1013, 1014]]).float().cpu().clone()]
+    got = [eng.step([slot], [toks[:n_prompt]], [first]).float().cpu().clone()]
     for t in toks[n_prompt:]:
         got.append(eng.step([slot], [[t]], "last").float().cpu().clone())
     eng.free_slot(slot)
-    rows = [0, 1, 511, 1013, 1014] + list(range(n_prompt, len(toks)))
+    rows = first + list(range(n_prompt, len(toks)))
     if dtype == "float32":
-        f32_close(torch.cat(got, 0), ref[rows], "benchmark-sized layers", longer_sums=10240 / 320)
+        f32_close(torch.cat(got, 0), ref[rows], f"{size} layers", longer_sums=sizes["intermediate_size"] / 320)
     else:
-        bf16_close(torch.cat(got, 0), ref[rows], "benchmark-sized layers")
+        bf16_close(torch.cat(got, 0), ref[rows], f"{size} layers")
