@@ -281,3 +281,25 @@ def test_layers_of_the_published_sizes(tmp_path, dtype, size):
         f32_close(torch.cat(got, 0), ref[rows], f"{size} layers", longer_sums=sizes["intermediate_size"] / 320)
     else:
         bf16_close(torch.cat(got, 0), ref[rows], f"{size} layers")
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_sizes_that_fit_no_fast_kernel(tmp_path, dtype):
+    """Width 100 and inner size 52 (no multiples of 8), heads of 20 (no multiple of 16), an odd
+    vocabulary, a window of 1: every matrix-core kernel refuses these, and the engine takes the
+    plain kernels instead of giving a wrong result."""
+    from agave_amd.engine import Engine
+    cfg = dict(P.tiny_config("A"), vocab_size=333, hidden_size=100, num_hidden_layers=3, num_attention_heads=5,
+               num_key_value_heads=5, head_dim=20, query_pre_attn_scalar=7, intermediate_size=52,
+               sliding_window=1, sliding_window_pattern=3, rms_norm_eps=3e-4)
+    cfg.pop("layer_types", None)
+    weights = P.random_weights(cfg, 21)
+    folder = U.write_model(str(tmp_path / "m"), cfg, weights)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=3, max_context=160)
+    toks = U.random_tokens(130, cfg["vocab_size"], 22)
+    ref = U.plain_logits(cfg, weights, toks)
+    close(dtype)(U.run_whole(eng, toks), ref, "whole")
+    close(dtype)(U.run_tail(eng, toks, 32), ref, "tail")
+    outs = U.run_batched(eng, [toks, toks[:70], toks[:9]], (90, 69, 1))
+    for o, n in zip(outs, (130, 70, 9)):
+        close(dtype)(o, ref[:n], f"batched, {n} tokens")
