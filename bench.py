@@ -85,11 +85,11 @@ def random_prompts(n: int, length: int, vocab: int, seed: int):
     return [rng.integers(0, vocab, size=length).tolist() for _ in range(n)]
 
 
-def run_decode(engine, batch: int, steps: int, warmup: int, seed: int):
-    """Prefill ``batch`` prompts of PROMPT_LEN tokens, then time ``steps`` decode steps."""
+def run_decode(engine, batch: int, steps: int, warmup: int, seed: int, prompt_len: int = PROMPT_LEN):
+    """Prefill ``batch`` prompts of ``prompt_len`` tokens, then time ``steps`` decode steps."""
     import torch
     from agave_amd.engine.generate import RowSampling
-    prompts = random_prompts(batch, PROMPT_LEN, engine.vocab_size, seed)
+    prompts = random_prompts(batch, prompt_len, engine.vocab_size, seed)
     slots = [engine.alloc_slot() for _ in range(batch)]
     rows = [RowSampling(0.0, 0, 1.0, 1.0, 0.0, []) for _ in range(batch)]
     try:
@@ -116,7 +116,7 @@ def run_decode(engine, batch: int, steps: int, warmup: int, seed: int):
         toks = engine.finish_step(running)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        first_ctx = PROMPT_LEN + warmup + 1          # keys the first timed step attends to
+        first_ctx = prompt_len + warmup + 1          # keys the first timed step attends to
         contexts = [first_ctx + (steps - 1) / 2.0] * batch
         return dt, contexts
     finally:
@@ -155,6 +155,9 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=0,
                     help="run fewer layers of the same sizes (reported in config)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
+                    help="tokens of every prompt before the decode steps (the default run: 1024)")
+    ap.add_argument("--context", type=int, default=CONTEXT, help="longest sequence a slot may hold")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the 2048-token prefill and print its record (for profiles)")
@@ -164,8 +167,8 @@ def main() -> int:
         if int(os.environ.get("RANK", "0")) == 0:
             print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
-    if args.steps + args.warmup > CONTEXT - PROMPT_LEN:
-        ap.error(f"--steps + --warmup must stay within {CONTEXT - PROMPT_LEN} decoded tokens")
+    if args.steps + args.warmup > args.context - args.prompt_len:
+        ap.error(f"--steps + --warmup must stay within {args.context - args.prompt_len} decoded tokens")
 
     import torch
     from agave_amd.engine import Engine
@@ -176,9 +179,9 @@ def main() -> int:
     cfg = dict(full, num_hidden_layers=args.layers)
     m = model_numbers(cfg, args.layers)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    per_seq = -(-(PROMPT_LEN + DECODE_LEN + 64) // 64) * 64
+    per_seq = -(-(args.prompt_len + max(DECODE_LEN, args.steps + args.warmup) + 64) // 64) * 64
     cache_tokens = max(max_batch * per_seq, -(-PREFILL_LEN // 64) * 64 + 64)
-    engine = Engine.from_random(cfg, seed=0, dtype=args.dtype, max_slots=max_batch, max_context=CONTEXT,
+    engine = Engine.from_random(cfg, seed=0, dtype=args.dtype, max_slots=max_batch, max_context=args.context,
                                 cache_tokens=cache_tokens, device="cuda:0")
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     if args.prefill_only:
@@ -189,13 +192,13 @@ def main() -> int:
               flush=True)
         return 0
 
-    dt, contexts = run_decode(engine, args.batch, args.steps, args.warmup, seed=1)
+    dt, contexts = run_decode(engine, args.batch, args.steps, args.warmup, seed=1, prompt_len=args.prompt_len)
     ms_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     need = decode_step_bytes(m, contexts)
     achieved = need / (ms_step * 1e-3) / 1e9
     out = {
-        "metric": f"decode tok/s, Gemma3-{args.model.upper()} {dkey}, batch {args.batch}, 1024-token prompts + 256 decoded",
+        "metric": f"decode tok/s, Gemma3-{args.model.upper()} {dkey}, batch {args.batch}, {args.prompt_len}-token prompts + 256 decoded",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dkey, "data": "synthetic: uniform-random token ids, random N(0,0.02) weights",
@@ -203,8 +206,8 @@ def main() -> int:
                    "hidden": m["e"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                    "head_dim": cfg["head_dim"], "intermediate": m["ff"], "vocab": m["v"],
                    "sliding_window": m["window"], "sliding_pattern": cfg["sliding_window_pattern"],
-                   "global_batch": args.batch, "seq_len": PROMPT_LEN + DECODE_LEN, "prompt_len": PROMPT_LEN,
-                   "context": CONTEXT, "prefill_len": PREFILL_LEN, "parallelism": "single GPU",
+                   "global_batch": args.batch, "seq_len": args.prompt_len + DECODE_LEN, "prompt_len": args.prompt_len,
+                   "context": args.context, "prefill_len": PREFILL_LEN, "parallelism": "single GPU",
                    "sampling": "greedy", "weights_gb": round(2 * (m["linear_params"] + m["table_params"]) / 1e9, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
