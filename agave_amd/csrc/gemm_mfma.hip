@@ -373,16 +373,17 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
 // the number of row tiles apart) tend to land on the same XCD and find them in its L2.
 typedef __attribute__((address_space(3))) u32x4_t tl_lds_u32x4;
 
-template <int WT, int KT, int NS, int EPI, typename TC, int NWV>
+template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT>
 __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
                                                          const uint4* __restrict__ Wp, TC* __restrict__ Y, long ldy,
                                                          int M, int N, int K, int KB, int NB) {
     constexpr int CPR = KT * 4;                       // 16-byte pieces per staged token row
     constexpr int RP = 16 / CPR;                      // token rows per 256 bytes of LDS
     constexpr int WTILES = 4 * WT;                    // packed 16-row weight tiles per workgroup
-    constexpr int X_BYTES = 256 * KT * 64, W_BYTES = WTILES * KT * 1024;
+    constexpr int X_BYTES = TT * KT * 64, W_BYTES = WTILES * KT * 1024;      // TT tokens per workgroup
     constexpr int STAGE_BYTES = X_BYTES + W_BYTES;
-    constexpr int XB = 16 / NWV;                      // 32-token tiles per wave: 4 (four waves, 2 x 2) or 2 (eight, 2 x 4)
+    constexpr int XB = (TT / 32) / (NWV / 2);         // 32-token tiles per wave
+    static_assert(XB >= 1 && XB * (NWV / 2) * 32 == TT, "the waves' token tiles must cover the workgroup's tokens");
     constexpr int X_LOADS = X_BYTES / 1024 / NWV, W_LOADS = W_BYTES / 1024 / NWV;     // per wave and stage
     static_assert(NWV == 4 || NWV == 8, "four or eight waves");
     static_assert(X_LOADS * NWV * 1024 == X_BYTES && W_LOADS * NWV * 1024 == W_BYTES, "whole loads per wave");
@@ -393,7 +394,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int wn = wave & 1, wm = wave >> 1;
     const int nbw = blockIdx.x * WTILES;                  // first packed weight tile of this workgroup
-    const int m0 = blockIdx.y * 256;                      // first token of this workgroup
+    const int m0 = blockIdx.y * TT;                       // first token of this workgroup
     const int n_stage = (KB + KT - 1) / KT;
     const int i32 = lane & 31, kg = lane >> 5;
 
@@ -516,21 +517,21 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
     }
 }
 
-template <int WT, int KT, int NS, int EPI, typename TC, int NWV>
+template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT>
 static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB, int NB,
                         hipStream_t stream) {
     constexpr int WTILES = 4 * WT;
-    const size_t lds = (size_t)NS * (256 * KT * 64 + WTILES * KT * 1024);
-    dim3 grid((NB + WTILES - 1) / WTILES, (M + 255) / 256);
+    const size_t lds = (size_t)NS * (TT * KT * 64 + WTILES * KT * 1024);
+    dim3 grid((NB + WTILES - 1) / WTILES, (M + TT - 1) / TT);
     AGAVE_CHECK(grid.y <= 65535, "gemm_tiled: M=%d exceeds the grid limit", M);
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         AGAVE_CHECK(e == hipSuccess, "gemm_tiled: cannot raise the LDS allowance");
         raised = true;
     }
-    gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
+    gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
                                                                       M, N, K, KB, NB);
     return 0;
 }
@@ -538,10 +539,27 @@ static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long l
 template <int EPI, typename TC>
 static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                           int NB, hipStream_t stream) {
-    // the larger tile once it still gives every compute unit two workgroups
-    const long big = (long)((NB + 15) / 16) * ((M + 255) / 256);
-    if (big >= 512) return launch_tiled<4, 1, 4, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-    return launch_tiled<2, 2, 3, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    // The largest tile that still gives some 160 workgroups (a larger tile reads a third less from
+    // L2 per flop, which outweighs idle compute units down to about that number); with few tokens
+    // or few rows none does, and the tile with the most workgroups is taken.
+    //   256 x 256, 128 x 256, 128 x 128, 64 x 128 (weight rows x tokens)
+    const long rows16 = (NB + 15) / 16, rows8 = (NB + 7) / 8, rows4 = (NB + 3) / 4;
+    const long t256 = (M + 255) / 256, t128 = (M + 127) / 128;
+    const long wgs[4] = {rows16 * t256, rows8 * t256, rows8 * t128, rows4 * t128};
+    int pick = -1;
+    for (int i = 0; i < 4 && pick < 0; ++i)
+        if (wgs[i] >= 160) pick = i;
+    if (pick < 0) {
+        pick = 0;
+        for (int i = 1; i < 4; ++i)
+            if (wgs[i] > wgs[pick]) pick = i;
+    }
+    switch (pick) {
+        case 0: return launch_tiled<4, 1, 4, EPI, TC, 8, 256>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 1: return launch_tiled<2, 2, 3, EPI, TC, 8, 256>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 2: return launch_tiled<2, 2, 3, EPI, TC, 8, 128>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        default: return launch_tiled<1, 2, 4, EPI, TC, 8, 128>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    }
 }
 
 extern "C" int agave_gemm_tiled(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,

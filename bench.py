@@ -125,10 +125,10 @@ def run_decode(engine, batch: int, steps: int, warmup: int, seed: int, prompt_le
         engine.prefill_chunk = 0
 
 
-def run_prefill(engine, seed: int, repeats: int = 3):
+def run_prefill(engine, seed: int, repeats: int = 3, length: int = PREFILL_LEN):
     import torch
     from agave_amd.engine.generate import RowSampling
-    prompt = random_prompts(1, PREFILL_LEN, engine.vocab_size, seed)
+    prompt = random_prompts(1, length, engine.vocab_size, seed)
     row = [RowSampling(0.0, 0, 1.0, 1.0, 0.0, [])]
     times = []
     for r in range(repeats + 1):                     # the first pass warms up
@@ -158,6 +158,7 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN,
                     help="tokens of every prompt before the decode steps (the default run: 1024)")
     ap.add_argument("--context", type=int, default=CONTEXT, help="longest sequence a slot may hold")
+    ap.add_argument("--prefill-len", type=int, default=PREFILL_LEN, help="tokens of the prefill prompt (the default run: 2048)")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the 2048-token prefill and print its record (for profiles)")
@@ -180,15 +181,15 @@ def main() -> int:
     m = model_numbers(cfg, args.layers)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     per_seq = -(-(args.prompt_len + max(DECODE_LEN, args.steps + args.warmup) + 64) // 64) * 64
-    cache_tokens = max(max_batch * per_seq, -(-PREFILL_LEN // 64) * 64 + 64)
+    cache_tokens = max(max_batch * per_seq, -(-max(PREFILL_LEN, args.prefill_len) // 64) * 64 + 64)
     engine = Engine.from_random(cfg, seed=0, dtype=args.dtype, max_slots=max_batch, max_context=args.context,
                                 cache_tokens=cache_tokens, device="cuda:0")
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
     if args.prefill_only:
-        pdt = run_prefill(engine, seed=2)
-        print(json.dumps({"prefill": {"value": round(PREFILL_LEN / pdt, 1), "tokens": PREFILL_LEN,
+        pdt = run_prefill(engine, seed=2, length=args.prefill_len)
+        print(json.dumps({"prefill": {"value": round(args.prefill_len / pdt, 1), "tokens": args.prefill_len,
                                       "ms": round(pdt * 1e3, 3),
-                                      "frac": round(prefill_flops(m, PREFILL_LEN) / pdt / PEAK_FLOPS[dkey], 4)}}),
+                                      "frac": round(prefill_flops(m, args.prefill_len) / pdt / PEAK_FLOPS[dkey], 4)}}),
               flush=True)
         return 0
 
