@@ -376,7 +376,7 @@ typedef __attribute__((address_space(3))) u32x4_t tl_lds_u32x4;
 template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT>
 __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
                                                          const uint4* __restrict__ Wp, TC* __restrict__ Y, long ldy,
-                                                         int M, int N, int K, int KB, int NB) {
+                                                         int M, int N, int K, int KB, int NB, long part_stride) {
     constexpr int CPR = KT * 4;                       // 16-byte pieces per staged token row
     constexpr int RP = 16 / CPR;                      // token rows per 256 bytes of LDS
     constexpr int WTILES = 4 * WT;                    // packed 16-row weight tiles per workgroup
@@ -395,7 +395,12 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
     const int wn = wave & 1, wm = wave >> 1;
     const int nbw = blockIdx.x * WTILES;                  // first packed weight tile of this workgroup
     const int m0 = blockIdx.y * TT;                       // first token of this workgroup
-    const int n_stage = (KB + KT - 1) / KT;
+    // gridDim.z workgroups share a tile's columns: each takes a run of stages and leaves its sum
+    // in its own slice of Y (a buffer of partial sums then, added up by gemm_sum_parts_kernel)
+    const int n_stage_all = (KB + KT - 1) / KT;
+    const int st0 = (int)((long)blockIdx.z * n_stage_all / gridDim.z);
+    const int n_stage = (int)((long)(blockIdx.z + 1) * n_stage_all / gridDim.z);      // one past this workgroup's last stage
+    Y += (size_t)blockIdx.z * part_stride;
     const int i32 = lane & 31, kg = lane >> 5;
 
     f32x16_t acc[WT][XB];
@@ -441,8 +446,8 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
 
 #pragma unroll
     for (int s0 = 0; s0 < NS - 1; ++s0)
-        if (s0 < n_stage) fetch(s0);
-    for (int st = 0; st < n_stage; ++st) {
+        if (st0 + s0 < n_stage) fetch(st0 + s0);
+    for (int st = st0; st < n_stage; ++st) {
         // stage st has landed once at most the loads of the NS-2 stages after it are outstanding
         const int ahead = (n_stage - 1 - st < NS - 2) ? n_stage - 1 - st : NS - 2;
         if (ahead >= 3) __builtin_amdgcn_s_waitcnt(0x0F70 | ((3 * LOADS) & 15) | (((3 * LOADS) >> 4) << 14));
@@ -519,10 +524,10 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
 
 template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT>
 static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB, int NB,
-                        hipStream_t stream) {
+                        hipStream_t stream, int splits = 1, long part_stride = 0) {
     constexpr int WTILES = 4 * WT;
     const size_t lds = (size_t)NS * (TT * KT * 64 + WTILES * KT * 1024);
-    dim3 grid((NB + WTILES - 1) / WTILES, (M + TT - 1) / TT);
+    dim3 grid((NB + WTILES - 1) / WTILES, (M + TT - 1) / TT, splits);
     AGAVE_CHECK(grid.y <= 65535, "gemm_tiled: M=%d exceeds the grid limit", M);
     static bool raised = false;
     if (!raised) {
@@ -532,13 +537,24 @@ static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long l
         raised = true;
     }
     gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
-                                                                      M, N, K, KB, NB);
+                                                                      M, N, K, KB, NB, part_stride);
     return 0;
+}
+
+// Y[m][n] = sum over the splits' partial sums
+template <typename TC>
+__global__ void gemm_sum_parts_kernel(const float* __restrict__ part, int splits, long part_stride, TC* __restrict__ Y,
+                                      long ldy, int M, int N) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;        // one output each
+    if (i >= (long)M * N) return;
+    float s = 0.f;
+    for (int z = 0; z < splits; ++z) s += part[(size_t)z * part_stride + i];
+    st(Y + (size_t)(i / N) * ldy + i % N, s);
 }
 
 template <int EPI, typename TC>
 static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
-                          int NB, hipStream_t stream) {
+                          int NB, float* part, long part_elems, hipStream_t stream) {
     // The largest tile that still gives some 160 workgroups (a larger tile reads a third less from
     // L2 per flop, which outweighs idle compute units down to about that number); with few tokens
     // or few rows none does, and the tile with the most workgroups is taken.
@@ -554,6 +570,28 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
         for (int i = 1; i < 4; ++i)
             if (wgs[i] > wgs[pick]) pick = i;
     }
+    // Still few workgroups and many columns: several workgroups share a tile's columns and leave
+    // partial sums (32-bit, in a buffer the caller lends), which a second kernel adds up.
+    int splits = 1;
+    if (EPI == 0 && part != nullptr && wgs[pick] < 160) {
+        const int n_stage = (KB + 1) / 2;                 // the two small tiles take two k-steps a stage
+        splits = (int)((256 + wgs[pick] - 1) / wgs[pick]);
+        if (splits > 8) splits = 8;
+        if (splits > K / (4 * M)) splits = K / (4 * M);       // the partial sums' traffic stays well below the weights'
+        while (splits > 1 && (n_stage / splits < 8 || (long)splits * M * N > part_elems)) --splits;
+        if (splits < 1) splits = 1;
+    }
+    if (splits > 1) {
+        const long stride = (long)M * N;
+        int rc;
+        if (pick == 2) rc = launch_tiled<2, 2, 3, 0, float, 8, 128>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
+        else rc = launch_tiled<1, 2, 4, 0, float, 8, 128>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
+        if (rc != 0) return rc;
+        AGAVE_LAUNCH_CHECK("gemm_tiled (partial sums)");
+        const long total = (long)M * N;
+        gemm_sum_parts_kernel<TC><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(part, splits, stride, (TC*)Y, ldy, M, N);
+        return 0;
+    }
     switch (pick) {
         case 0: return launch_tiled<4, 1, 4, EPI, TC, 8, 256>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
         case 1: return launch_tiled<2, 2, 3, EPI, TC, 8, 256>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
@@ -562,8 +600,11 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
     }
 }
 
+// N: logical outputs (rows of W, or ff for the GeGLU epilogue); Wp holds NB row blocks.  part: an
+// optional buffer of part_elems floats for partial sums (products with few tiles and many columns
+// are then shared out along the columns); null: never.
 extern "C" int agave_gemm_tiled(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,
-                                int K, int epilogue, hipStream_t stream) {
+                                int K, int epilogue, float* part, long part_elems, hipStream_t stream) {
     AGAVE_CHECK(M >= 0 && N > 0 && K > 0, "gemm_tiled: bad sizes M=%d N=%d K=%d", M, N, K);
     AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
                 "gemm_tiled: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
@@ -574,12 +615,12 @@ extern "C" int agave_gemm_tiled(const void* X, long ldx, const void* Wp, int dt_
     const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
     int rc;
     if (epilogue == 0) {
-        if (dt_y == AGAVE_BF16) rc = dispatch_tiled<0, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-        else if (dt_y == AGAVE_F32) rc = dispatch_tiled<0, float>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        if (dt_y == AGAVE_BF16) rc = dispatch_tiled<0, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, part, part_elems, stream);
+        else if (dt_y == AGAVE_F32) rc = dispatch_tiled<0, float>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, part, part_elems, stream);
         else AGAVE_CHECK(false, "gemm_tiled: unknown output dtype %d", dt_y);
     } else {
         AGAVE_CHECK(dt_y == AGAVE_BF16, "gemm_tiled: the GeGLU epilogue writes bfloat16");
-        rc = dispatch_tiled<1, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        rc = dispatch_tiled<1, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, nullptr, 0, stream);
     }
     if (rc != 0) return rc;
     AGAVE_LAUNCH_CHECK("gemm_tiled");

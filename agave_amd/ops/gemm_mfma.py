@@ -12,7 +12,7 @@ kernels.register_signatures("gemm_mfma", {
     "agave_pack_w16": [_P, _L, _P, _I, _I, _I, _I, _P],
     "agave_embed_scale_packed": [_P, _P, _F, _P, _I, _I, _I, _P],
     "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P],
-    "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P],
+    "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P, _L, _P],
 })
 
 SKINNY_MAX_M = 64
@@ -52,6 +52,24 @@ def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int,
     _launch("agave_gemm_skinny", x, packed, out, n_out, epilogue)
 
 
+# The tiled kernel shares a product out along its columns only when it has fewer than 160 tiles of
+# 64 x 128, and among at most 8 workgroups a tile: the partial sums never need more than this.
+PARTS_ELEMS = 8 * 160 * 64 * 128
+_parts = {}
+
+
+def _partial_sums(x: torch.Tensor, epilogue: int):
+    """The buffer of 32-bit partial sums that the tiled kernel may use for a product with few tiles
+    and many columns.  One per device, of a fixed size, so that its address can be recorded in a
+    graph."""
+    if epilogue:
+        return None
+    buf = _parts.get(x.device)
+    if buf is None:
+        buf = _parts[x.device] = torch.empty(PARTS_ELEMS, dtype=torch.float32, device=x.device)
+    return buf
+
+
 def _launch(fn: str, x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, epilogue: int) -> None:
     if not (x.is_cuda and packed.is_cuda and out.is_cuda):
         raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
@@ -63,6 +81,12 @@ def _launch(fn: str, x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n
     nb = (n_out + 7) // 8 if epilogue else (n_out + 15) // 16
     if packed.numel() != nb * ((k + 31) // 32) * 512:
         raise ValueError("packed product: the packed weight does not fit these sizes")
+    if fn == "agave_gemm_tiled":
+        part = _partial_sums(x, epilogue)
+        library.call(kernels.lib("gemm_mfma"), fn, x.data_ptr(), x.stride(0), packed.data_ptr(),
+                     kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue,
+                     kernels.ptr(part), part.numel() if part is not None else 0, kernels.stream())
+        return
     library.call(kernels.lib("gemm_mfma"), fn, x.data_ptr(), x.stride(0), packed.data_ptr(),
                  kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue, kernels.stream())
 

@@ -487,8 +487,10 @@ def test_attn_mfma_far_key_and_window_edge(K, decode):
     assert torch.allclose(got_e[-1, 0], vs[0][3, 0].double(), atol=2e-2)
 
 
-# the last three shapes take the 128 x 128, 128 x 256 and 256 x 256 tiles, the others the 64 x 128 one
-@pytest.mark.parametrize("m,n,k", [(65, 53, 72), (300, 256, 2560), (257, 1000, 96), (2048, 300, 136), (130, 4100, 64),
+# the last three shapes take the 128 x 128, 128 x 256 and 256 x 256 tiles, the others the 64 x 128 one; the
+# shapes with few tiles and many columns are shared out along the columns (2, 5, 3 and 7 partial sums)
+@pytest.mark.parametrize("m,n,k", [(65, 53, 72), (300, 256, 2560), (100, 250, 2560), (70, 200, 1560), (65, 2560, 10240),
+                                   (257, 1000, 96), (2048, 300, 136), (130, 4100, 64),
                                    (1000, 4096, 96), (2048, 4090, 64), (1024, 10240, 72)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_tiled(G, m, n, k, out_dtype):
