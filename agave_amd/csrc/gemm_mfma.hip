@@ -97,9 +97,13 @@ extern "C" int agave_embed_scale_packed(const int* tokens, const void* P, float 
 }
 
 // ------------------------------------------------------------------ skinny product (decode)
+// gelu with the tanh approximation: 0.5 (1 + tanh u) = 1 / (1 + exp(-2u)), u = sqrt(2/pi) (x + 0.044715 x^3);
+// the hardware's exp2 and reciprocal (about an ulp each) stand for tanhf, whose many instructions
+// a product's last step has no time for
 __device__ __forceinline__ float gelu_tanh_f(float x) {
-    const float c = 0.7978845608028654f;
-    return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
+    const float c2 = -2.0f * 0.7978845608028654f * 1.4426950408889634f;        // -2 sqrt(2/pi) log2(e)
+    const float e = __builtin_amdgcn_exp2f(c2 * (x + 0.044715f * x * x * x));
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // R: row blocks (of 16 weight rows) per workgroup; MT: tiles of 16 tokens; EPI 0: store, 1: GeGLU;
@@ -373,8 +377,17 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
 // the number of row tiles apart) tend to land on the same XCD and find them in its L2.
 typedef __attribute__((address_space(3))) u32x4_t tl_lds_u32x4;
 
-template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT>
-__global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
+// a loop whose index is a compile-time constant in the body (f gets IntC<I>): for instructions' immediate fields
+template <int I> struct IntC { static constexpr int value = I; };
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(IntC<I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, int MODE>
+__global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
                                                          const uint4* __restrict__ Wp, TC* __restrict__ Y, long ldy,
                                                          int M, int N, int K, int KB, int NB, long part_stride) {
     constexpr int CPR = KT * 4;                       // 16-byte pieces per staged token row
@@ -388,10 +401,9 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
     static_assert(NWV == 4 || NWV == 8, "four or eight waves");
     static_assert(X_LOADS * NWV * 1024 == X_BYTES && W_LOADS * NWV * 1024 == W_BYTES, "whole loads per wave");
     constexpr int LOADS = X_LOADS + W_LOADS;
-    static_assert(LOADS * (NS - 2) < 64, "the load counter holds 6 bits");
-    static_assert(NS >= 2 && NS <= 5, "the waits below name up to three stages in flight behind the awaited one");
+    static_assert(NS >= 2, "a stage is loaded while another is multiplied");
     extern __shared__ __attribute__((aligned(16))) unsigned char tl_lds[];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int wn = wave & 1, wm = wave >> 1;
     const int nbw = blockIdx.x * WTILES;                  // first packed weight tile of this workgroup
     const int m0 = blockIdx.y * TT;                       // first token of this workgroup
@@ -411,74 +423,193 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
 
-    // this lane's part of the staging
-    const bf16* xsrc[X_LOADS];
-    int xcol[X_LOADS];
+    // Staging.  Everything that is the same for a whole wave is kept in scalar registers (the wave's
+    // number is made scalar above), so that a load costs the vector unit nothing but its issue: the
+    // address is a scalar base, moved from stage to stage, plus a per-lane offset fixed at the start.
+    const unsigned char* xbase = (const unsigned char*)(X + (size_t)m0 * ldx);
+    unsigned xoff[X_LOADS], xoff_last[X_LOADS];
+    const int st_last = n_stage_all - 1;                               // the stage that may hold columns past K
 #pragma unroll
     for (int i = 0; i < X_LOADS; ++i) {
         const int o = ((wave * X_LOADS + i) * 64 + lane);              // 16-byte slot in the stage
         const int row = o / CPR, pos = o % CPR;                        // LDS row and position this lane's piece lands in
         const int piece = pos ^ ((row / RP) % CPR);                    // which 8 columns of that row it holds
-        int mrow = m0 + row;
-        if (mrow >= M) mrow = M - 1;                                   // rows past the end repeat the last one (never stored)
-        xcol[i] = piece * 8;
-        xsrc[i] = X + (size_t)mrow * ldx + piece * 8;
+        int mrow = row;
+        if (m0 + mrow >= M) mrow = M - 1 - m0;                         // rows past the end repeat the last one (never stored)
+        xoff[i] = (unsigned)(((size_t)mrow * ldx + piece * 8) * 2);
+        // in the last stage a piece past the last column reads the stage's first columns instead
+        // (any valid address: the weights are zero there)
+        xoff_last[i] = st_last * (KT * 32) + piece * 8 >= K ? (unsigned)(((size_t)mrow * ldx) * 2) : xoff[i];
     }
-    auto fetch = [&](int st) {
+    const unsigned woff = lane * 16;
+    // load i (of LOADS) of stage st; stages past the last load the last one again and are never multiplied
+    auto fetch_one = [&](int st, int i) {
         unsigned char* buf = tl_lds + (size_t)(st % NS) * STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < X_LOADS; ++i) {
-            int k = st * (KT * 32);
-            if (k + xcol[i] >= K) k = -xcol[i];                        // past the last column: any valid address (weights are zero there)
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xsrc[i] + k),
+        const int ste = st < st_last ? st : st_last;
+        if (i < X_LOADS) {
+            const unsigned char* src = xbase + (size_t)ste * (KT * 64);
+            const unsigned off = ste == st_last ? xoff_last[i] : xoff[i];
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + off),
                                              (__attribute__((address_space(3))) void*)(buf + (wave * X_LOADS + i) * 1024), 16, 0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < W_LOADS; ++i) {
-            const int tt = wave * W_LOADS + i;                         // tile: row tile tt / KT, k-step tt % KT
-            int nb = nbw + tt / KT, kb = st * KT + tt % KT;
+        } else {
+            const int tt = wave * W_LOADS + (i - X_LOADS);             // tile: row tile tt / KT, k-step tt % KT
+            int nb = nbw + tt / KT, kb = ste * KT + tt % KT;
             if (nb >= NB) nb = NB - 1;                                 // rows past the end: never stored
             if (kb >= KB) kb = KB - 1;                                 // k-steps past the end: never multiplied
-            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(Wp + ((size_t)nb * KB + kb) * 64 + lane),
+            const unsigned char* src = (const unsigned char*)(Wp + ((size_t)nb * KB + kb) * 64);
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + woff),
                                              (__attribute__((address_space(3))) void*)(buf + X_BYTES + tt * 1024), 16, 0, 0);
         }
     };
+    // this lane's operands of one k-step of 16 columns (phase ph of a stage: k-step ph / 2 of 32 columns, its half ph % 2).
+    // A 32-row weight operand is made of two packed 16-row tiles: rows 0..15 from the first,
+    // 16..31 from the second; the lane holding (row, columns 8*(2h+kg)..) there.
+    constexpr int PH = 2 * KT;                                         // phases per stage
+    struct Operands { frag16 w[WT]; frag16 x[XB]; };
+    // The token rows' 16-byte pieces are permuted by (row / RP) % CPR, which is the same for all of a
+    // lane's rows (they are 32 apart), so one address per phase serves them all.
+    const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)tl_lds;
+    const unsigned w_lane = lds0 + X_BYTES + (wn * (2 * WT) + (i32 >> 4)) * KT * 1024 + ((i32 & 15) + 16 * kg) * 16;
+    unsigned x_lane[PH];
+#pragma unroll
+    for (int ph = 0; ph < PH; ++ph)
+        x_lane[ph] = lds0 + (wm * XB * 32 + i32) * (CPR * 16) + (((ph * 2) ^ kg ^ ((i32 / RP) % CPR)) * 16);
+    // The reads are written as instructions, with the waits for them placed by hand: the compiler
+    // counts a load that goes straight into LDS as an LDS access of unknown order and would wait for
+    // every pending LDS read before each multiplication, the ones just asked for included.
+    auto read_operands = [&](Operands& f, int st, auto phc) {
+        constexpr int ph = decltype(phc)::value;
+        const unsigned buf = (unsigned)(st % NS) * STAGE_BYTES;
+        const unsigned wa = w_lane + buf, xa = x_lane[ph] + buf;
+        static_for<0, WT>([&](auto a) {
+            frag16& dst = f.w[a.value];                                // (operands of asm do not capture by themselves)
+            const unsigned addr = wa;
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst.r)
+                         : "v"(addr), "n"(2 * a.value * KT * 1024 + (ph >> 1) * 1024 + (ph & 1) * 512));
+        });
+        static_for<0, XB>([&](auto b) {
+            frag16& dst = f.x[b.value];
+            const unsigned addr = xa;
+            asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst.r) : "v"(addr), "n"(b.value * 32 * CPR * 16));
+        });
+    };
+    // every read asked for has returned; what uses f comes after this
+    auto settle = [&](Operands& f) {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int a = 0; a < WT; ++a) asm volatile("" : "+v"(f.w[a].r));
+#pragma unroll
+        for (int b = 0; b < XB; ++b) asm volatile("" : "+v"(f.x[b].r));
+    };
 
+    // The stage loop.  Loads run NS-1 stages ahead.  MODE says how a wave's work is laid out in time:
+    //   0, 1: loads are issued one at a time between the multiplications (all at once they queue up
+    //      at the address unit, which takes 16 cycles for each, while the matrix cores wait), and the
+    //      operands of a phase are read from LDS while the phase before it multiplies.  1: the first
+    //      operands of the next stage are read during the last phase of this one, for which every
+    //      stage must have landed one barrier earlier.
+    //   2: the two waves of a SIMD take turns (waves 0-3 and 4-7, half a stage apart): one reads its
+    //      operands of a whole stage and issues its loads while the other multiplies, then a barrier,
+    //      and they change places.  The matrix cores then always have a wave that does nothing else.
+    constexpr bool AHEAD = MODE == 1;
+    constexpr int IN_FLIGHT = LOADS * (NS - 2 - (MODE != 0 ? 1 : 0)); // loads that may be outstanding at a barrier
+    static_assert(IN_FLIGHT >= 0 && IN_FLIGHT < 64, "the load counter holds 6 bits");
 #pragma unroll
     for (int s0 = 0; s0 < NS - 1; ++s0)
-        if (st0 + s0 < n_stage) fetch(st0 + s0);
-    for (int st = st0; st < n_stage; ++st) {
-        // stage st has landed once at most the loads of the NS-2 stages after it are outstanding
-        const int ahead = (n_stage - 1 - st < NS - 2) ? n_stage - 1 - st : NS - 2;
-        if (ahead >= 3) __builtin_amdgcn_s_waitcnt(0x0F70 | ((3 * LOADS) & 15) | (((3 * LOADS) >> 4) << 14));
-        else if (ahead == 2) __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * LOADS) & 15) | (((2 * LOADS) >> 4) << 14));
-        else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0F70 | (LOADS & 15) | ((LOADS >> 4) << 14));
-        else __builtin_amdgcn_s_waitcnt(0x0F70);
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) fetch_one(st0 + s0, i);
+    auto landed = [&]() {
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (IN_FLIGHT & 15) | ((IN_FLIGHT >> 4) << 14));
         // a bare barrier: __syncthreads() would also wait for the loads still wanted in flight
         __builtin_amdgcn_s_barrier();
-        if (st + NS - 1 < n_stage) fetch(st + NS - 1);
-        const unsigned char* buf = tl_lds + (size_t)(st % NS) * STAGE_BYTES;
+    };
+    if (MODE == 2) {
+        static_assert(MODE != 2 || (NWV == 8 && NS >= 4), "two waves per SIMD take turns; a stage is in flight behind the awaited one");
+        // Slots between barriers: the first group reads stage i in slot 2i and multiplies in slot
+        // 2i+1, the second group one slot later; the loads for stage i+NS-1 are issued while stage
+        // i is multiplied.  The first group reads stage i+1 in slot 2i+2, so every wave's loads
+        // for it must have landed by the end of slot 2i+1, which is where the second group's waves
+        // wait, after reading stage i: the loads of the NS-3 stages after i+1, all that are issued
+        // by then, may be in flight.  (The first group waits at the same place in its own order,
+        // a slot earlier than it would have to.)  A buffer is loaded into again at least a slot
+        // after the second group read it.
+        const bool second = wave >= 4;
+        Operands f[PH];
+        landed();
+        if (second) __builtin_amdgcn_s_barrier();
+        for (int st = st0; st < n_stage; ++st) {
+            static_for<0, PH>([&](auto ph) { read_operands(f[ph.value], st, ph); });
 #pragma unroll
-        for (int k16 = 0; k16 < KT * 2; ++k16) {
-            const int ks = k16 >> 1, h = k16 & 1;                      // k-step of 32 columns and its half
-            if (st * KT + ks >= KB) break;
-            // a 32-row weight operand is made of two packed 16-row tiles: rows 0..15 from the
-            // first, 16..31 from the second; the lane holding (row, columns 8*(2h+kg)..) there
-            frag16 wf[WT];
+            for (int ph = 0; ph < PH; ++ph) settle(f[ph]);
+            landed();
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(1);
+            // the loads go between the multiplications: issued in their shadow, they cost no time
+            int li = 0;
 #pragma unroll
-            for (int a = 0; a < WT; ++a) {
-                const int nt = wn * (2 * WT) + 2 * a + (i32 >> 4);
-                wf[a].r = *(const tl_lds_u32x4*)(buf + X_BYTES + (nt * KT + ks) * 1024 + ((i32 & 15) + 16 * (2 * h + kg)) * 16);
+            for (int ph = 0; ph < PH; ++ph) {
+                const bool live = KT == 1 || st * KT + (ph >> 1) < KB;
+#pragma unroll
+                for (int b = 0; b < XB; ++b) {
+                    if (live) {
+#pragma unroll
+                        for (int a = 0; a < WT; ++a) acc[a][b] = mfma_32x32x16(f[ph].w[a], f[ph].x[b], acc[a][b]);
+                    }
+                    if (li < LOADS) {
+                        __builtin_amdgcn_sched_barrier(0);
+                        fetch_one(st + NS - 1, li++);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
             }
+#pragma unroll
+            for (; li < LOADS; ++li) fetch_one(st + NS - 1, li);
+            __builtin_amdgcn_s_setprio(0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (!(second && st + 1 == n_stage)) __builtin_amdgcn_s_barrier();
+        }
+    } else {
+    Operands f[2];
+    if (AHEAD) {
+        landed();
+        read_operands(f[0], st0, IntC<0>{});
+        settle(f[0]);
+    }
+    for (int st = st0; st < n_stage; ++st) {
+        if (!AHEAD) {
+            landed();
+            read_operands(f[0], st, IntC<0>{});
+            settle(f[0]);
+        }
+        static_for<0, PH>([&](auto phc) {
+            constexpr int ph = decltype(phc)::value;
+            const bool more = ph + 1 < PH || AHEAD;
+            if constexpr (ph + 1 < PH) read_operands(f[(ph + 1) & 1], st, IntC<ph + 1>{});
+            else if (AHEAD) read_operands(f[0], st + 1, IntC<0>{});     // after the last stage: stale, unused
+            __builtin_amdgcn_sched_barrier(0);
+            const Operands& o = f[ph & 1];
+            const bool live = KT == 1 || st * KT + (ph >> 1) < KB;
+            const int L0 = (ph * LOADS + PH - 1) / PH, L1 = ((ph + 1) * LOADS + PH - 1) / PH;        // this phase's loads
+            int li = L0;
 #pragma unroll
             for (int b = 0; b < XB; ++b) {
-                const int row = (wm * XB + b) * 32 + i32;
-                frag16 xb;
-                xb.r = *(const tl_lds_u32x4*)(buf + row * (CPR * 16) + (((k16 * 2 + kg) ^ ((row / RP) % CPR)) * 16));
+                if (live) {
 #pragma unroll
-                for (int a = 0; a < WT; ++a) acc[a][b] = mfma_32x32x16(wf[a], xb, acc[a][b]);
+                    for (int a = 0; a < WT; ++a) acc[a][b] = mfma_32x32x16(o.w[a], o.x[b], acc[a][b]);
+                }
+                if (li < L1) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    fetch_one(st + NS - 1, li++);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
-        }
+#pragma unroll
+            for (; li < L1; ++li) fetch_one(st + NS - 1, li);
+            __builtin_amdgcn_sched_barrier(0);
+            if (more) settle(f[(ph + 1) & 1]);
+        });
+        if (AHEAD) landed();
+    }
     }
 
     // D[i][j]: this lane holds token j = lane % 32 and rows i = 8*q + 4*kg + e (q, e = 0..3)
@@ -522,7 +653,7 @@ __global__ __launch_bounds__(NWV * 64) void gemm_tiled_kernel(const bf16* __rest
     }
 }
 
-template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT>
+template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, int MODE>
 static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB, int NB,
                         hipStream_t stream, int splits = 1, long part_stride = 0) {
     constexpr int WTILES = 4 * WT;
@@ -531,12 +662,12 @@ static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long l
     AGAVE_CHECK(grid.y <= 65535, "gemm_tiled: M=%d exceeds the grid limit", M);
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT, MODE>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         AGAVE_CHECK(e == hipSuccess, "gemm_tiled: cannot raise the LDS allowance");
         raised = true;
     }
-    gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
+    gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT, MODE><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
                                                                       M, N, K, KB, NB, part_stride);
     return 0;
 }
@@ -584,8 +715,8 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
     if (splits > 1) {
         const long stride = (long)M * N;
         int rc;
-        if (pick == 2) rc = launch_tiled<2, 2, 3, 0, float, 8, 128>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
-        else rc = launch_tiled<1, 2, 4, 0, float, 8, 128>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
+        if (pick == 2) rc = launch_tiled<2, 2, 3, 0, float, 8, 128, 0>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
+        else rc = launch_tiled<1, 2, 4, 0, float, 8, 128, 0>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
         if (rc != 0) return rc;
         AGAVE_LAUNCH_CHECK("gemm_tiled (partial sums)");
         const long total = (long)M * N;
@@ -593,10 +724,10 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
         return 0;
     }
     switch (pick) {
-        case 0: return launch_tiled<4, 1, 4, EPI, TC, 8, 256>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-        case 1: return launch_tiled<2, 2, 3, EPI, TC, 8, 256>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-        case 2: return launch_tiled<2, 2, 3, EPI, TC, 8, 128>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-        default: return launch_tiled<1, 2, 4, EPI, TC, 8, 128>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 0: return launch_tiled<4, 1, 4, EPI, TC, 8, 256, 2>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 1: return launch_tiled<2, 2, 3, EPI, TC, 8, 256, 0>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 2: return launch_tiled<2, 2, 3, EPI, TC, 8, 128, 0>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        default: return launch_tiled<1, 2, 4, EPI, TC, 8, 128, 0>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     }
 }
 
@@ -609,6 +740,7 @@ extern "C" int agave_gemm_tiled(const void* X, long ldx, const void* Wp, int dt_
     AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
                 "gemm_tiled: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
     AGAVE_CHECK(ldx >= K && ldy >= N, "gemm_tiled: a row stride is too small");
+    AGAVE_CHECK(ldx < (1L << 22), "gemm_tiled: a row stride of %ld elements is beyond the kernel's 32-bit offsets", ldx);
     AGAVE_CHECK(epilogue == 0 || epilogue == 1, "gemm_tiled: unknown epilogue %d", epilogue);
     if (M == 0) return 0;
     const int KB = (K + 31) / 32;

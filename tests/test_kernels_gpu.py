@@ -491,7 +491,9 @@ def test_attn_mfma_far_key_and_window_edge(K, decode):
 # shapes with few tiles and many columns are shared out along the columns (2, 5, 3 and 7 partial sums)
 @pytest.mark.parametrize("m,n,k", [(65, 53, 72), (300, 256, 2560), (100, 250, 2560), (70, 200, 1560), (65, 2560, 10240),
                                    (257, 1000, 96), (2048, 300, 136), (130, 4100, 64),
-                                   (1000, 4096, 96), (2048, 4090, 64), (1024, 10240, 72)])
+                                   (1000, 4096, 96), (2048, 4090, 64), (1024, 10240, 72),
+                                   # many stages (the loads run several stages ahead of the multiplications): each tile
+                                   (300, 2000, 1000), (600, 5000, 1000), (1024, 5120, 1000), (1024, 10240, 1000)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_tiled(G, m, n, k, out_dtype):
     g = torch.Generator().manual_seed(m + n + k)
@@ -506,7 +508,7 @@ def test_gemm_tiled(G, m, n, k, out_dtype):
     assert float((out.cpu().double() - ref).abs().max()) <= tol
 
 
-@pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40)])
+@pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40), (1024, 5120, 1000)])
 def test_gemm_tiled_geglu(G, m, ff, k):
     g = torch.Generator().manual_seed(ff + m)
     x = torch.randn(m, k, generator=g).bfloat16()
