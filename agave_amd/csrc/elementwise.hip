@@ -42,8 +42,8 @@ extern "C" int agave_embed_scale(int dtype, const int* tokens, const void* table
 //   if out:    out[i] = rmsnorm(h[r]) * pre_gain
 // Gains are 32-bit and already hold the "+1" where the architecture has it.
 template <typename T>
-__global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb,
-                                     const float* __restrict__ post_gain, float post_eps,
+__global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
+                                     long part_stride, const float* __restrict__ post_gain, float post_eps,
                                      T* __restrict__ out, long ldo, const float* __restrict__ pre_gain,
                                      float pre_eps, const int* __restrict__ rows, int e) {
     __shared__ float red[16];
@@ -53,18 +53,26 @@ __global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict_
     float ss_h = 0.f;
     if (branch) {
         const T* br = branch + (size_t)r * ldb;
+        // n_parts > 0: the branch is the sum of that many 32-bit slices, part_stride elements apart
+        const float* parts = reinterpret_cast<const float*>(branch) + (size_t)r * ldb;
+        auto at = [&](int c) {
+            if (n_parts == 0) return ld(br + c);
+            float v = 0.f;
+            for (int p = 0; p < n_parts; ++p) v += parts[(size_t)p * part_stride + c];
+            return v;
+        };
         float inv = 1.0f;
         if (post_gain) {
             float ss = 0.f;
             for (int c = threadIdx.x; c < e; c += blockDim.x) {
-                const float v = ld(br + c);
+                const float v = at(c);
                 ss += v * v;
             }
             ss = block_sum(ss, red);
             inv = 1.0f / sqrtf(ss / (float)e + post_eps);
         }
         for (int c = threadIdx.x; c < e; c += blockDim.x) {
-            const float y = post_gain ? ld(br + c) * inv * post_gain[c] : ld(br + c);
+            const float y = post_gain ? at(c) * inv * post_gain[c] : at(c);
             const float hv = hr[c] + y;
             hr[c] = hv;
             ss_h += hv * hv;
@@ -106,8 +114,8 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
 }
 
 template <typename T, int VPT>
-__global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb,
-                                          const float* __restrict__ post_gain, float post_eps,
+__global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
+                                          long part_stride, const float* __restrict__ post_gain, float post_eps,
                                           T* __restrict__ out, long ldo, const float* __restrict__ pre_gain,
                                           float pre_eps, const int* __restrict__ rows, int e) {
     __shared__ float red[16];
@@ -121,7 +129,20 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
         const bool in = c < e;
         const float4 z = float4{0.f, 0.f, 0.f, 0.f};
         hv[v] = in ? *reinterpret_cast<const float4*>(hr + c) : z;
-        bv[v] = (in && branch) ? load4(branch + (size_t)r * ldb + c) : z;
+        if (n_parts == 0) {
+            bv[v] = (in && branch) ? load4(branch + (size_t)r * ldb + c) : z;
+        } else {
+            // the branch is the sum of 32-bit slices (a product that was shared out along its columns)
+            const float* parts = reinterpret_cast<const float*>(branch) + (size_t)r * ldb + c;
+            bv[v] = z;
+            for (int p = 0; p < n_parts && in; ++p) {
+                const float4 t = *reinterpret_cast<const float4*>(parts + (size_t)p * part_stride);
+                bv[v].x += t.x;
+                bv[v].y += t.y;
+                bv[v].z += t.z;
+                bv[v].w += t.w;
+            }
+        }
         g1[v] = (in && branch && post_gain) ? *reinterpret_cast<const float4*>(post_gain + c) : z;
         g2[v] = (in && out) ? *reinterpret_cast<const float4*>(pre_gain + c) : z;
     }
@@ -169,11 +190,13 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
 }
 
 template <typename T>
-static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, const float* post_gain, float post_eps,
+static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, int n_parts, long part_stride,
+                                      const float* post_gain, float post_eps,
                                       void* out, long ldo, const float* pre_gain, float pre_eps, const int* rows,
                                       int n_rows, int e, hipStream_t stream) {
     const size_t align = sizeof(T) * 4;
-    if (e % 4 != 0 || e > 16384 || (branch && (ldb % 4 != 0 || (uintptr_t)branch % align != 0)) ||
+    if (e % 4 != 0 || e > 16384 || (branch && (ldb % 4 != 0 || (uintptr_t)branch % (n_parts ? 16 : align) != 0)) ||
+        (n_parts && part_stride % 4 != 0) ||
         (out && (ldo % 4 != 0 || (uintptr_t)out % align != 0)) || (uintptr_t)h % 16 != 0 ||
         (post_gain && (uintptr_t)post_gain % 16 != 0) || (pre_gain && (uintptr_t)pre_gain % 16 != 0))
         return false;
@@ -183,7 +206,8 @@ static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, co
                                                                     : (e <= 4096 ? 256 : 1024);
     const int vpt = (e / 4 + threads - 1) / threads;
 #define RN_FAST(V)                                                                                                    \
-    residual_norm_fast_kernel<T, V><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, post_gain, post_eps,   \
+    residual_norm_fast_kernel<T, V><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts, part_stride,  \
+                                                                    post_gain, post_eps,                             \
                                                                     (T*)out, ldo, pre_gain, pre_eps, rows, e)
     if (vpt <= 1) RN_FAST(1);
     else if (vpt <= 2) RN_FAST(2);
@@ -192,26 +216,32 @@ static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, co
     return true;
 }
 
-extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long ldb, const float* post_gain,
-                                   float post_eps, void* out, long ldo, const float* pre_gain, float pre_eps,
-                                   const int* rows, int n_rows, int e, hipStream_t stream) {
+// n_parts > 0: branch points at that many 32-bit slices [n_rows][ldb], part_stride elements apart,
+// whose sum is the branch (whatever dtype says, which then names out's type alone).
+extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long ldb, int n_parts, long part_stride,
+                                   const float* post_gain, float post_eps, void* out, long ldo, const float* pre_gain,
+                                   float pre_eps, const int* rows, int n_rows, int e, hipStream_t stream) {
     AGAVE_CHECK(n_rows >= 0 && e > 0, "residual_norm: bad sizes rows=%d e=%d", n_rows, e);
     AGAVE_CHECK(h != nullptr, "residual_norm: residual stream is null");
     AGAVE_CHECK(!out || pre_gain, "residual_norm: output without its gain");
     AGAVE_CHECK(!branch || ldb >= e, "residual_norm: branch row stride %ld < %d", ldb, e);
     AGAVE_CHECK(!out || ldo >= e, "residual_norm: output row stride %ld < %d", ldo, e);
     AGAVE_CHECK(!(rows && branch), "residual_norm: row gather with a branch is not supported");
+    AGAVE_CHECK(n_parts >= 0 && n_parts <= 64 && (n_parts == 0 || branch), "residual_norm: %d slices", n_parts);
     if (n_rows == 0 || (!branch && !out)) return 0;
     const int threads = e >= 2048 ? 512 : (e >= 512 ? 256 : 64);
-    if (dtype == AGAVE_F32 && launch_residual_norm_fast<float>(h, branch, ldb, post_gain, post_eps, out, ldo, pre_gain,
-                                                              pre_eps, rows, n_rows, e, stream)) {
-    } else if (dtype == AGAVE_BF16 && launch_residual_norm_fast<bf16>(h, branch, ldb, post_gain, post_eps, out, ldo,
-                                                                     pre_gain, pre_eps, rows, n_rows, e, stream)) {
+    if (dtype == AGAVE_F32 && launch_residual_norm_fast<float>(h, branch, ldb, n_parts, part_stride, post_gain, post_eps,
+                                                              out, ldo, pre_gain, pre_eps, rows, n_rows, e, stream)) {
+    } else if (dtype == AGAVE_BF16 && launch_residual_norm_fast<bf16>(h, branch, ldb, n_parts, part_stride, post_gain,
+                                                                     post_eps, out, ldo, pre_gain, pre_eps, rows, n_rows,
+                                                                     e, stream)) {
     } else if (dtype == AGAVE_F32)
-        residual_norm_kernel<float><<<n_rows, threads, 0, stream>>>(h, (const float*)branch, ldb, post_gain, post_eps,
+        residual_norm_kernel<float><<<n_rows, threads, 0, stream>>>(h, (const float*)branch, ldb, n_parts, part_stride,
+                                                                    post_gain, post_eps,
                                                                     (float*)out, ldo, pre_gain, pre_eps, rows, e);
     else if (dtype == AGAVE_BF16)
-        residual_norm_kernel<bf16><<<n_rows, threads, 0, stream>>>(h, (const bf16*)branch, ldb, post_gain, post_eps,
+        residual_norm_kernel<bf16><<<n_rows, threads, 0, stream>>>(h, (const bf16*)branch, ldb, n_parts, part_stride,
+                                                                   post_gain, post_eps,
                                                                    (bf16*)out, ldo, pre_gain, pre_eps, rows, e);
     else
         AGAVE_CHECK(false, "residual_norm: unknown dtype %d", dtype);

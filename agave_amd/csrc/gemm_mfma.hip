@@ -117,7 +117,7 @@ __device__ __forceinline__ float gelu_tanh_f(float x) {
 template <int R, int MT, int EPI, int NW, typename TC, int XR>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __restrict__ X, long ldx,
                                                           const uint4* __restrict__ Wp, TC* __restrict__ Y,
-                                                          long ldy, int M, int N, int K, int KB, int NB) {
+                                                          long ldy, int M, int N, int K, int KB, int NB, long part_stride) {
     constexpr int KS = MT <= 2 ? 4 : 2;
     constexpr int ROW = KS * 32 + 8;                                // bf16 per staged X row, 16 bytes of padding
     constexpr int PIECES = KS * 4;                                  // 16-byte pieces per staged row
@@ -138,8 +138,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     const int j = lane & 15, g = lane >> 4;
     const int xr = lane / PIECES, xp = lane % PIECES;               // staging: row within an instruction, piece
     const int nb0 = blockIdx.x * R;
-    const int n_chunks = (KB + KS - 1) / KS;
+    // gridDim.y workgroups share a row block's columns: each takes a run of chunks and leaves its
+    // sums in its own slice of Y (partial sums then, which the reader adds up)
+    const int n_chunks_all = (KB + KS - 1) / KS;
+    const int c_lo = (int)((long)blockIdx.y * n_chunks_all / gridDim.y);
+    const int n_chunks = (int)((long)(blockIdx.y + 1) * n_chunks_all / gridDim.y) - c_lo;
     const int n_iter = (n_chunks + NW - 1) / NW;
+    Y += (size_t)blockIdx.y * part_stride;
 
     f32x4_t acc[R][MT];
 #pragma unroll
@@ -179,7 +184,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     {                                                                                            \
         int c_ = (IT) * NW + wave;                    /* chunks are dealt to the waves in turn */ \
         c_ = (c_ < n_chunks ? c_ : n_chunks - 1) + rot;                                          \
-        c_ = c_ < n_chunks ? c_ : c_ - n_chunks;                                                 \
+        c_ = (c_ < n_chunks ? c_ : c_ - n_chunks) + c_lo;                                        \
         _Pragma("unroll") for (int r = 0; r < R; ++r)                                            \
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                  \
                 const int kb = c_ * KS + ks;           /* past the last tile: any tile, X is zero there */ \
@@ -194,7 +199,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 #define SK_USE(ST, IT)                                                                           \
     if ((IT) * NW + wave < n_chunks) {                                                           \
         const int pc_ = (IT) * NW + wave + rot;                                                  \
-        const bool in_ = (pc_ < n_chunks ? pc_ : pc_ - n_chunks) * (KS * 32) + xp * 8 < K;       \
+        const bool in_ = ((pc_ < n_chunks ? pc_ : pc_ - n_chunks) + c_lo) * (KS * 32) + xp * 8 < K; \
         _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                        \
             _Pragma("unroll") for (int i = 0; i < NI; ++i)                                       \
                 *reinterpret_cast<uint4*>(my_xs + (mt * 16 + RPI * i + xr) * ROW + xp * 8) =     \
@@ -266,10 +271,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
 
 template <int R, int MT, int EPI, int NW, typename TC, int XR>
 static void launch_skinny_nw(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
-                             int NB, hipStream_t stream) {
-    const int grid = (NB + R - 1) / R;
+                             int NB, int splits, hipStream_t stream) {
+    const dim3 grid((NB + R - 1) / R, splits);
     gemm_skinny_kernel<R, MT, EPI, NW, TC, XR><<<grid, NW * 64, 0, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y,
-                                                                        ldy, M, N, K, KB, NB);
+                                                                        ldy, M, N, K, KB, NB, (long)M * ldy);
 }
 
 // Waves per workgroup: the fewest that put some 640 waves on the chip.  Every wave keeps two
@@ -283,24 +288,24 @@ static int skinny_waves(int groups, int n_chunks, int max_nw) {
 
 template <int R, int MT, int EPI, typename TC, int XR>
 static void launch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
-                          int NB, hipStream_t stream) {
+                          int NB, int splits, hipStream_t stream) {
     constexpr int KS = MT <= 2 ? 4 : 2;
     constexpr int MAX_NW = (R * MT <= 2) ? 16 : (R * MT <= 8 ? 8 : 4);
-    const int n_chunks = (KB + KS - 1) / KS;
-    const int groups = (NB + R - 1) / R;
+    const int n_chunks = ((KB + KS - 1) / KS) / splits;
+    const int groups = (NB + R - 1) / R * splits;
     const int nw = skinny_waves(groups, n_chunks, MAX_NW);
     if (nw == 16) {
-        if constexpr (MAX_NW >= 16) launch_skinny_nw<R, MT, EPI, 16, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        if constexpr (MAX_NW >= 16) launch_skinny_nw<R, MT, EPI, 16, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream);
     } else if (nw == 8) {
-        if constexpr (MAX_NW >= 8) launch_skinny_nw<R, MT, EPI, 8, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        if constexpr (MAX_NW >= 8) launch_skinny_nw<R, MT, EPI, 8, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream);
     } else {
-        launch_skinny_nw<R, MT, EPI, 4, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        launch_skinny_nw<R, MT, EPI, 4, TC, XR>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream);
     }
 }
 
 template <int EPI, typename TC>
 static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
-                           int NB, hipStream_t stream) {
+                           int NB, int splits, hipStream_t stream) {
     const int mt = (M + 15) / 16;
     // Row blocks per workgroup: every workgroup reads all of X, so the traffic from L2 is
     // (1 + 16*MT/(16*R)) times the weights'; more row blocks as long as enough workgroups remain.
@@ -309,12 +314,12 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
     else if (mt == 2) r = NB >= 4096 ? 4 : (NB >= 1024 ? 2 : 1);
     else r = NB >= 1024 ? 4 : 1;
 #define SK_CASE(R_, MT_)                                                                        \
-    launch_skinny<R_, MT_, EPI, TC, 16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);          \
+    launch_skinny<R_, MT_, EPI, TC, 16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream);          \
     break
 #define SK_CASE1(R_)                                                                            \
-    if (M <= 4) launch_skinny<R_, 1, EPI, TC, 4>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream); \
-    else if (M <= 8) launch_skinny<R_, 1, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream); \
-    else launch_skinny<R_, 1, EPI, TC, 16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);       \
+    if (M <= 4) launch_skinny<R_, 1, EPI, TC, 4>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream); \
+    else if (M <= 8) launch_skinny<R_, 1, EPI, TC, 8>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream); \
+    else launch_skinny<R_, 1, EPI, TC, 16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream);       \
     break
     switch (mt * 8 + r) {
         case 1 * 8 + 1: SK_CASE1(1);
@@ -334,8 +339,11 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
 }
 
 // N: logical outputs (rows of W, or ff for the GeGLU epilogue); Wp holds NB row blocks.
+// splits > 1: Y is 32-bit, [splits][M][ldy]; slice s gets the sums over the s-th run of columns,
+// and whoever reads Y adds the slices up (a product with few row blocks and many columns then
+// has workgroups enough to keep the memory busy).
 extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,
-                                 int K, int epilogue, hipStream_t stream) {
+                                 int K, int epilogue, int splits, hipStream_t stream) {
     AGAVE_CHECK(M >= 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: bad sizes M=%d N=%d K=%d (M <= 64)", M, N, K);
     AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
                 "gemm_skinny: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
@@ -344,14 +352,17 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
     if (M == 0) return 0;
     const int KB = (K + 31) / 32;
     const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
+    AGAVE_CHECK(splits >= 1 && splits <= 64 && (splits == 1 || splits * 16 <= KB), "gemm_skinny: %d slices for %d columns",
+                splits, K);
+    AGAVE_CHECK(splits == 1 || (epilogue == 0 && dt_y == AGAVE_F32), "gemm_skinny: partial sums are plain 32-bit sums");
     int rc;
     if (epilogue == 0) {
-        if (dt_y == AGAVE_BF16) rc = dispatch_skinny<0, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-        else if (dt_y == AGAVE_F32) rc = dispatch_skinny<0, float>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        if (dt_y == AGAVE_BF16) rc = dispatch_skinny<0, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, 1, stream);
+        else if (dt_y == AGAVE_F32) rc = dispatch_skinny<0, float>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream);
         else AGAVE_CHECK(false, "gemm_skinny: unknown output dtype %d", dt_y);
     } else {
         AGAVE_CHECK(dt_y == AGAVE_BF16, "gemm_skinny: the GeGLU epilogue writes bfloat16");
-        rc = dispatch_skinny<1, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        rc = dispatch_skinny<1, bf16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, 1, stream);
     }
     if (rc != 0) return rc;
     AGAVE_LAUNCH_CHECK("gemm_skinny");
@@ -722,6 +733,25 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
         const long total = (long)M * N;
         gemm_sum_parts_kernel<TC><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(part, splits, stride, (TC*)Y, ldy, M, N);
         return 0;
+    }
+    if (pick == 0) {
+        // 256 compute units take 256 tiles at a time.  When the last round would be at most half
+        // full, the rows of that round are computed in tiles of half the height instead, in a
+        // second launch: all compute units then work for half a round, not half of them for a whole one.
+        const long tiles = wgs[0], rest = tiles % 256;
+        long rows_main = 0;                                // 256-row tiles of the first launch
+        if (tiles > 256 && rest > 0 && rest <= 128) {
+            rows_main = (tiles - rest) / t256;             // whole rounds, if they are whole rows of tiles
+            if (rows_main * t256 != tiles - rest || (rows16 - rows_main) * 2 * t256 > 256) rows_main = 0;
+        }
+        if (rows_main > 0) {
+            const int nb_main = (int)rows_main * 16;
+            const int n_main = EPI == 0 ? nb_main * 16 : nb_main * 8;
+            int rc = launch_tiled<4, 1, 4, EPI, TC, 8, 256, 2>(X, ldx, Wp, Y, ldy, M, n_main, K, KB, nb_main, stream);
+            if (rc != 0) return rc;
+            return launch_tiled<2, 2, 3, EPI, TC, 8, 256, 0>(X, ldx, (const uint4*)Wp + (size_t)nb_main * KB * 64, (TC*)Y + n_main,
+                                                             ldy, M, N - n_main, K, KB, NB - nb_main, stream);
+        }
     }
     switch (pick) {
         case 0: return launch_tiled<4, 1, 4, EPI, TC, 8, 256, 2>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);

@@ -11,7 +11,7 @@ from .kernels import _F, _I, _L, _P
 kernels.register_signatures("gemm_mfma", {
     "agave_pack_w16": [_P, _L, _P, _I, _I, _I, _I, _P],
     "agave_embed_scale_packed": [_P, _P, _F, _P, _I, _I, _I, _P],
-    "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P],
+    "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _I, _P],
     "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P, _L, _P],
 })
 
@@ -52,6 +52,33 @@ def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int,
     _launch("agave_gemm_skinny", x, packed, out, n_out, epilogue)
 
 
+def slices_for(m: int, n_out: int, k: int) -> int:
+    """How many slices of partial sums a product of few tokens is worth: its row blocks are its
+    workgroups, and fewer than some 200 of them leave compute units without work while the
+    others cannot ask for memory any faster; with many columns, two or three workgroups share
+    each row block."""
+    blocks = (n_out + 15) // 16
+    if m < 4 or m > 16 or blocks > 192 or k < 4096:       # (a step of one or two tokens gains nothing)
+        return 1
+    return max(1, min(512 // blocks, k // 2048, 4))
+
+
+def skinny_slices(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int) -> None:
+    """out[s] = the sums over the s-th run of columns of x[M, K] @ W^T; out is float32 [slices, M, n_out]
+    and its slices add up to the product (M <= 64)."""
+    if not (x.is_cuda and packed.is_cuda and out.is_cuda):
+        raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
+    if not _x_ok(x):
+        raise ValueError("packed product: input must be 16-byte aligned bfloat16 rows with K and the row stride multiples of 8")
+    m, k = x.shape
+    if out.dtype != torch.float32 or out.dim() != 3 or out.shape[1:] != (m, n_out) or not out.is_contiguous():
+        raise ValueError(f"partial sums must be a contiguous float32 [slices, {m}, {n_out}] tensor")
+    if packed.numel() != ((n_out + 15) // 16) * ((k + 31) // 32) * 512:
+        raise ValueError("packed product: the packed weight does not fit these sizes")
+    library.call(kernels.lib("gemm_mfma"), "agave_gemm_skinny", x.data_ptr(), x.stride(0), packed.data_ptr(),
+                 kernels.dt(out), out.data_ptr(), n_out, m, n_out, k, 0, out.shape[0], kernels.stream())
+
+
 # The tiled kernel shares a product out along its columns only when it has fewer than 160 tiles of
 # 64 x 128, and among at most 8 workgroups a tile: the partial sums never need more than this.
 PARTS_ELEMS = 8 * 160 * 64 * 128
@@ -88,7 +115,7 @@ def _launch(fn: str, x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n
                      kernels.ptr(part), part.numel() if part is not None else 0, kernels.stream())
         return
     library.call(kernels.lib("gemm_mfma"), fn, x.data_ptr(), x.stride(0), packed.data_ptr(),
-                 kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue, kernels.stream())
+                 kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue, 1, kernels.stream())
 
 
 def try_linear(x: torch.Tensor, lin, out: torch.Tensor) -> bool:

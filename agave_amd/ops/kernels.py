@@ -21,7 +21,7 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 _SIGNATURES = {
     "elementwise": {
         "agave_embed_scale": [_I, _P, _P, _F, _P, _I, _I, _I, _P],
-        "agave_residual_norm": [_I, _P, _P, _L, _P, _F, _P, _L, _P, _F, _P, _I, _I, _P],
+        "agave_residual_norm": [_I, _P, _P, _L, _I, _L, _P, _F, _P, _L, _P, _F, _P, _I, _I, _P],
         "agave_qk_norm_rope_kv": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F,
                                   _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
@@ -121,7 +121,9 @@ def residual_norm(h: torch.Tensor, branch: Optional[torch.Tensor], post_gain: Op
                   post_eps: float, out: Optional[torch.Tensor], pre_gain: Optional[torch.Tensor],
                   pre_eps: float, rows: Optional[torch.Tensor] = None) -> None:
     """If ``branch``: h += rmsnorm(branch) * post_gain.  If ``out``: out = rmsnorm(h) * pre_gain.
-    ``rows`` (int32) picks the rows of ``h`` that ``out`` is computed for."""
+    ``rows`` (int32) picks the rows of ``h`` that ``out`` is computed for.  A three-dimensional
+    float32 ``branch`` [slices, rows, hidden] stands for the sum of its slices (a product that was
+    shared out along its columns)."""
     _dev(h, branch, post_gain, out, pre_gain, rows)
     if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
         raise ValueError("residual stream must be a contiguous float32 [rows, hidden] tensor")
@@ -131,8 +133,15 @@ def residual_norm(h: torch.Tensor, branch: Optional[torch.Tensor], post_gain: Op
     act = branch if branch is not None else out
     if act is None:
         return
-    ldb = ldo = 0
-    if branch is not None:
+    ldb = ldo = n_parts = part_stride = 0
+    if branch is not None and branch.dim() == 3:
+        if branch.dtype != torch.float32 or branch.shape[1:] != (n_h, e) or not branch.is_contiguous():
+            raise ValueError(f"partial sums must be a contiguous float32 [slices, {n_h}, {e}] tensor")
+        n_parts, part_stride, ldb = branch.shape[0], n_h * e, e
+        _f32vec(post_gain, "post_gain", e)
+        if out is not None:
+            act = out
+    elif branch is not None:
         ldb = _rows(branch, "branch")
         if branch.shape != (n_h, e):
             raise ValueError(f"branch must be [{n_h}, {e}], got {tuple(branch.shape)}")
@@ -142,10 +151,10 @@ def residual_norm(h: torch.Tensor, branch: Optional[torch.Tensor], post_gain: Op
         if out.shape != (n, e):
             raise ValueError(f"out must be [{n}, {e}], got {tuple(out.shape)}")
         _f32vec(pre_gain, "pre_gain", e)
-        if branch is not None and branch.dtype != out.dtype:
+        if branch is not None and n_parts == 0 and branch.dtype != out.dtype:
             raise TypeError("branch and out must have the same dtype")
-    library.call(lib("elementwise"), "agave_residual_norm", dt(act), ptr(h), ptr(branch), ldb, ptr(post_gain),
-                 post_eps, ptr(out), ldo, ptr(pre_gain), pre_eps, ptr(rows), n, e, stream())
+    library.call(lib("elementwise"), "agave_residual_norm", dt(act), ptr(h), ptr(branch), ldb, n_parts, part_stride,
+                 ptr(post_gain), post_eps, ptr(out), ldo, ptr(pre_gain), pre_eps, ptr(rows), n, e, stream())
 
 
 def qk_norm_rope_kv(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Optional[torch.Tensor],

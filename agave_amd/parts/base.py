@@ -16,7 +16,8 @@ Interfaces (duck-typed; the classes below document them):
 * mixer:       ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, ``kv_need() -> GroupKey | None``,
                ``state_need() -> StateNeed | None``,
                ``forward(x[N, hidden], step, memory, writes) -> [N, hidden]``.
-* feed-forward: ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, ``forward(x[N, hidden], step) -> [N, hidden]``.
+* feed-forward: ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, ``forward(x[N, hidden], step) -> [N, hidden]``
+               (or float32 [slices, N, hidden] whose slices add up to it: the block's residual kernel adds them).
 * block:       ``tensor_needs(spec)``, ``__init__(spec, weights, env)``,
                ``forward(h, pending, step, memory, writes) -> pending`` (see ``block.py``).
 """

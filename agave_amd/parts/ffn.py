@@ -43,7 +43,7 @@ class GatedFfn:
         if not self.gate_up.forward_geglu(x, act):
             gu = self.gate_up.forward(x, tag="gate_up")
             kernels.geglu(gu[:, :ff], gu[:, ff:], act)
-        return self.down.forward(act, tag="ffn_down")
+        return self.down.forward(act, tag="ffn_down", slices_ok=True)    # the block adds it to the residual stream
 
 
 register("ffn", "gated_dense", GatedFfn)

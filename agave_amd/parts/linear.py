@@ -48,8 +48,22 @@ class Linear:
         self.interleave_ff = interleave_ff if self.packed is not None else 0
 
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
-                out_dtype: Optional[torch.dtype] = None, tag: Optional[str] = None) -> torch.Tensor:
+                out_dtype: Optional[torch.dtype] = None, tag: Optional[str] = None,
+                slices_ok: bool = False) -> torch.Tensor:
+        """``slices_ok``: the caller also takes a float32 [slices, n, out] tensor whose slices add
+        up to the product (a norm that adds a branch to the residual stream does); a product
+        with few rows of W and many columns is then shared out along the columns."""
         n = x.shape[0]
+        if slices_ok and out is None and self.packed is not None and not self.interleave_ff:
+            from ..ops import gemm_mfma, library
+            slices = gemm_mfma.slices_for(n, self.out_features, self.in_features)
+            if slices > 1 and gemm_mfma._x_ok(x):
+                out = self.env.workspace.get((tag or self.name) + "_slices", slices * n, self.out_features,
+                                             torch.float32).view(slices, n, self.out_features)
+                library.profile.label = self.name
+                gemm_mfma.skinny_slices(x, self.packed, out, self.out_features)
+                library.profile.label = None
+                return out
         if out is None:
             out = self.env.workspace.get(tag or self.name, n, self.out_features, out_dtype or x.dtype)
         from ..ops import gemm, library

@@ -70,6 +70,29 @@ def test_residual_norm(K, dtype, e):
     assert torch.allclose(h3.cpu().double(), h.double() + br.double(), atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("e", [72, 2560, 5000])
+def test_residual_norm_takes_a_branch_in_slices(K, dtype, e):
+    """A float32 [slices, rows, hidden] branch stands for the sum of its slices: the same residual
+    stream and output as with the sum given as one 32-bit branch (both row-in-registers and plain kernel)."""
+    n, slices = 5, 3
+    h = torch.randn(n, e) * 3
+    parts = torch.randn(slices, n, e) * 0.3
+    gp, gq = torch.randn(e) * 0.1 + 1, torch.randn(e) * 0.1 + 1
+    hd = h.clone().to(DEV)
+    out = torch.empty(n, e, dtype=dtype, device=DEV)
+    K.residual_norm(hd, parts.to(DEV), gp.to(DEV), 1e-5, out, gq.to(DEV), 3e-6)
+    h_ref = h.double() + P.rms_norm(parts.double().sum(0), gp.double(), 1e-5, add_one=False)
+    o_ref = P.rms_norm(h_ref, gq.double(), 3e-6, add_one=False)
+    assert torch.allclose(hd.cpu().double(), h_ref, atol=3e-6, rtol=1e-6)
+    assert torch.allclose(out.cpu().double(), o_ref, **_tol(dtype))
+    h3 = h.clone().to(DEV)
+    K.residual_norm(h3, parts.to(DEV), None, 0.0, None, None, 0.0)           # a plain add of the slices
+    assert torch.allclose(h3.cpu().double(), h.double() + parts.double().sum(0), atol=2e-6)
+    with pytest.raises(ValueError):
+        K.residual_norm(h3, parts[:, :4].to(DEV), None, 0.0, None, None, 0.0)
+
+
 @pytest.mark.parametrize("n", [128, 1152, 2560, 3136])
 def test_residual_norm_golden(K, n):
     # research/kernels/generate_golden.py:98-110 (eps 1e-5, plain weight)
@@ -376,6 +399,24 @@ def test_gemm_skinny_geglu(G, m, ff, k):
     assert float((out.cpu().double() - ref).abs().max()) <= 8e-3 * float(ref.abs().max())
 
 
+@pytest.mark.parametrize("m,n,k,slices", [(8, 160, 10240, 3), (1, 53, 4104, 2), (16, 256, 2560, 5), (40, 100, 1096, 2)])
+def test_gemm_skinny_in_slices(G, m, n, k, slices):
+    """The product shared out along its columns: the 32-bit slices add up to it; runs of columns of
+    unequal length, and a last one that ends inside a tile."""
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    packed = G.pack_weight(w.to(DEV))
+    out = torch.full((slices, m, n), float("nan"), device=DEV)
+    G.skinny_slices(x.to(DEV), packed, out, n)
+    ref = x.double() @ w.double().T
+    assert float((out.cpu().double().sum(0) - ref).abs().max()) <= 2e-5 * float(ref.abs().max()) * math.sqrt(k / 64)
+    assert float(out[0].abs().max()) > 0 and float(out[-1].abs().max()) > 0
+    with pytest.raises(ValueError):
+        G.skinny_slices(x.to(DEV), packed, out.bfloat16(), n)
+    assert G.slices_for(8, 2560, 10240) > 1 and G.slices_for(8, 10240, 2560) == 1 and G.slices_for(64, 2560, 10240) == 1
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do(G):
     w = G.pack_weight(torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV))
     out = torch.empty(65, 32, dtype=torch.bfloat16, device=DEV)
@@ -493,7 +534,9 @@ def test_attn_mfma_far_key_and_window_edge(K, decode):
                                    (257, 1000, 96), (2048, 300, 136), (130, 4100, 64),
                                    (1000, 4096, 96), (2048, 4090, 64), (1024, 10240, 72),
                                    # many stages (the loads run several stages ahead of the multiplications): each tile
-                                   (300, 2000, 1000), (600, 5000, 1000), (1024, 5120, 1000), (1024, 10240, 1000)])
+                                   (300, 2000, 1000), (600, 5000, 1000), (1024, 5120, 1000), (1024, 10240, 1000),
+                                   # 640 tiles: two rounds of 256 x 256 tiles and the last rows in tiles of half the height
+                                   (2048, 20470, 64)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_tiled(G, m, n, k, out_dtype):
     g = torch.Generator().manual_seed(m + n + k)
@@ -508,7 +551,7 @@ def test_gemm_tiled(G, m, n, k, out_dtype):
     assert float((out.cpu().double() - ref).abs().max()) <= tol
 
 
-@pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40), (1024, 5120, 1000)])
+@pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40), (1024, 5120, 1000), (2048, 10236, 64)])
 def test_gemm_tiled_geglu(G, m, ff, k):
     g = torch.Generator().manual_seed(ff + m)
     x = torch.randn(m, k, generator=g).bfloat16()
