@@ -202,8 +202,14 @@ static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, in
         return false;
     // few rows (decode steps): as many threads per row as it has float4, so that every thread's
     // loads are one round trip; many rows: 256 threads with several float4 each
-    const int threads = (e <= 1024 || (n_rows <= 64 && e <= 4096)) ? 64 * ((e / 4 + 63) / 64)
-                                                                    : (e <= 4096 ? 256 : 1024);
+    int threads;
+    if (e <= 1024 || (n_rows <= 64 && e <= 4096)) {
+        threads = 64 * ((e / 4 + 63) / 64);
+    } else {
+        // two float4 a thread if 1024 threads cover the row so, else four; no more waves than the row needs
+        const int per = e / 4 <= 2048 ? 2 : 4;
+        threads = 64 * ((e / 4 + per * 64 - 1) / (per * 64));
+    }
     const int vpt = (e / 4 + threads - 1) / threads;
 #define RN_FAST(V)                                                                                                    \
     residual_norm_fast_kernel<T, V><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts, part_stride,  \

@@ -623,6 +623,11 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
     }
     }
 
+    // The loads issued for stages past the last one write into this workgroup's LDS: they must
+    // have landed before the workgroup ends and its LDS is given to another (waited for here and
+    // not after the stores below, whose completion would take longer to wait for).
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+
     // D[i][j]: this lane holds token j = lane % 32 and rows i = 8*q + 4*kg + e (q, e = 0..3)
 #pragma unroll
     for (int a = 0; a < WT; ++a) {
