@@ -371,19 +371,23 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
 
 
 // ------------------------------------------------------------------ tiled product (prefill)
-// A workgroup computes WT*64 weight rows x 256 tokens in tiles of 32 x 32
-// (v_mfma_f32_32x32x16_bf16): four waves (2 x 2, a wave WT x 4 tiles) or eight (2 x 4, a wave
-// WT x 2 tiles).  Eight waves are two per SIMD: while one waits for a stage of loads or at the
-// barrier the other multiplies, which a single wave per SIMD cannot hide (a third of its time
-// was waiting); they read a half more from LDS per flop, which the LDS has to spare.
-// Both operands come into LDS straight from
-// global memory (no registers in between), KT k-steps of 32 columns per stage, in a ring of
-// NS buffers: the loads of NS-1 stages ahead are in flight while a stage is multiplied.
+// A workgroup computes WT*64 weight rows x TT tokens in tiles of 32 x 32
+// (v_mfma_f32_32x32x16_bf16) with eight waves (2 x 4, a wave WT x TT/128 tiles): two per SIMD,
+// so that one multiplies while the other waits for a stage of loads, at a barrier or for its
+// operands, which a single wave per SIMD cannot hide (a third of its time was waiting); they
+// read a half more from LDS per flop, which the LDS (256 bytes a clock) has to spare.
+// Both operands come into LDS straight from global memory (no registers in between), KT k-steps
+// of 32 columns per stage, in a ring of NS buffers: the loads of NS-1 stages ahead are in flight
+// while a stage is multiplied.  What a compute unit can load is 64 bytes a clock (a load of one
+// kilobyte keeps its address unit busy for 16 cycles), half of which a 256 x 256 tile needs
+// when the matrix cores never wait; smaller tiles need more, which is why the largest tile that
+// still fills the chip is taken.
 // Weight tiles arrive in their packed order (one kilobyte per wave load; a 32-row operand is
 // read out of two packed 16-row tiles); token rows are stored with their 16-byte pieces
 // permuted so that the rows an MFMA operand reads fall into different banks.
-//   WT 2, KT 2, NS 3:  128 x 256 tiles, 144 KB of LDS - more workgroups for small products
-//   WT 4, KT 1, NS 4:  256 x 256 tiles, 128 KB of LDS - a third less traffic from L2 per flop
+//   WT 4, KT 1, NS 4:  256 x 256 tiles, 128 KB of LDS, the two waves of a SIMD taking turns
+//   WT 2, KT 2, NS 3:  128 x 256 and 128 x 128 tiles - more workgroups for smaller products
+//   WT 1, KT 2, NS 4:  64 x 128 tiles
 // blockIdx.x walks the weight rows, so that workgroups sharing weight rows (ids a multiple of
 // the number of row tiles apart) tend to land on the same XCD and find them in its L2.
 typedef __attribute__((address_space(3))) u32x4_t tl_lds_u32x4;
@@ -397,7 +401,7 @@ template <int I, int N, typename F> __device__ __forceinline__ void static_for(F
     }
 }
 
-template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, int MODE>
+template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, bool TURNS>
 __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
                                                          const uint4* __restrict__ Wp, TC* __restrict__ Y, long ldy,
                                                          int M, int N, int K, int KB, int NB, long part_stride) {
@@ -513,17 +517,15 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
         for (int b = 0; b < XB; ++b) asm volatile("" : "+v"(f.x[b].r));
     };
 
-    // The stage loop.  Loads run NS-1 stages ahead.  MODE says how a wave's work is laid out in time:
-    //   0, 1: loads are issued one at a time between the multiplications (all at once they queue up
-    //      at the address unit, which takes 16 cycles for each, while the matrix cores wait), and the
-    //      operands of a phase are read from LDS while the phase before it multiplies.  1: the first
-    //      operands of the next stage are read during the last phase of this one, for which every
-    //      stage must have landed one barrier earlier.
-    //   2: the two waves of a SIMD take turns (waves 0-3 and 4-7, half a stage apart): one reads its
-    //      operands of a whole stage and issues its loads while the other multiplies, then a barrier,
-    //      and they change places.  The matrix cores then always have a wave that does nothing else.
-    constexpr bool AHEAD = MODE == 1;
-    constexpr int IN_FLIGHT = LOADS * (NS - 2 - (MODE != 0 ? 1 : 0)); // loads that may be outstanding at a barrier
+    // The stage loop.  Loads run NS-1 stages ahead and are issued one at a time between the
+    // multiplications: in their shadow they cost no time, while all at once they queue up at the
+    // address unit, which takes 16 cycles for each, and the matrix cores wait.
+    //   TURNS false: every wave reads the operands of a phase from LDS while the phase before it
+    //      multiplies; the first phase's are read after the stage's barrier.
+    //   TURNS true: the two waves of a SIMD take turns (waves 0-3 and 4-7, half a stage apart): one
+    //      reads its operands of a whole stage while the other multiplies, then a barrier, and they
+    //      change places.  The matrix cores then always have a wave that does nothing else.
+    constexpr int IN_FLIGHT = LOADS * (NS - 2 - (TURNS ? 1 : 0));     // loads that may be outstanding at a barrier
     static_assert(IN_FLIGHT >= 0 && IN_FLIGHT < 64, "the load counter holds 6 bits");
 #pragma unroll
     for (int s0 = 0; s0 < NS - 1; ++s0)
@@ -534,8 +536,27 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
         // a bare barrier: __syncthreads() would also wait for the loads still wanted in flight
         __builtin_amdgcn_s_barrier();
     };
-    if (MODE == 2) {
-        static_assert(MODE != 2 || (NWV == 8 && NS >= 4), "two waves per SIMD take turns; a stage is in flight behind the awaited one");
+    // the multiplications of phase ph with this phase's share (or, all = true, all) of the stage's loads between them
+    auto multiply = [&](const Operands& o, int st, int ph, int first_load, int end_load) {
+        const bool live = KT == 1 || st * KT + (ph >> 1) < KB;
+        int li = first_load;
+#pragma unroll
+        for (int b = 0; b < XB; ++b) {
+            if (live) {
+#pragma unroll
+                for (int a = 0; a < WT; ++a) acc[a][b] = mfma_32x32x16(o.w[a], o.x[b], acc[a][b]);
+            }
+            if (li < end_load) {
+                __builtin_amdgcn_sched_barrier(0);
+                fetch_one(st + NS - 1, li++);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (; li < end_load; ++li) fetch_one(st + NS - 1, li);
+    };
+    if constexpr (TURNS) {
+        static_assert(NWV == 8 && NS >= 4, "two waves per SIMD take turns; a stage is in flight behind the awaited one");
         // Slots between barriers: the first group reads stage i in slot 2i and multiplies in slot
         // 2i+1, the second group one slot later; the loads for stage i+NS-1 are issued while stage
         // i is multiplied.  The first group reads stage i+1 in slot 2i+2, so every wave's loads
@@ -543,7 +564,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
         // wait, after reading stage i: the loads of the NS-3 stages after i+1, all that are issued
         // by then, may be in flight.  (The first group waits at the same place in its own order,
         // a slot earlier than it would have to.)  A buffer is loaded into again at least a slot
-        // after the second group read it.
+        // after the second group read it.  Both groups pass the same number of barriers.
         const bool second = wave >= 4;
         Operands f[PH];
         landed();
@@ -555,72 +576,28 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
             landed();
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_setprio(1);
-            // the loads go between the multiplications: issued in their shadow, they cost no time
-            int li = 0;
 #pragma unroll
-            for (int ph = 0; ph < PH; ++ph) {
-                const bool live = KT == 1 || st * KT + (ph >> 1) < KB;
-#pragma unroll
-                for (int b = 0; b < XB; ++b) {
-                    if (live) {
-#pragma unroll
-                        for (int a = 0; a < WT; ++a) acc[a][b] = mfma_32x32x16(f[ph].w[a], f[ph].x[b], acc[a][b]);
-                    }
-                    if (li < LOADS) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        fetch_one(st + NS - 1, li++);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-            }
-#pragma unroll
-            for (; li < LOADS; ++li) fetch_one(st + NS - 1, li);
+            for (int ph = 0; ph < PH; ++ph)
+                multiply(f[ph], st, ph, ph * LOADS / PH, ph + 1 == PH ? LOADS : (ph + 1) * LOADS / PH);
             __builtin_amdgcn_s_setprio(0);
             __builtin_amdgcn_sched_barrier(0);
             if (!(second && st + 1 == n_stage)) __builtin_amdgcn_s_barrier();
         }
     } else {
-    Operands f[2];
-    if (AHEAD) {
-        landed();
-        read_operands(f[0], st0, IntC<0>{});
-        settle(f[0]);
-    }
-    for (int st = st0; st < n_stage; ++st) {
-        if (!AHEAD) {
+        Operands f[2];
+        for (int st = st0; st < n_stage; ++st) {
             landed();
             read_operands(f[0], st, IntC<0>{});
             settle(f[0]);
+            static_for<0, PH>([&](auto phc) {
+                constexpr int ph = decltype(phc)::value;
+                if constexpr (ph + 1 < PH) read_operands(f[(ph + 1) & 1], st, IntC<ph + 1>{});
+                __builtin_amdgcn_sched_barrier(0);
+                multiply(f[ph & 1], st, ph, (ph * LOADS + PH - 1) / PH, ((ph + 1) * LOADS + PH - 1) / PH);
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (ph + 1 < PH) settle(f[(ph + 1) & 1]);
+            });
         }
-        static_for<0, PH>([&](auto phc) {
-            constexpr int ph = decltype(phc)::value;
-            const bool more = ph + 1 < PH || AHEAD;
-            if constexpr (ph + 1 < PH) read_operands(f[(ph + 1) & 1], st, IntC<ph + 1>{});
-            else if (AHEAD) read_operands(f[0], st + 1, IntC<0>{});     // after the last stage: stale, unused
-            __builtin_amdgcn_sched_barrier(0);
-            const Operands& o = f[ph & 1];
-            const bool live = KT == 1 || st * KT + (ph >> 1) < KB;
-            const int L0 = (ph * LOADS + PH - 1) / PH, L1 = ((ph + 1) * LOADS + PH - 1) / PH;        // this phase's loads
-            int li = L0;
-#pragma unroll
-            for (int b = 0; b < XB; ++b) {
-                if (live) {
-#pragma unroll
-                    for (int a = 0; a < WT; ++a) acc[a][b] = mfma_32x32x16(o.w[a], o.x[b], acc[a][b]);
-                }
-                if (li < L1) {
-                    __builtin_amdgcn_sched_barrier(0);
-                    fetch_one(st + NS - 1, li++);
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            }
-#pragma unroll
-            for (; li < L1; ++li) fetch_one(st + NS - 1, li);
-            __builtin_amdgcn_sched_barrier(0);
-            if (more) settle(f[(ph + 1) & 1]);
-        });
-        if (AHEAD) landed();
-    }
     }
 
     // The loads issued for stages past the last one write into this workgroup's LDS: they must
@@ -669,7 +646,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
     }
 }
 
-template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, int MODE>
+template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, bool TURNS>
 static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB, int NB,
                         hipStream_t stream, int splits = 1, long part_stride = 0) {
     constexpr int WTILES = 4 * WT;
@@ -678,12 +655,12 @@ static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long l
     AGAVE_CHECK(grid.y <= 65535, "gemm_tiled: M=%d exceeds the grid limit", M);
     static bool raised = false;
     if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT, MODE>,
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT, TURNS>,
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         AGAVE_CHECK(e == hipSuccess, "gemm_tiled: cannot raise the LDS allowance");
         raised = true;
     }
-    gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT, MODE><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
+    gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT, TURNS><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
                                                                       M, N, K, KB, NB, part_stride);
     return 0;
 }
@@ -731,8 +708,8 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
     if (splits > 1) {
         const long stride = (long)M * N;
         int rc;
-        if (pick == 2) rc = launch_tiled<2, 2, 3, 0, float, 8, 128, 0>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
-        else rc = launch_tiled<1, 2, 4, 0, float, 8, 128, 0>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
+        if (pick == 2) rc = launch_tiled<2, 2, 3, 0, float, 8, 128, false>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
+        else rc = launch_tiled<1, 2, 4, 0, float, 8, 128, false>(X, ldx, Wp, part, N, M, N, K, KB, NB, stream, splits, stride);
         if (rc != 0) return rc;
         AGAVE_LAUNCH_CHECK("gemm_tiled (partial sums)");
         const long total = (long)M * N;
@@ -752,17 +729,17 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
         if (rows_main > 0) {
             const int nb_main = (int)rows_main * 16;
             const int n_main = EPI == 0 ? nb_main * 16 : nb_main * 8;
-            int rc = launch_tiled<4, 1, 4, EPI, TC, 8, 256, 2>(X, ldx, Wp, Y, ldy, M, n_main, K, KB, nb_main, stream);
+            int rc = launch_tiled<4, 1, 4, EPI, TC, 8, 256, true>(X, ldx, Wp, Y, ldy, M, n_main, K, KB, nb_main, stream);
             if (rc != 0) return rc;
-            return launch_tiled<2, 2, 3, EPI, TC, 8, 256, 0>(X, ldx, (const uint4*)Wp + (size_t)nb_main * KB * 64, (TC*)Y + n_main,
+            return launch_tiled<2, 2, 3, EPI, TC, 8, 256, false>(X, ldx, (const uint4*)Wp + (size_t)nb_main * KB * 64, (TC*)Y + n_main,
                                                              ldy, M, N - n_main, K, KB, NB - nb_main, stream);
         }
     }
     switch (pick) {
-        case 0: return launch_tiled<4, 1, 4, EPI, TC, 8, 256, 2>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-        case 1: return launch_tiled<2, 2, 3, EPI, TC, 8, 256, 0>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-        case 2: return launch_tiled<2, 2, 3, EPI, TC, 8, 128, 0>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
-        default: return launch_tiled<1, 2, 4, EPI, TC, 8, 128, 0>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 0: return launch_tiled<4, 1, 4, EPI, TC, 8, 256, true>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 1: return launch_tiled<2, 2, 3, EPI, TC, 8, 256, false>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 2: return launch_tiled<2, 2, 3, EPI, TC, 8, 128, false>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        default: return launch_tiled<1, 2, 4, EPI, TC, 8, 128, false>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
     }
 }
 
