@@ -58,7 +58,7 @@ def slices_for(m: int, n_out: int, k: int) -> int:
     others cannot ask for memory any faster; with many columns, two or three workgroups share
     each row block."""
     blocks = (n_out + 15) // 16
-    if m < 4 or m > 16 or blocks > 192 or k < 4096:       # (a step of one or two tokens gains nothing)
+    if m < 4 or m > SKINNY_MAX_M or blocks > 192 or k < 4096:       # (a step of one or two tokens gains nothing)
         return 1
     return max(1, min(512 // blocks, k // 2048, 4))
 

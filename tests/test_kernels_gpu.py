@@ -414,7 +414,7 @@ def test_gemm_skinny_in_slices(G, m, n, k, slices):
     assert float(out[0].abs().max()) > 0 and float(out[-1].abs().max()) > 0
     with pytest.raises(ValueError):
         G.skinny_slices(x.to(DEV), packed, out.bfloat16(), n)
-    assert G.slices_for(8, 2560, 10240) > 1 and G.slices_for(8, 10240, 2560) == 1 and G.slices_for(64, 2560, 10240) == 1
+    assert G.slices_for(8, 2560, 10240) > 1 and G.slices_for(8, 10240, 2560) == 1 and G.slices_for(65, 2560, 10240) == 1
 
 
 def test_gemm_skinny_refuses_what_it_cannot_do(G):
