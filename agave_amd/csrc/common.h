@@ -45,17 +45,37 @@ __host__ __device__ __forceinline__ float bf16_to_f32(bf16 v) {
     return c.f;
 }
 
-// round to nearest, ties to even; NaN stays NaN
-__host__ __device__ __forceinline__ bf16 f32_to_bf16(float f) {
-    union { uint32_t u; float f; } c;
-    c.f = f;
-    bf16 r;
-    if ((c.u & 0x7fffffffu) > 0x7f800000u) {
-        r.x = 0x7fc0;
-        return r;
+// round to nearest, ties to even; NaN stays NaN.  On the device this is one instruction for two
+// values (v_cvt_pk_bf16_f32); in software it takes half a dozen, which a product's last step, with
+// 128 values a lane, has no time for.
+__host__ __device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef __bf16 hw_bf16x2 __attribute__((ext_vector_type(2)));
+    typedef float hw_f32x2 __attribute__((ext_vector_type(2)));
+    const hw_f32x2 v = {lo, hi};
+    const hw_bf16x2 r = __builtin_convertvector(v, hw_bf16x2);
+    return __builtin_bit_cast(uint32_t, r);
+#else
+    uint32_t out = 0;
+    const float in[2] = {lo, hi};
+    for (int i = 0; i < 2; ++i) {
+        union { uint32_t u; float f; } c;
+        c.f = in[i];
+        uint32_t h;
+        if ((c.u & 0x7fffffffu) > 0x7f800000u) {
+            h = 0x7fc0;
+        } else {
+            c.u += 0x7fffu + ((c.u >> 16) & 1u);
+            h = c.u >> 16;
+        }
+        out |= h << (16 * i);
     }
-    c.u += 0x7fffu + ((c.u >> 16) & 1u);
-    r.x = (uint16_t)(c.u >> 16);
+    return out;
+#endif
+}
+__host__ __device__ __forceinline__ bf16 f32_to_bf16(float f) {
+    bf16 r;
+    r.x = (uint16_t)(f32x2_to_bf16x2(f, 0.f) & 0xffffu);
     return r;
 }
 

@@ -108,8 +108,8 @@ template <typename T> __device__ __forceinline__ void store4(T* p, float4 v);
 template <> __device__ __forceinline__ void store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
     uint2 u;
-    u.x = (uint32_t)f32_to_bf16(v.x).x | ((uint32_t)f32_to_bf16(v.y).x << 16);
-    u.y = (uint32_t)f32_to_bf16(v.z).x | ((uint32_t)f32_to_bf16(v.w).x << 16);
+    u.x = f32x2_to_bf16x2(v.x, v.y);
+    u.y = f32x2_to_bf16x2(v.z, v.w);
     *reinterpret_cast<uint2*>(p) = u;
 }
 

@@ -19,8 +19,8 @@ template <typename T> __device__ __forceinline__ void store4(T* p, float4 v);
 template <> __device__ __forceinline__ void store4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
     uint2 u;
-    u.x = (uint32_t)f32_to_bf16(v.x).x | ((uint32_t)f32_to_bf16(v.y).x << 16);
-    u.y = (uint32_t)f32_to_bf16(v.z).x | ((uint32_t)f32_to_bf16(v.w).x << 16);
+    u.x = f32x2_to_bf16x2(v.x, v.y);
+    u.y = f32x2_to_bf16x2(v.z, v.w);
     *reinterpret_cast<uint2*>(p) = u;
 }
 
@@ -605,21 +605,77 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
     // not after the stores below, whose completion would take longer to wait for).
     __builtin_amdgcn_s_waitcnt(0x0F70);
 
-    // D[i][j]: this lane holds token j = lane % 32 and rows i = 8*q + 4*kg + e (q, e = 0..3)
+    // D[i][j]: this lane holds token j = lane % 32 and rows i = 8*q + 4*kg + e (q, e = 0..3): four
+    // consecutive outputs of one token, 32 tokens a store, each in a cache line of its own.  Stored
+    // that way the finished tile takes a sixth of the workgroup's time (the same with half the bytes:
+    // it is the number of lines touched that counts).  So the tile goes through LDS, which is free
+    // now, and leaves it row by row: 16 bytes a lane, whole lines.  The 16-byte pieces of a row are
+    // permuted by the token so that the 32 tokens of a store into LDS fall into different banks.
+    constexpr int ES = (int)sizeof(TC);
+    constexpr int OUT_COLS = EPI == 0 ? WT * 64 : WT * 32;            // columns of Y this workgroup computes
+    constexpr int ROW_BYTES = OUT_COLS * ES, CH = ROW_BYTES / 16;     // 16-byte pieces per row
+    constexpr bool VIA_LDS = TT * ROW_BYTES <= NS * STAGE_BYTES && CH >= 1 && CH <= 64;
+    const int n_base = EPI == 0 ? nbw * 16 : nbw * 8;
+    if constexpr (VIA_LDS) {
+        constexpr int SWZ = (CH < 32 ? CH : 32) - 1;
+        __builtin_amdgcn_s_barrier();                                  // every wave has read its last operands
 #pragma unroll
-    for (int a = 0; a < WT; ++a) {
+        for (int a = 0; a < WT; ++a) {
 #pragma unroll
-        for (int b = 0; b < XB; ++b) {
-            const int m = m0 + (wm * XB + b) * 32 + i32;
-            if (m >= M) continue;
+            for (int b = 0; b < XB; ++b) {
+                const int t = (wm * XB + b) * 32 + i32;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int nb = nbw + wn * (2 * WT) + 2 * a + (q >> 1); // packed 16-row tile of these four rows
-                if (nb >= NB) continue;
-                const int r4 = ((2 * q + kg) & 3) * 4;                  // their first row inside that tile
-                const float s0 = acc[a][b][4 * q], s1 = acc[a][b][4 * q + 1], s2 = acc[a][b][4 * q + 2],
-                            s3 = acc[a][b][4 * q + 3];
-                if (EPI == 0) {
+                for (int q = 0; q < 4; ++q) {
+                    const int tile = wn * (2 * WT) + 2 * a + (q >> 1);  // packed 16-row tile of these four rows
+                    const int r4 = ((2 * q + kg) & 3) * 4;              // their first row inside that tile
+                    const float s0 = acc[a][b][4 * q], s1 = acc[a][b][4 * q + 1], s2 = acc[a][b][4 * q + 2],
+                                s3 = acc[a][b][4 * q + 3];
+                    const int off = (EPI == 0 ? tile * 16 + r4 : tile * 8 + (r4 >> 1)) * ES;     // byte in the row
+                    unsigned char* dst = tl_lds + t * ROW_BYTES + (((off >> 4) ^ (t & SWZ)) << 4) + (off & 15);
+                    if (EPI == 0) {
+                        store4(reinterpret_cast<TC*>(dst), float4{s0, s1, s2, s3});
+                    } else {
+                        const float v0 = gelu_tanh_f(s0) * s2, v1 = gelu_tanh_f(s1) * s3;
+                        *reinterpret_cast<uint32_t*>(dst) = f32x2_to_bf16x2(v0, v1);
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        constexpr int EPC = 16 / ES;                                    // elements per piece
+        constexpr int ROWS_PER = 64 / CH;                               // rows one store instruction covers
+        const bool whole = (((uintptr_t)Y | (uintptr_t)(ldy * ES)) & 15) == 0;       // pieces are aligned in memory
+        const int piece = lane % CH;
+#pragma unroll 4
+        for (int r = wave * ROWS_PER + lane / CH; r < TT; r += NWV * ROWS_PER) {
+            const int m = m0 + r, n = n_base + piece * EPC;
+            if (m >= M || n >= N) continue;
+            const uint4 v = *reinterpret_cast<const uint4*>(tl_lds + r * ROW_BYTES + ((piece ^ (r & SWZ)) << 4));
+            TC* dst = Y + (size_t)m * ldy + n;
+            if (whole && n + EPC <= N) {
+                *reinterpret_cast<uint4*>(dst) = v;
+            } else {
+                const TC* e = reinterpret_cast<const TC*>(&v);
+#pragma unroll
+                for (int i = 0; i < EPC; ++i)
+                    if (n + i < N) dst[i] = e[i];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int a = 0; a < WT; ++a) {
+#pragma unroll
+            for (int b = 0; b < XB; ++b) {
+                const int m = m0 + (wm * XB + b) * 32 + i32;
+                if (m >= M) continue;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nb = nbw + wn * (2 * WT) + 2 * a + (q >> 1);
+                    if (nb >= NB) continue;
+                    const int r4 = ((2 * q + kg) & 3) * 4;
+                    const float s0 = acc[a][b][4 * q], s1 = acc[a][b][4 * q + 1], s2 = acc[a][b][4 * q + 2],
+                                s3 = acc[a][b][4 * q + 3];
+                    static_assert(VIA_LDS || EPI == 0, "only a plain 32-bit tile is too large for the LDS");
                     const int n = nb * 16 + r4;
                     TC* dst = Y + (size_t)m * ldy + n;
                     if (n + 3 < N && (ldy & 3) == 0) {
@@ -629,16 +685,6 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
                         if (n + 1 < N) st(dst + 1, s1);
                         if (n + 2 < N) st(dst + 2, s2);
                         if (n + 3 < N) st(dst + 3, s3);
-                    }
-                } else {
-                    const int n = nb * 8 + (r4 >> 1);                   // N counts output columns (ff)
-                    const float v0 = gelu_tanh_f(s0) * s2, v1 = gelu_tanh_f(s1) * s3;
-                    if (n + 1 < N && (ldy & 1) == 0) {
-                        const uint32_t u = (uint32_t)f32_to_bf16(v0).x | ((uint32_t)f32_to_bf16(v1).x << 16);
-                        *reinterpret_cast<uint32_t*>(Y + (size_t)m * ldy + n) = u;
-                    } else {
-                        if (n < N) st(Y + (size_t)m * ldy + n, v0);
-                        if (n + 1 < N) st(Y + (size_t)m * ldy + n + 1, v1);
                     }
                 }
             }
