@@ -53,14 +53,18 @@ def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int,
 
 
 def slices_for(m: int, n_out: int, k: int) -> int:
-    """How many slices of partial sums a product of few tokens is worth: its row blocks are its
-    workgroups, and fewer than some 200 of them leave compute units without work while the
-    others cannot ask for memory any faster; with many columns, two or three workgroups share
-    each row block."""
+    """How many slices of partial sums a product of few tokens is worth.  Its row blocks are its
+    workgroups, 256 of which run at a time: 160 leave compute units without work while the others
+    cannot ask for memory any faster, 336 leave most of them idle in the second round.  With
+    many columns, two to four workgroups then share each row block, whichever fills the rounds best."""
     blocks = (n_out + 15) // 16
-    if m < 4 or m > SKINNY_MAX_M or blocks > 192 or k < 4096:       # (a step of one or two tokens gains nothing)
+
+    def filled(groups: int) -> float:
+        return groups / (256.0 * ((groups + 255) // 256))
+    if m < 4 or m > SKINNY_MAX_M or k < 4096 or filled(blocks) >= 0.85:      # (a step of one or two tokens gains nothing)
         return 1
-    return max(1, min(512 // blocks, k // 2048, 4))
+    best = max((s for s in (2, 3, 4) if k // s >= 1024), key=lambda s: (filled(blocks * s), -s), default=1)
+    return best if filled(blocks * best) > filled(blocks) + 0.1 else 1
 
 
 def skinny_slices(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int) -> None:

@@ -71,7 +71,7 @@ class Attention:
             inv_freq, pos_scale = fused()
             attn_ops.qk_attention(q, k, v, q_out, ctx_out, qg, kg, qe, ke, inv_freq, pos_scale, k_pages, v_pages,
                                   table, base, step, s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, packed)
-            return self.o.forward(ctx_out, tag="attn_o")
+            return self.o.forward(ctx_out, tag="attn_o", slices_ok=True)       # the block adds it to the residual stream
         else:
             # a position encoding the q/k kernel does not know: the norms, then the part's own
             # ``apply`` on the normalised rows, then the cache write
@@ -89,7 +89,7 @@ class Attention:
                                         packed)
         attn_ops.attention(q_out, ctx_out, k_pages, v_pages, table, base, step, s.n_heads, s.n_kv_heads,
                            s.head_dim, s.scale, s.window, packed)
-        return self.o.forward(ctx_out, tag="attn_o")
+        return self.o.forward(ctx_out, tag="attn_o", slices_ok=True)       # the block adds it to the residual stream
 
 
 register("mixer", "attention", Attention)

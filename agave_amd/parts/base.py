@@ -15,7 +15,7 @@ Interfaces (duck-typed; the classes below document them):
                (k is None in a run that appends nothing), positions in ``step.tok_pos``.
 * mixer:       ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, ``kv_need() -> GroupKey | None``,
                ``state_need() -> StateNeed | None``,
-               ``forward(x[N, hidden], step, memory, writes) -> [N, hidden]``.
+               ``forward(x[N, hidden], step, memory, writes) -> [N, hidden]`` (or slices of it, as below).
 * feed-forward: ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, ``forward(x[N, hidden], step) -> [N, hidden]``
                (or float32 [slices, N, hidden] whose slices add up to it: the block's residual kernel adds them).
 * block:       ``tensor_needs(spec)``, ``__init__(spec, weights, env)``,
