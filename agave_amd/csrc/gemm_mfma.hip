@@ -303,16 +303,62 @@ static void launch_skinny(const void* X, long ldx, const void* Wp, void* Y, long
     }
 }
 
+// How a product of few tokens is cut into workgroups: r row blocks (of 16 weight rows) by 1/z of
+// the columns each.  z > 1 only where the reader takes 32-bit slices that add up to the product.
+//
+// 256 workgroups run at a time, and a compute unit cannot pull more than some 40 GB/s: the
+// workgroups must fill their rounds evenly (1280 row blocks at 4 a workgroup are 320
+// workgroups, a quarter of the compute units with twice the others' work, and take a third
+// longer than at 5 a workgroup; 160 row blocks leave 96 compute units idle).  Every workgroup
+// reads the X columns of its slice, so what comes from L2 besides the weights is X once per
+// group of r row blocks, whatever z is: with many tokens, many row blocks a workgroup and many
+// slices are better than few of either (X counted half, it comes from L2).  A slice more costs
+// its partial sums.  With one tile of tokens X is small, and the older, measured rule stands.
+struct SkinnyCut { int r, z; };
+// only_z > 0: the best row blocks for exactly that many slices.
+static SkinnyCut cut_skinny(int M, int NB, int KB, int max_z, int only_z = 0) {
+    const int mt = (M + 15) / 16;
+    auto filled = [](long groups) { return (double)groups / (256.0 * ((groups + 255) / 256)); };
+    SkinnyCut cut = {1, 1};
+    if (mt == 1) {
+        cut.r = NB >= 4096 ? 2 : 1;
+        const long groups = (NB + cut.r - 1) / cut.r;
+        if (only_z > 0) {
+            cut.z = only_z;
+            return cut;
+        }
+        if (M < 4 || KB < 128 || filled(groups) >= 0.85) return cut;       // (one or two tokens gain nothing)
+        double best = filled(groups) + 0.1;
+        for (int z = 2; z <= 4 && z <= max_z && KB / z >= 32; ++z)
+            if (filled(groups * z) > best) {
+                best = filled(groups * z);
+                cut.z = z;
+            }
+        return cut;
+    }
+    static const int cand2[] = {1, 2, 4, 5, 0}, cand3[] = {1, 4, 5, 0};
+    const int* cand = mt == 2 ? cand2 : cand3;
+    const int n_chunks = (KB + (mt <= 2 ? 4 : 2) - 1) / (mt <= 2 ? 4 : 2);
+    double best = 1e30;
+    for (int i = 0; cand[i]; ++i) {
+        for (int z = only_z > 0 ? only_z : 1; z <= (only_z > 0 ? only_z : (max_z < 8 ? max_z : 8)); ++z) {
+            if (only_z == 0 && z > 1 && n_chunks / z < 8) break;
+            const long groups = (long)((NB + cand[i] - 1) / cand[i]) * z;
+            const double cost = (1.0 + 0.5 * mt / cand[i]) / filled(groups) + 0.03 * (z - 1);
+            if (cost < best) {
+                best = cost;
+                cut = {cand[i], z};
+            }
+        }
+    }
+    return cut;
+}
+
 template <int EPI, typename TC>
 static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB,
                            int NB, int splits, hipStream_t stream) {
     const int mt = (M + 15) / 16;
-    // Row blocks per workgroup: every workgroup reads all of X, so the traffic from L2 is
-    // (1 + 16*MT/(16*R)) times the weights'; more row blocks as long as enough workgroups remain.
-    int r = 1;
-    if (mt == 1) r = NB >= 4096 ? 2 : 1;
-    else if (mt == 2) r = NB >= 4096 ? 4 : (NB >= 1024 ? 2 : 1);
-    else r = NB >= 1024 ? 4 : 1;
+    const int r = cut_skinny(M, NB, KB, splits, splits).r;       // the row blocks that go with this many slices
 #define SK_CASE(R_, MT_)                                                                        \
     launch_skinny<R_, MT_, EPI, TC, 16>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, splits, stream);          \
     break
@@ -327,15 +373,25 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
         case 2 * 8 + 1: SK_CASE(1, 2);
         case 2 * 8 + 2: SK_CASE(2, 2);
         case 2 * 8 + 4: SK_CASE(4, 2);
+        case 2 * 8 + 5: SK_CASE(5, 2);
         case 3 * 8 + 1: SK_CASE(1, 3);
         case 3 * 8 + 4: SK_CASE(4, 3);
+        case 3 * 8 + 5: SK_CASE(5, 3);
         case 4 * 8 + 1: SK_CASE(1, 4);
         case 4 * 8 + 4: SK_CASE(4, 4);
+        case 4 * 8 + 5: SK_CASE(5, 4);
         default: AGAVE_CHECK(false, "gemm_skinny: no kernel for %d tokens with %d row blocks a workgroup", M, r);
     }
 #undef SK_CASE1
 #undef SK_CASE
     return 0;
+}
+
+// How many 32-bit slices a product of M <= 64 tokens is best computed in by a caller that can add
+// them up (1: as one product).
+extern "C" int agave_gemm_skinny_slices(int M, int N, int K) {
+    if (M <= 0 || M > 64 || N <= 0 || K <= 0) return 1;
+    return cut_skinny(M, (N + 15) / 16, (K + 31) / 32, 8).z;
 }
 
 // N: logical outputs (rows of W, or ff for the GeGLU epilogue); Wp holds NB row blocks.
@@ -352,7 +408,7 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
     if (M == 0) return 0;
     const int KB = (K + 31) / 32;
     const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
-    AGAVE_CHECK(splits >= 1 && splits <= 64 && (splits == 1 || splits * 16 <= KB), "gemm_skinny: %d slices for %d columns",
+    AGAVE_CHECK(splits >= 1 && splits <= 64 && (splits == 1 || splits * 4 <= KB), "gemm_skinny: %d slices for %d columns",
                 splits, K);
     AGAVE_CHECK(splits == 1 || (epilogue == 0 && dt_y == AGAVE_F32), "gemm_skinny: partial sums are plain 32-bit sums");
     int rc;

@@ -12,6 +12,7 @@ kernels.register_signatures("gemm_mfma", {
     "agave_pack_w16": [_P, _L, _P, _I, _I, _I, _I, _P],
     "agave_embed_scale_packed": [_P, _P, _F, _P, _I, _I, _I, _P],
     "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _I, _P],
+    "agave_gemm_skinny_slices": [_I, _I, _I],
     "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P, _L, _P],
 })
 
@@ -52,19 +53,20 @@ def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int,
     _launch("agave_gemm_skinny", x, packed, out, n_out, epilogue)
 
 
-def slices_for(m: int, n_out: int, k: int) -> int:
-    """How many slices of partial sums a product of few tokens is worth.  Its row blocks are its
-    workgroups, 256 of which run at a time: 160 leave compute units without work while the others
-    cannot ask for memory any faster, 336 leave most of them idle in the second round.  With
-    many columns, two to four workgroups then share each row block, whichever fills the rounds best."""
-    blocks = (n_out + 15) // 16
+_slices = {}
 
-    def filled(groups: int) -> float:
-        return groups / (256.0 * ((groups + 255) // 256))
-    if m < 4 or m > SKINNY_MAX_M or k < 4096 or filled(blocks) >= 0.85:      # (a step of one or two tokens gains nothing)
-        return 1
-    best = max((s for s in (2, 3, 4) if k // s >= 1024), key=lambda s: (filled(blocks * s), -s), default=1)
-    return best if filled(blocks * best) > filled(blocks) + 0.1 else 1
+
+def slices_for(m: int, n_out: int, k: int) -> int:
+    """How many 32-bit slices a product of few tokens is worth to a caller that can add them up
+    (the kernel library decides: it knows how it cuts a product into workgroups)."""
+    key = (m, n_out, k)
+    got = _slices.get(key)
+    if got is None:
+        got = 1
+        if 0 < m <= SKINNY_MAX_M:
+            fn = kernels.lib("gemm_mfma").agave_gemm_skinny_slices
+            got = _slices[key] = int(fn(m, n_out, k))
+    return got
 
 
 def skinny_slices(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int) -> None:
