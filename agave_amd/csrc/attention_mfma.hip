@@ -822,9 +822,16 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     const int lo_blk = a.window > 0 ? (p_blk0 - a.window + 1 > 0 ? p_blk0 - a.window + 1 : 0) : 0;
     const int page_first = lo_blk / AGAVE_PAGE, page_last = (p_blk0 + blk_n - 1) / AGAVE_PAGE;
 
+    // The ids of the pages this workgroup goes through, looked up once: a lookup inside the loop
+    // is two dependent loads from memory a page, and waiting for them also waits for the next
+    // page's loads, which were issued just before and should travel while this page is worked on.
+    int* pg_ids = reinterpret_cast<int*>(page_lds + (size_t)2 * buf_tiles * 64);
+    for (int i = threadIdx.x; i <= page_last - page_first; i += NWV * 64) pg_ids[i] = (int)page_of(a, b, page_first + i);
+    __syncthreads();
+
     constexpr size_t k_stride = (size_t)n_k * 64, v_stride = (size_t)n_v * 64;
     auto fetch = [&](int pi, int buf) {
-        const long pg = page_of(a, b, pi);
+        const long pg = __builtin_amdgcn_readfirstlane(pg_ids[pi - page_first]);
         if (pg < 0) return;
         const uint4* ksrc = a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride;
         const uint4* vsrc = a.v_pages + ((size_t)pg * a.nkv + kvh) * v_stride;
@@ -842,22 +849,33 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     for (int pi = page_first; pi <= page_last; ++pi) {
         const int buf = (pi - page_first) & 1;
         if (pi < page_last) fetch(pi + 1, buf ^ 1);
-        if (wave_on && pi >= my_first && pi <= my_last && page_of(a, b, pi) >= 0) {
-            const lds_u32x4* kl = (const lds_u32x4*)(page_lds + (size_t)buf * buf_tiles * 64);
-            const lds_u32x4* vl = kl + (size_t)n_k * 64;
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
+        if (wave_on && pi >= my_first && pi <= my_last && pg_ids[pi - page_first] >= 0) {
+            // this lane's 16 bytes of the page's first tile; tiles follow each other by 1 KB
+            const unsigned kaddr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint4*)page_lds +
+                                   (unsigned)(buf * buf_tiles * 64 + lane) * 16u;
+            static_for<0, 2>([&](auto halfc) {
+                constexpr int half = decltype(halfc)::value;
                 const int key0 = pi * AGAVE_PAGE + 32 * half;
-                if (key0 > p_max || key0 + 31 < lo_min) continue;              // no column sees this unit
+                if (key0 > p_max || key0 + 31 < lo_min) return;                // no column sees this unit
+                // all of the unit's key tiles are asked for at once, then multiplied; the value tiles
+                // are asked for before the exponentials and arrive while those are computed
+                frag16 fr[2 * KS > HDT ? 2 * KS : HDT];
+                static_for<0, KS>([&](auto ks) {
+                    lds_read16<((2 * half) * KS + ks.value) * 1024>(fr[2 * ks.value], kaddr);
+                    lds_read16<((2 * half + 1) * KS + ks.value) * 1024>(fr[2 * ks.value + 1], kaddr);
+                });
+                lds_settle();
+#pragma unroll
+                for (int i = 0; i < 2 * KS; ++i) lds_use(fr[i]);
                 f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    frag16 k0, k1;
-                    k0.r = kl[((2 * half) * KS + ks) * 64 + lane];
-                    k1.r = kl[((2 * half + 1) * KS + ks) * 64 + lane];
-                    st0 = mfma_16x16x32(k0, qf[ks], st0);
-                    st1 = mfma_16x16x32(k1, qf[ks], st1);
+                    st0 = mfma_16x16x32(fr[2 * ks], qf[ks], st0);
+                    st1 = mfma_16x16x32(fr[2 * ks + 1], qf[ks], st1);
                 }
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<0, HDT>([&](auto d) { lds_read16<(n_k + d.value * 2 + half) * 1024>(fr[d.value], kaddr); });
+                __builtin_amdgcn_sched_barrier(0);
                 float s[8];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
@@ -898,13 +916,13 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
                     pf.v[e] = (__bf16)pe;
                 }
                 l += sum;
+                lds_settle();
 #pragma unroll
                 for (int d = 0; d < HDT; ++d) {
-                    frag16 vb;
-                    vb.r = vl[(d * 2 + half) * 64 + lane];
-                    o[d] = mfma_16x16x32(pf, vb, o[d]);
+                    lds_use(fr[d]);
+                    o[d] = mfma_16x16x32(pf, fr[d], o[d]);
                 }
-            }
+            });
         }
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
@@ -1058,14 +1076,17 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
                         "attn_prefill_mfma: cannot raise the LDS allowance");
         raised = true;
     }
+    // the streamlined kernel also keeps the ids of a workgroup's pages in LDS (at most the table's width)
+    const size_t lds_fast = lds + (size_t)width * sizeof(int);
+    AGAVE_CHECK(!fast || lds_fast <= 144 * 1024, "attn_prefill_mfma: a page table of %d columns does not fit the LDS", width);
     if (fast && nwv == 8) {
-        if (hd == 64) attn_prefill_fast_kernel<4, 8><<<grid, 512, lds, stream>>>(a, hw);
-        else if (hd == 128) attn_prefill_fast_kernel<8, 8><<<grid, 512, lds, stream>>>(a, hw);
-        else attn_prefill_fast_kernel<16, 8><<<grid, 512, lds, stream>>>(a, hw);
+        if (hd == 64) attn_prefill_fast_kernel<4, 8><<<grid, 512, lds_fast, stream>>>(a, hw);
+        else if (hd == 128) attn_prefill_fast_kernel<8, 8><<<grid, 512, lds_fast, stream>>>(a, hw);
+        else attn_prefill_fast_kernel<16, 8><<<grid, 512, lds_fast, stream>>>(a, hw);
     } else if (fast) {
-        if (hd == 64) attn_prefill_fast_kernel<4, 4><<<grid, 256, lds, stream>>>(a, hw);
-        else if (hd == 128) attn_prefill_fast_kernel<8, 4><<<grid, 256, lds, stream>>>(a, hw);
-        else attn_prefill_fast_kernel<16, 4><<<grid, 256, lds, stream>>>(a, hw);
+        if (hd == 64) attn_prefill_fast_kernel<4, 4><<<grid, 256, lds_fast, stream>>>(a, hw);
+        else if (hd == 128) attn_prefill_fast_kernel<8, 4><<<grid, 256, lds_fast, stream>>>(a, hw);
+        else attn_prefill_fast_kernel<16, 4><<<grid, 256, lds_fast, stream>>>(a, hw);
     } else if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else if (hd <= 128) attn_prefill_mfma_kernel<8, 2><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else attn_prefill_mfma_kernel<16, 1><<<grid, 256, lds, stream>>>(a, qt_heads, hw);

@@ -448,14 +448,6 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
 // the number of row tiles apart) tend to land on the same XCD and find them in its L2.
 typedef __attribute__((address_space(3))) u32x4_t tl_lds_u32x4;
 
-// a loop whose index is a compile-time constant in the body (f gets IntC<I>): for instructions' immediate fields
-template <int I> struct IntC { static constexpr int value = I; };
-template <int I, int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
-    if constexpr (I < N) {
-        f(IntC<I>{});
-        static_for<I + 1, N>(f);
-    }
-}
 
 template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, bool TURNS>
 __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,

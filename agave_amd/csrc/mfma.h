@@ -36,3 +36,23 @@ typedef float f32x16_t __attribute__((ext_vector_type(16)));
 __device__ __forceinline__ f32x16_t mfma_32x32x16(const frag16& a, const frag16& b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
 }
+
+// A loop whose index is a compile-time constant in the body (f gets IntC<I>): for instructions' immediate fields.
+template <int I> struct IntC { static constexpr int value = I; };
+template <int I, int N, typename F> __device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(IntC<I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+// An LDS read written as an instruction, for kernels that also load straight into LDS: the compiler
+// counts such a load as an LDS access of unknown order and then waits for every pending LDS read
+// where one is used, the ones just asked for included; or it keeps so few reads in flight that
+// every multiplication waits out the LDS's latency.  The caller places the wait: lds_settle after
+// the reads, then lds_use on each value before its first use.
+template <int OFFSET> __device__ __forceinline__ void lds_read16(frag16& dst, unsigned addr) {
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst.r) : "v"(addr), "n"(OFFSET));
+}
+__device__ __forceinline__ void lds_settle() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void lds_use(frag16& v) { asm volatile("" : "+v"(v.r)); }
