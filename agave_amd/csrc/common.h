@@ -88,15 +88,31 @@ template <> __device__ __forceinline__ void st<float>(float* p, float v) { *p = 
 template <> __device__ __forceinline__ void st<bf16>(bf16* p, float v) { *p = f32_to_bf16(v); }
 
 // ---------------------------------------------------------------- wave64 reductions
+// With the lanes' cross-lane operand modes (DPP): six vector instructions and a read of lane 63,
+// where a shuffle is an LDS instruction with its latency each time (six to a reduction).
+//   quad_perm, row_half_mirror, row_mirror: every lane gets its row's (16 lanes') result;
+//   row_bcast15 to rows 1 and 3, row_bcast31 to rows 2 and 3: lane 63 gets the wave's.
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float dpp_get(float keep, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, keep), __builtin_bit_cast(int, v),
+                                                                 CTRL, ROW_MASK, 0xF, false));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+    v += dpp_get<0xB1, 0xF>(0.f, v);          // quad_perm [1,0,3,2]
+    v += dpp_get<0x4E, 0xF>(0.f, v);          // quad_perm [2,3,0,1]
+    v += dpp_get<0x141, 0xF>(0.f, v);         // row_half_mirror
+    v += dpp_get<0x140, 0xF>(0.f, v);         // row_mirror
+    v += dpp_get<0x142, 0xA>(0.f, v);         // row_bcast15
+    v += dpp_get<0x143, 0xC>(0.f, v);         // row_bcast31
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fmaxf(v, dpp_get<0xB1, 0xF>(v, v));
+    v = fmaxf(v, dpp_get<0x4E, 0xF>(v, v));
+    v = fmaxf(v, dpp_get<0x141, 0xF>(v, v));
+    v = fmaxf(v, dpp_get<0x140, 0xF>(v, v));
+    v = fmaxf(v, dpp_get<0x142, 0xA>(v, v));
+    v = fmaxf(v, dpp_get<0x143, 0xC>(v, v));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
 // Block-wide reductions for blocks of up to 1024 threads; `red` is 16 floats of LDS.
