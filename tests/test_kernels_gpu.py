@@ -417,6 +417,31 @@ def test_gemm_skinny_in_slices(G, m, n, k, slices):
     assert G.slices_for(8, 2560, 10240) > 1 and G.slices_for(8, 10240, 2560) == 1 and G.slices_for(65, 2560, 10240) == 1
 
 
+def test_product_of_many_shapes(G):
+    """Shapes drawn at random (fixed seed) across the kernels' cuts: tokens from 1 to 700, rows and
+    columns that are multiples of nothing in particular (columns a multiple of 8, which the packed
+    product requires), plain and sliced; each against a 64-bit product."""
+    rng = np.random.default_rng(7)
+    for case in range(48):
+        m = int(rng.choice([1, 3, 8, 15, 16, 17, 31, 33, 48, 63, 64, 65, 100, 129, 255, 257, 400, 700]))
+        n = int(rng.integers(1, 6000))
+        k = 8 * int(rng.integers(1, 700))
+        g = torch.Generator().manual_seed(case)
+        x = torch.randn(m, k, generator=g).bfloat16()
+        w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+        packed = G.pack_weight(w.to(DEV))
+        ref = x.double() @ w.double().T
+        scale = float(ref.abs().max()) + 1e-6
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+        G.product(x.to(DEV), packed, out, n)
+        assert float((out.cpu().double() - ref).abs().max()) <= 6e-3 * scale, (case, m, n, k)
+        z = G.slices_for(m, n, k)
+        if z > 1:
+            parts = torch.full((z, m, n), float("nan"), device=DEV)
+            G.skinny_slices(x.to(DEV), packed, parts, n)
+            assert float((parts.cpu().double().sum(0) - ref).abs().max()) <= 2e-5 * scale * math.sqrt(k / 64), (case, m, n, k, z)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_do(G):
     w = G.pack_weight(torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV))
     out = torch.empty(65, 32, dtype=torch.bfloat16, device=DEV)
