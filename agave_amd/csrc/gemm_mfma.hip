@@ -30,7 +30,7 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
 //         4q+0, 4q+1 are gate[8nb+2q], gate[8nb+2q+1] and rows 4q+2, 4q+3 the same two of up.
 __global__ void pack_w16_kernel(const bf16* __restrict__ W, long ldw, uint4* __restrict__ P, int N, int K,
                                 int NB, int KB, int mode, int ff) {
-    const long tile = blockIdx.x;          // nb * KB + kb
+    const long tile = blockIdx.x;          // source order: nb * KB + kb
     const int nb = (int)(tile / KB), kb = (int)(tile % KB);
     const int lane = threadIdx.x;
     const int i = lane & 15, g = lane >> 4;
@@ -51,7 +51,7 @@ __global__ void pack_w16_kernel(const bf16* __restrict__ W, long ldw, uint4* __r
         z.x = 0;
         f.h[e] = (src >= 0 && k < K) ? W[src * ldw + k] : z;
     }
-    P[tile * 64 + lane] = f.u;
+    P[w_tile(nb, kb, NB, KB) * 64 + lane] = f.u;
 }
 
 extern "C" int agave_pack_w16(const void* W, long ldw, void* P, int N, int K, int mode, int ff, hipStream_t stream) {
@@ -78,7 +78,7 @@ __global__ void embed_scale_packed_kernel(const int* __restrict__ tokens, const 
     for (int piece = threadIdx.x; piece * 8 < e; piece += blockDim.x) {     // 8 columns per piece
         const int kb = piece >> 2, g = piece & 3;
         frag16 f;
-        f.u = P[((size_t)nb * KB + kb) * 64 + i + 16 * g];
+        f.u = P[w_tile(nb, kb, (vocab + 15) / 16, KB) * 64 + i + 16 * g];
 #pragma unroll
         for (int x = 0; x < 8; ++x) {
             const int k = piece * 8 + x;
@@ -163,7 +163,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     // results are never stored)
     const uint4* wrow[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) wrow[r] = Wp + (size_t)(nb0 + r < NB ? nb0 + r : NB - 1) * KB * 64 + lane;
+    for (int r = 0; r < R; ++r) wrow[r] = Wp + w_tile(nb0 + r < NB ? nb0 + r : NB - 1, 0, NB, KB) * 64 + lane;
+    const size_t wstep = (w_tile(0, 1, NB, KB) - w_tile(0, 0, NB, KB)) * 64;        // from a k-step to the next
     const bf16* xrow[MT][NI];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
@@ -173,22 +174,19 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
             xrow[mt][i] = X + (size_t)(row < M ? row : M - 1) * ldx;
         }
 
-    // Workgroups walk the columns from different starting chunks (and wrap around): row blocks lie
-    // a multiple of the memory channels' period apart for some K, and workgroups that move in step
-    // would then all read from the same few channels.
-    const int rot = blockIdx.x % n_chunks;
+    // Workgroups walk the columns in step: the tiles of a k-step lie side by side in the packed
+    // matrix, so what the workgroups read at any moment is one contiguous stretch of memory.
     // Loads are issued without any condition around them (a chunk past the end repeats the last
     // one and is not used): only then can a wait name the loads it needs and leave the younger
     // ones in flight.
 #define SK_LOAD(ST, IT)                                                                          \
     {                                                                                            \
         int c_ = (IT) * NW + wave;                    /* chunks are dealt to the waves in turn */ \
-        c_ = (c_ < n_chunks ? c_ : n_chunks - 1) + rot;                                          \
-        c_ = (c_ < n_chunks ? c_ : c_ - n_chunks) + c_lo;                                        \
+        c_ = (c_ < n_chunks ? c_ : n_chunks - 1) + c_lo;                                         \
         _Pragma("unroll") for (int r = 0; r < R; ++r)                                            \
             _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                  \
                 const int kb = c_ * KS + ks;           /* past the last tile: any tile, X is zero there */ \
-                wreg[ST][r][ks].u = wrow[r][(size_t)(kb < KB ? kb : KB - 1) * 64];               \
+                wreg[ST][r][ks].u = wrow[r][(size_t)(kb < KB ? kb : KB - 1) * wstep];            \
             }                                                                                    \
         const int k_ = c_ * (KS * 32) + xp * 8;         /* past the last column: any piece, zeroed when used */ \
         _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                        \
@@ -198,8 +196,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16* __rest
     // The staged rows are this wave's own and LDS serves a wave's accesses in order: no barrier.
 #define SK_USE(ST, IT)                                                                           \
     if ((IT) * NW + wave < n_chunks) {                                                           \
-        const int pc_ = (IT) * NW + wave + rot;                                                  \
-        const bool in_ = ((pc_ < n_chunks ? pc_ : pc_ - n_chunks) + c_lo) * (KS * 32) + xp * 8 < K; \
+        const bool in_ = ((IT) * NW + wave + c_lo) * (KS * 32) + xp * 8 < K;                     \
         _Pragma("unroll") for (int mt = 0; mt < MT; ++mt)                                        \
             _Pragma("unroll") for (int i = 0; i < NI; ++i)                                       \
                 *reinterpret_cast<uint4*>(my_xs + (mt * 16 + RPI * i + xr) * ROW + xp * 8) =     \
@@ -452,7 +449,8 @@ typedef __attribute__((address_space(3))) u32x4_t tl_lds_u32x4;
 template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, bool TURNS>
 __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __restrict__ X, long ldx,
                                                          const uint4* __restrict__ Wp, TC* __restrict__ Y, long ldy,
-                                                         int M, int N, int K, int KB, int NB, long part_stride) {
+                                                         int M, int N, int K, int KB, int NB, int NBS, long part_stride) {
+    // NBS: row blocks of the whole packed matrix (Wp may point at a later row block of it)
     constexpr int CPR = KT * 4;                       // 16-byte pieces per staged token row
     constexpr int RP = 16 / CPR;                      // token rows per 256 bytes of LDS
     constexpr int WTILES = 4 * WT;                    // packed 16-row weight tiles per workgroup
@@ -519,7 +517,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
             int nb = nbw + tt / KT, kb = ste * KT + tt % KT;
             if (nb >= NB) nb = NB - 1;                                 // rows past the end: never stored
             if (kb >= KB) kb = KB - 1;                                 // k-steps past the end: never multiplied
-            const unsigned char* src = (const unsigned char*)(Wp + ((size_t)nb * KB + kb) * 64);
+            const unsigned char* src = (const unsigned char*)(Wp + w_tile(nb, kb, NBS, KB) * 64);
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(src + woff),
                                              (__attribute__((address_space(3))) void*)(buf + X_BYTES + tt * 1024), 16, 0, 0);
         }
@@ -742,7 +740,7 @@ __global__ __launch_bounds__(NWV * 64, 2) void gemm_tiled_kernel(const bf16* __r
 
 template <int WT, int KT, int NS, int EPI, typename TC, int NWV, int TT, bool TURNS>
 static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K, int KB, int NB,
-                        hipStream_t stream, int splits = 1, long part_stride = 0) {
+                        hipStream_t stream, int splits = 1, long part_stride = 0, int NBS = 0) {
     constexpr int WTILES = 4 * WT;
     const size_t lds = (size_t)NS * (TT * KT * 64 + WTILES * KT * 1024);
     dim3 grid((NB + WTILES - 1) / WTILES, (M + TT - 1) / TT, splits);
@@ -755,7 +753,7 @@ static int launch_tiled(const void* X, long ldx, const void* Wp, void* Y, long l
         raised = true;
     }
     gemm_tiled_kernel<WT, KT, NS, EPI, TC, NWV, TT, TURNS><<<grid, NWV * 64, lds, stream>>>((const bf16*)X, ldx, (const uint4*)Wp, (TC*)Y, ldy,
-                                                                      M, N, K, KB, NB, part_stride);
+                                                                      M, N, K, KB, NB, NBS > 0 ? NBS : NB, part_stride);
     return 0;
 }
 
@@ -823,10 +821,11 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
         if (rows_main > 0) {
             const int nb_main = (int)rows_main * 16;
             const int n_main = EPI == 0 ? nb_main * 16 : nb_main * 8;
-            int rc = launch_tiled<4, 1, 4, EPI, TC, 8, 256, true>(X, ldx, Wp, Y, ldy, M, n_main, K, KB, nb_main, stream);
+            int rc = launch_tiled<4, 1, 4, EPI, TC, 8, 256, true>(X, ldx, Wp, Y, ldy, M, n_main, K, KB, nb_main, stream, 1, 0, NB);
             if (rc != 0) return rc;
-            return launch_tiled<2, 2, 3, EPI, TC, 8, 256, false>(X, ldx, (const uint4*)Wp + (size_t)nb_main * KB * 64, (TC*)Y + n_main,
-                                                             ldy, M, N - n_main, K, KB, NB - nb_main, stream);
+            return launch_tiled<2, 2, 3, EPI, TC, 8, 256, false>(X, ldx, (const uint4*)Wp + w_tile(nb_main, 0, NB, KB) * 64,
+                                                                 (TC*)Y + n_main, ldy, M, N - n_main, K, KB, NB - nb_main, stream,
+                                                                 1, 0, NB);
         }
     }
     switch (pick) {

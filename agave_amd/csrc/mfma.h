@@ -6,9 +6,9 @@
 //   D[i][j] is held by lane j + 16*(i/4) as element i%4   (4 floats per lane)
 //
 // Packed weights ("P16"): W[N][K] (bf16, row-major [out, in]) is cut into tiles of 16 rows by
-// 32 columns; a tile is stored as the 64 lanes' A operands one after another (1 KB), tiles of
-// one row block follow each other along K:
-//   packed[((nb * KB + kb) * 64 + lane) * 8 + e] = W[16*nb + lane%16][32*kb + 8*(lane/16) + e]
+// 32 columns; a tile is stored as the 64 lanes' A operands one after another (1 KB), the tiles
+// of one k-step (all row blocks) follow each other:
+//   packed[(w_tile(nb, kb) * 64 + lane) * 8 + e] = W[16*nb + lane%16][32*kb + 8*(lane/16) + e]
 // with NB = ceil(N/16), KB = ceil(K/32) and zeros outside the matrix.  A wave reads a tile with
 // one fully coalesced 16-byte load per lane, straight into the registers the MFMA wants.
 #pragma once
@@ -17,6 +17,14 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+// Place of tile (row block nb, k-step kb) in a packed matrix of NB row blocks and KB k-steps.
+// k-step by k-step: workgroups that each stream their own row blocks then read neighbouring
+// kilobytes at any moment, as a plain streaming read does, instead of NB regions far apart.
+__host__ __device__ __forceinline__ size_t w_tile(long nb, long kb, long NB, long KB) {
+    (void)KB;
+    return (size_t)(kb * NB + nb);
+}
 
 union frag16 {            // 16 bytes: one lane's share of an MFMA operand
     uint4 u;
