@@ -113,6 +113,12 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
     *reinterpret_cast<uint2*>(p) = u;
 }
 
+// Loads are written without a per-lane condition around them: under one the compiler splits a
+// 16-byte load into four, each in a branch of its own.  A lane past the row's end reads the
+// row's start instead; its values are left out of the sums and never stored.  Nothing that was
+// loaded is touched before everything has been asked for, so the loads travel together.
+__device__ __forceinline__ float sumsq(bool in, float4 v) { return in ? v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w : 0.f; }
+
 template <typename T, int VPT>
 __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
                                           long part_stride, const float* __restrict__ post_gain, float post_eps,
@@ -122,36 +128,57 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
     const int i = blockIdx.x;
     const int r = rows ? rows[i] : i;
     float* hr = h + (size_t)r * e;
-    float4 hv[VPT], bv[VPT], g1[VPT], g2[VPT];
+    const float4 z = float4{0.f, 0.f, 0.f, 0.f};
+    constexpr int PB = 4;                       // slices asked for at a time
+    float4 hv[VPT], bv[VPT], g1[VPT], g2[VPT], pv[PB][VPT];
+    int col[VPT];
+    bool in[VPT];
+    // a gain that is not there is read from the row itself and not used
+    const float* g1p = (branch && post_gain) ? post_gain : hr;
+    const float* g2p = out ? pre_gain : hr;
 #pragma unroll
     for (int v = 0; v < VPT; ++v) {
         const int c = (threadIdx.x + v * blockDim.x) * 4;
-        const bool in = c < e;
-        const float4 z = float4{0.f, 0.f, 0.f, 0.f};
-        hv[v] = in ? *reinterpret_cast<const float4*>(hr + c) : z;
-        if (n_parts == 0) {
-            bv[v] = (in && branch) ? load4(branch + (size_t)r * ldb + c) : z;
-        } else {
-            // the branch is the sum of 32-bit slices (a product that was shared out along its columns)
-            const float* parts = reinterpret_cast<const float*>(branch) + (size_t)r * ldb + c;
-            bv[v] = z;
-            for (int p = 0; p < n_parts && in; ++p) {
-                const float4 t = *reinterpret_cast<const float4*>(parts + (size_t)p * part_stride);
-                bv[v].x += t.x;
-                bv[v].y += t.y;
-                bv[v].z += t.z;
-                bv[v].w += t.w;
+        in[v] = c < e;
+        col[v] = in[v] ? c : 0;
+        g1[v] = *reinterpret_cast<const float4*>(g1p + col[v]);
+        g2[v] = *reinterpret_cast<const float4*>(g2p + col[v]);
+        hv[v] = *reinterpret_cast<const float4*>(hr + col[v]);
+        bv[v] = z;
+    }
+    if (branch && n_parts == 0) {
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) bv[v] = load4(branch + (size_t)r * ldb + col[v]);
+    } else if (branch) {
+        // the branch is the sum of 32-bit slices (a product that was shared out along its columns)
+        for (int p0 = 0; p0 < n_parts; p0 += PB) {
+#pragma unroll
+            for (int u = 0; u < PB; ++u) {
+                const int p = p0 + u < n_parts ? p0 + u : n_parts - 1;
+#pragma unroll
+                for (int v = 0; v < VPT; ++v)
+                    pv[u][v] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(branch) + (size_t)r * ldb +
+                                                                col[v] + (size_t)p * part_stride);
+            }
+#pragma unroll
+            for (int u = 0; u < PB; ++u) {
+                const bool live = p0 + u < n_parts;
+#pragma unroll
+                for (int v = 0; v < VPT; ++v) {
+                    bv[v].x += live ? pv[u][v].x : 0.f;
+                    bv[v].y += live ? pv[u][v].y : 0.f;
+                    bv[v].z += live ? pv[u][v].z : 0.f;
+                    bv[v].w += live ? pv[u][v].w : 0.f;
+                }
             }
         }
-        g1[v] = (in && branch && post_gain) ? *reinterpret_cast<const float4*>(post_gain + c) : z;
-        g2[v] = (in && out) ? *reinterpret_cast<const float4*>(pre_gain + c) : z;
     }
     if (branch) {
         float inv = 1.0f;
         if (post_gain) {
             float ss = 0.f;
 #pragma unroll
-            for (int v = 0; v < VPT; ++v) ss += bv[v].x * bv[v].x + bv[v].y * bv[v].y + bv[v].z * bv[v].z + bv[v].w * bv[v].w;
+            for (int v = 0; v < VPT; ++v) ss += sumsq(in[v], bv[v]);
             ss = block_sum(ss, red);
             inv = 1.0f / sqrtf(ss / (float)e + post_eps);
         }
@@ -168,23 +195,21 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
                 hv[v].z += bv[v].z;
                 hv[v].w += bv[v].w;
             }
-            const int c = (threadIdx.x + v * blockDim.x) * 4;
-            if (c < e) *reinterpret_cast<float4*>(hr + c) = hv[v];
+            if (in[v]) *reinterpret_cast<float4*>(hr + col[v]) = hv[v];
         }
     }
     if (out) {
         float ss = 0.f;
 #pragma unroll
-        for (int v = 0; v < VPT; ++v) ss += hv[v].x * hv[v].x + hv[v].y * hv[v].y + hv[v].z * hv[v].z + hv[v].w * hv[v].w;
+        for (int v = 0; v < VPT; ++v) ss += sumsq(in[v], hv[v]);
         ss = block_sum(ss, red);
         const float inv = 1.0f / sqrtf(ss / (float)e + pre_eps);
         T* o = out + (size_t)i * ldo;
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
-            const int c = (threadIdx.x + v * blockDim.x) * 4;
-            if (c < e)
-                store4(o + c, float4{hv[v].x * inv * g2[v].x, hv[v].y * inv * g2[v].y, hv[v].z * inv * g2[v].z,
-                                     hv[v].w * inv * g2[v].w});
+            if (in[v])
+                store4(o + col[v], float4{hv[v].x * inv * g2[v].x, hv[v].y * inv * g2[v].y, hv[v].z * inv * g2[v].z,
+                                          hv[v].w * inv * g2[v].w});
         }
     }
 }
