@@ -328,18 +328,23 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     // FUSED: the first rows of the q/k work are requested before anything else (wave w takes query
     // head w of the chunk; the wave after the last head takes the key and value rows, in case
     // this workgroup turns out to be the one that writes them)
-    QkRow row0;
-    bf16 vreg0[QK_ROPE_HD_MAX / 64];
+    constexpr int NV = HDT / 4;               // groups of 64 elements in a head
+    QkRow<bf16, NV> row0;
+    bf16 vreg0[NV];
     const bool row0_q = FUSED && wave < slots, row0_k = FUSED && wave == slots && f.k_raw != nullptr;
     if constexpr (FUSED) {
         constexpr int hd0 = HDT * 16;
+        // a wave without a row reads the token's first query head (and nothing uses it); no load
+        // stands under a condition, so all of them leave together
         const bf16* src0 = row0_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + wave) * hd0
-                                  : (row0_k ? f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd0 : a.q);
-        row0 = qk_row_load<bf16>(src0, row0_q ? f.q_gain : f.k_gain, f.inv_freq, f.rot_half, hd0, lane, row0_q || row0_k);
+                                  : (row0_k ? f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd0 : a.q + (size_t)t * a.ldq);
+        row0 = qk_row_load<bf16, NV>(src0, row0_q ? f.q_gain : f.k_gain, f.inv_freq, f.rot_half, hd0, lane);
 #pragma unroll
-        for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) {
-            const int d = lane + 64 * k;
-            vreg0[k] = (row0_k && d < hd0) ? f.v_raw[(size_t)t * f.ldv + (size_t)kvh * hd0 + d] : bf16{0};
+        for (int k = 0; k < NV; ++k) vreg0[k] = bf16{0};
+        if (row0_k) {
+            const bf16* vsrc0 = f.v_raw + (size_t)t * f.ldv + (size_t)kvh * hd0;
+#pragma unroll
+            for (int k = 0; k < NV; ++k) vreg0[k] = vsrc0[lane + 64 * k];
         }
     }
     const int b = a.seq_is_token ? t : a.tok_seq[t];
@@ -442,24 +447,28 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
         for (int job0 = 0; job0 < jobs; job0 += 4) {
             const int job = job0 + wave;
             const bool active = job < jobs, is_q = job < slots;
-            QkRow row;
-            bf16 vreg[QK_ROPE_HD_MAX / 64];
+            QkRow<bf16, NV> row;
+            bf16 vreg[NV];
             if (job0 == 0) {                       // requested at the kernel's start
                 row = row0;
 #pragma unroll
-                for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) vreg[k] = vreg0[k];
+                for (int k = 0; k < NV; ++k) vreg[k] = vreg0[k];
             } else {
-                const bf16* src = is_q ? a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + (active ? job : 0)) * hd
-                                       : f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd;
-                row = qk_row_load<bf16>(src, is_q ? f.q_gain : f.k_gain, f.inv_freq, f.rot_half, hd, lane, active);
+                // (a wave past the last job reads the chunk's first head; the key's job only exists with k_raw)
+                const bool k_job = active && !is_q;
+                const bf16* src = k_job ? f.k_raw + (size_t)t * f.ldk + (size_t)kvh * hd
+                                        : a.q + (size_t)t * a.ldq + (size_t)(kvh * G + chunk * 16 + (active ? job : 0)) * hd;
+                row = qk_row_load<bf16, NV>(src, is_q ? f.q_gain : f.k_gain, f.inv_freq, f.rot_half, hd, lane);
 #pragma unroll
-                for (int k = 0; k < QK_ROPE_HD_MAX / 64; ++k) {
-                    const int d = lane + 64 * k;
-                    vreg[k] = (active && !is_q && d < hd) ? f.v_raw[(size_t)t * f.ldv + (size_t)kvh * hd + d] : bf16{0};
+                for (int k = 0; k < NV; ++k) vreg[k] = bf16{0};
+                if (k_job) {
+                    const bf16* vsrc = f.v_raw + (size_t)t * f.ldv + (size_t)kvh * hd;
+#pragma unroll
+                    for (int k = 0; k < NV; ++k) vreg[k] = vsrc[lane + 64 * k];
                 }
             }
-            qk_row_finish(row, ybuf, (is_q ? f.q_gain : f.k_gain) != nullptr, is_q ? f.eps_q : f.eps_k, f.rot_half, pf,
-                          hd, lane, active);
+            qk_row_finish<bf16, NV>(row, ybuf, (is_q ? f.q_gain : f.k_gain) != nullptr, is_q ? f.eps_q : f.eps_k, f.rot_half,
+                                    pf, hd, lane, active);
             if (active && is_q) {
                 for (int d = lane; d < hd; d += 64) q_s[job * hd + d] = f32_to_bf16(ybuf[d]);
             } else if (active) {
@@ -474,7 +483,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
                 if (wpg >= 0) {
                     bf16* dk = (bf16*)(a.k_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)4 * KS * 64));
                     bf16* dv = (bf16*)(a.v_pages + ((size_t)wpg * a.nkv + kvh) * ((size_t)HDT * 2 * 64));
-                    store_kv_row_packed_regs<bf16>(dk, dv, ybuf, vreg, p % AGAVE_PAGE, hd, lane);
+                    store_kv_row_packed_regs<bf16, NV>(dk, dv, ybuf, vreg, p % AGAVE_PAGE, hd, lane);
                 }
             }
         }

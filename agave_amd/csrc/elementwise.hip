@@ -286,7 +286,10 @@ extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long
 // [page][kv head][hd][64 rows]; position p of sequence b lies in page
 // table[b][p/64 - base[b]], row p % 64.
 #define QK_HD_MAX 512
-template <typename T>
+// NV: groups of 64 elements a head has (1, 2, 4 or 8).  Everything a wave needs is asked for at
+// its start: its row with the gains and frequencies, the value row, the position and the
+// sequence; the page id follows as soon as those two are there and travels during the arithmetic.
+template <typename T, int NV>
 __global__ void qk_norm_rope_kv_kernel(const T* q, long ldq, const T* __restrict__ k, long ldk,
                                        const T* __restrict__ v, long ldv, T* q_out, long ldqo,
                                        const float* __restrict__ q_gain, const float* __restrict__ k_gain,
@@ -296,13 +299,13 @@ __global__ void qk_norm_rope_kv_kernel(const T* q, long ldq, const T* __restrict
                                        T* __restrict__ v_pages, const int* __restrict__ table, int width,
                                        const int* __restrict__ base, int n_pages, int N, int nh, int nkv, int hd,
                                        int packed) {
-    __shared__ float buf[4][QK_HD_MAX];
+    __shared__ float buf[4][NV * 64];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int heads = nh + nkv;
-    const long unit = (long)blockIdx.x * 4 + wave;
-    const bool active = unit < (long)N * heads;
-    const int t = active ? (int)(unit / heads) : 0;
-    const int hh = active ? (int)(unit % heads) : 0;
+    const int unit = blockIdx.x * 4 + wave;                 // (the host checks that the units fit 31 bits)
+    const bool active = unit < N * heads;
+    const int t = active ? unit / heads : 0;
+    const int hh = active ? unit % heads : 0;
     const bool is_q = hh < nh;
     const int head = is_q ? hh : hh - nh;
     const T* src = is_q ? q + (size_t)t * ldq + (size_t)head * hd : k + (size_t)t * ldk + (size_t)head * hd;
@@ -310,35 +313,75 @@ __global__ void qk_norm_rope_kv_kernel(const T* q, long ldq, const T* __restrict
     const float eps = is_q ? eps_q : eps_k;
     float* y = buf[wave];
 
-    const int p = active ? tok_pos[t] : 0;
-    qk_norm_rope_wave<T>(src, y, gain, eps, inv_freq, rot_half, (float)p * pos_scale, hd, lane, active);
+    const QkRow<T, NV> row = qk_row_load<T, NV>(src, gain, inv_freq, rot_half, hd, lane);
+    const int p = tok_pos[t];
+    T vreg[NV];
+    int b = 0;
+    if (!is_q) {                       // a key's wave also takes the value row, and looks its page up
+        const T* sv = v + (size_t)t * ldv + (size_t)head * hd;
+#pragma unroll
+        for (int kk = 0; kk < NV; ++kk) {
+            const int d = lane + 64 * kk;
+            vreg[kk] = sv[d < hd ? d : 0];
+        }
+        b = tok_seq[t];
+    }
+    int col = 0;
+    int pg = -1;                       // (kept as it was loaded: widening it would wait for the load here)
+    const int row_in_page = p % AGAVE_PAGE;
+    if (!is_q) {
+        col = p / AGAVE_PAGE - base[b];
+        if (col >= 0 && col < width) pg = table[(size_t)b * width + col];
+    }
+    qk_row_finish<T, NV>(row, y, gain != nullptr, eps, rot_half, (float)p * pos_scale, hd, lane, active);
     if (!active) return;
     if (is_q) {
         T* dst = q_out + (size_t)t * ldqo + (size_t)head * hd;
-        for (int d = lane; d < hd; d += 64) st(dst + d, y[d]);
+#pragma unroll
+        for (int kk = 0; kk < NV; ++kk) {
+            const int d = lane + 64 * kk;
+            if (d < hd) st(dst + d, y[d]);
+        }
         return;
     }
-    const int b = tok_seq[t];
-    const int col = p / AGAVE_PAGE - base[b];
-    const int row = p % AGAVE_PAGE;
-    long pg = -1;
-    if (col >= 0 && col < width) pg = table[(size_t)b * width + col];
     if (pg < 0 || pg >= n_pages) return;   // a table the host built wrongly: write nothing
-    const T* sv = v + (size_t)t * ldv + (size_t)head * hd;
     if (!packed) {
-        T* dk = k_pages + (((size_t)pg * nkv + head) * AGAVE_PAGE + row) * hd;
-        T* dv = v_pages + ((size_t)pg * nkv + head) * hd * AGAVE_PAGE + row;
-        for (int d = lane; d < hd; d += 64) {
-            st(dk + d, y[d]);
-            dv[(size_t)d * AGAVE_PAGE] = sv[d];
+        T* dk = k_pages + (((size_t)pg * nkv + head) * AGAVE_PAGE + row_in_page) * hd;
+        T* dv = v_pages + ((size_t)pg * nkv + head) * hd * AGAVE_PAGE + row_in_page;
+#pragma unroll
+        for (int kk = 0; kk < NV; ++kk) {
+            const int d = lane + 64 * kk;
+            if (d < hd) {
+                st(dk + d, y[d]);
+                dv[(size_t)d * AGAVE_PAGE] = vreg[kk];
+            }
         }
     } else {
         // matrix-core tile order (see attention_mfma.hip)
         const int ks_n = (hd + 31) >> 5;
         T* dk = k_pages + ((size_t)pg * nkv + head) * (size_t)(AGAVE_PAGE * ks_n * 32);
         T* dv = v_pages + ((size_t)pg * nkv + head) * (size_t)hd * AGAVE_PAGE;
-        store_kv_row_packed<T>(dk, dv, y, sv, row, hd, lane);
+        store_kv_row_packed_regs<T, NV>(dk, dv, y, vreg, row_in_page, hd, lane);
     }
+}
+
+template <typename T>
+static void launch_qk_norm_rope_kv(int blocks, hipStream_t stream, const void* q, long ldq, const void* k, long ldk,
+                                   const void* v, long ldv, void* q_out, long ldqo, const float* q_gain,
+                                   const float* k_gain, float eps_q, float eps_k, const float* inv_freq, int rot_half,
+                                   float pos_scale, const int* tok_seq, const int* tok_pos, void* k_pages, void* v_pages,
+                                   const int* table, int width, const int* base, int n_pages, int N, int nh, int nkv,
+                                   int hd, int packed) {
+#define QK_LAUNCH(NV_)                                                                                               \
+    qk_norm_rope_kv_kernel<T, NV_><<<blocks, 256, 0, stream>>>(                                                      \
+        (const T*)q, ldq, (const T*)k, ldk, (const T*)v, ldv, (T*)q_out, ldqo, q_gain, k_gain, eps_q, eps_k, inv_freq, \
+        rot_half, pos_scale, tok_seq, tok_pos, (T*)k_pages, (T*)v_pages, table, width, base, n_pages, N, nh, nkv, hd, \
+        packed)
+    if (hd <= 64) QK_LAUNCH(1);
+    else if (hd <= 128) QK_LAUNCH(2);
+    else if (hd <= 256) QK_LAUNCH(4);
+    else QK_LAUNCH(8);
+#undef QK_LAUNCH
 }
 
 extern "C" int agave_qk_norm_rope_kv(int dtype, const void* q, long ldq, const void* k, long ldk, const void* v,
@@ -359,17 +402,16 @@ extern "C" int agave_qk_norm_rope_kv(int dtype, const void* q, long ldq, const v
     AGAVE_CHECK(!packed || (dtype == AGAVE_BF16 && hd % 16 == 0), "qk_norm_rope_kv: packed pages need bfloat16 and head_dim %% 16 == 0");
     const long units = (long)N * (nh + nkv);
     if (units == 0) return 0;
+    AGAVE_CHECK(units < (1L << 31) - 4, "qk_norm_rope_kv: %ld (token, head) pairs exceed what one launch takes", units);
     const int blocks = (int)((units + 3) / 4);
     if (dtype == AGAVE_F32)
-        qk_norm_rope_kv_kernel<float><<<blocks, 256, 0, stream>>>(
-            (const float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv, (float*)q_out, ldqo, q_gain, k_gain,
-            eps_q, eps_k, inv_freq, rot_half, pos_scale, tok_seq, tok_pos, (float*)k_pages, (float*)v_pages, table,
-            width, base, n_pages, N, nh, nkv, hd, packed);
+        launch_qk_norm_rope_kv<float>(blocks, stream, q, ldq, k, ldk, v, ldv, q_out, ldqo, q_gain, k_gain, eps_q, eps_k,
+                                      inv_freq, rot_half, pos_scale, tok_seq, tok_pos, k_pages, v_pages, table, width,
+                                      base, n_pages, N, nh, nkv, hd, packed);
     else if (dtype == AGAVE_BF16)
-        qk_norm_rope_kv_kernel<bf16><<<blocks, 256, 0, stream>>>(
-            (const bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv, (bf16*)q_out, ldqo, q_gain, k_gain, eps_q,
-            eps_k, inv_freq, rot_half, pos_scale, tok_seq, tok_pos, (bf16*)k_pages, (bf16*)v_pages, table, width,
-            base, n_pages, N, nh, nkv, hd, packed);
+        launch_qk_norm_rope_kv<bf16>(blocks, stream, q, ldq, k, ldk, v, ldv, q_out, ldqo, q_gain, k_gain, eps_q, eps_k,
+                                     inv_freq, rot_half, pos_scale, tok_seq, tok_pos, k_pages, v_pages, table, width,
+                                     base, n_pages, N, nh, nkv, hd, packed);
     else
         AGAVE_CHECK(false, "qk_norm_rope_kv: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("qk_norm_rope_kv");
