@@ -75,14 +75,21 @@ __global__ void embed_scale_packed_kernel(const int* __restrict__ tokens, const 
     tok = tok < 0 ? 0 : (tok >= vocab ? vocab - 1 : tok);
     const int nb = tok >> 4, i = tok & 15;
     float* o = out + (size_t)t * e;
-    for (int piece = threadIdx.x; piece * 8 < e; piece += blockDim.x) {     // 8 columns per piece
+    // a thread per piece of 8 columns where the row allows it: the row then arrives in one round trip
+    for (int piece = threadIdx.x; piece * 8 < e; piece += blockDim.x) {
         const int kb = piece >> 2, g = piece & 3;
         frag16 f;
         f.u = P[w_tile(nb, kb, (vocab + 15) / 16, KB) * 64 + i + 16 * g];
+        const int k0 = piece * 8;
+        if (k0 + 8 <= e && e % 4 == 0 && ((uintptr_t)out & 15) == 0) {
+            *reinterpret_cast<float4*>(o + k0) = float4{bf16_to_f32(f.h[0]) * scale, bf16_to_f32(f.h[1]) * scale,
+                                                        bf16_to_f32(f.h[2]) * scale, bf16_to_f32(f.h[3]) * scale};
+            *reinterpret_cast<float4*>(o + k0 + 4) = float4{bf16_to_f32(f.h[4]) * scale, bf16_to_f32(f.h[5]) * scale,
+                                                            bf16_to_f32(f.h[6]) * scale, bf16_to_f32(f.h[7]) * scale};
+        } else {
 #pragma unroll
-        for (int x = 0; x < 8; ++x) {
-            const int k = piece * 8 + x;
-            if (k < e) o[k] = bf16_to_f32(f.h[x]) * scale;
+            for (int x = 0; x < 8; ++x)
+                if (k0 + x < e) o[k0 + x] = bf16_to_f32(f.h[x]) * scale;
         }
     }
 }
@@ -91,7 +98,9 @@ extern "C" int agave_embed_scale_packed(const int* tokens, const void* P, float 
                                         int e, int vocab, hipStream_t stream) {
     AGAVE_CHECK(n_tokens >= 0 && e > 0 && vocab > 0, "embed_scale_packed: bad sizes");
     if (n_tokens == 0) return 0;
-    embed_scale_packed_kernel<<<n_tokens, 64, 0, stream>>>(tokens, (const uint4*)P, scale, out, e, vocab, (e + 31) / 32);
+    const int pieces = (e + 7) / 8;
+    const int threads = pieces >= 1024 ? 1024 : 64 * ((pieces + 63) / 64);
+    embed_scale_packed_kernel<<<n_tokens, threads, 0, stream>>>(tokens, (const uint4*)P, scale, out, e, vocab, (e + 31) / 32);
     AGAVE_LAUNCH_CHECK("embed_scale_packed");
     return 0;
 }

@@ -1,6 +1,7 @@
 // Sampling over 32-bit logits for gfx950: argmax, temperature / top-k / top-p draws, and the
-// repeat penalty.  One workgroup of 1024 threads per row; every sum is taken in a fixed
-// order, so a row's result depends only on the row and its parameters.
+// repeat penalty.  Small vocabularies: one workgroup of 1024 threads per row; large ones: a row
+// is shared among workgroups (see below).  Every sum is taken in a fixed order, so a row's
+// result depends only on the row and its parameters.
 //
 // Reference: src/ops/math.zig:32-50 (argmax, first index on ties), :186-197 (repeat penalty),
 // :209-372 (sampleToken): logits * 1/T; top-k keeps values >= the k-th largest (k capped at
@@ -61,11 +62,24 @@ __device__ void block_argmax(const float* __restrict__ x, int n, float mult, flo
                              int* out_i) {
     float best = -INFINITY;
     int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) {
-        const float v = x[i] * mult;
-        if (idx == 0x7fffffff || v > best) {      // a thread meets its indices in rising order
-            best = v;
-            idx = i;
+    // eight loads a thread are asked for before the first is compared (a load and its comparison
+    // in turn would be a round trip to memory each); an index past the end reads the last element
+    constexpr int U = 8;
+    for (int i0 = threadIdx.x; i0 < n; i0 += blockDim.x * U) {
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * blockDim.x;
+            v[u] = x[i < n ? i : n - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * blockDim.x;
+            const float val = v[u] * mult;
+            if (i < n && (idx == 0x7fffffff || val > best)) {      // a thread meets its indices in rising order
+                best = val;
+                idx = i;
+            }
         }
     }
 #pragma unroll
@@ -95,31 +109,497 @@ __device__ void block_argmax(const float* __restrict__ x, int n, float mult, flo
     *out_i = idx;
 }
 
-// Greedy rows, first pass: the row is cut into ARGMAX_PARTS pieces, one workgroup each, which
-// leave (max, lowest index holding it); sample_kernel picks among them.
-#define ARGMAX_PARTS 64
-__global__ __launch_bounds__(256) void argmax_parts_kernel(const float* __restrict__ logits, long ld,
-                                                           const float* __restrict__ params,
-                                                           float* __restrict__ part_v, int* __restrict__ part_i, int V) {
+// ------------------------------------------------------------------ large vocabularies: a row shared among workgroups
+// One workgroup reads a row of a quarter of a million logits no faster than one compute unit
+// pulls data, and the draw needs several passes over the row.  So a row is cut into SP_PARTS
+// pieces, one workgroup each, in a handful of small kernels: the pieces' maxima; the pieces'
+// sums of weights (rows whose draw ranges over the whole row); for rows with top-k or top-p a
+// radix selection of the value of the (at most 1024) largest entries in three rounds of
+// histograms (11, 11 and 10 bits of the ordered key), and the collection of those entries; last,
+// one workgroup per row decides.  With a filter the kept entries are among the collected ones,
+// which are sorted by value (thresholds) and then by index (the draw).  Without one the piece that
+// holds u * sum is found from the pieces' sums and only that piece is read again.
+// Words of scratch per row:
+#define SP_PARTS 64
+#define SP_THREADS 256
+#define SP_OFF_MAX 0                          // float[64]: the pieces' maxima
+#define SP_OFF_IDX 64                         // int[64]: lowest index holding each
+#define SP_OFF_SUM 128                        // float[64]: the pieces' sums of weights
+#define SP_OFF_NCAND 192                      // uint: collected entries
+#define SP_OFF_H0 256                         // uint[2048]: histogram of key bits 31..21
+#define SP_OFF_H1 (SP_OFF_H0 + 2048)          // uint[2048]: bits 20..10 under the first digit
+#define SP_OFF_H2 (SP_OFF_H1 + 2048)          // uint[1024]: bits 9..0 under the first two
+#define SP_OFF_CV (SP_OFF_H2 + 1024)          // float[1024]: collected values (scaled logits)
+#define SP_OFF_CI (SP_OFF_CV + MAX_CAND)      // int[1024]: their indices
+#define SP_ROW_WORDS (SP_OFF_CI + MAX_CAND)
+#define SP_HIST_WORDS (SP_OFF_CV - SP_OFF_H0)
+static_assert(SP_HIST_WORDS % SP_PARTS == 0, "the pieces' workgroups clear equal shares of the histograms");
+
+extern "C" int agave_sample_scratch_words() { return SP_ROW_WORDS; }
+
+struct RowMode {
+    float inv_t, top_p, u;
+    int top_k, want;
+    bool greedy, use_k, use_p, filt, whole_sum;
+};
+__device__ __forceinline__ RowMode row_mode(const float* __restrict__ params, int b, int V) {
+    RowMode m;
+    const float t = params[b * 4 + 0];
+    m.top_k = (int)params[b * 4 + 1];
+    m.top_p = params[b * 4 + 2];
+    m.u = params[b * 4 + 3];
+    m.greedy = t == 0.f;
+    m.inv_t = m.greedy ? 1.0f : 1.0f / t;
+    m.use_k = m.top_k > 0 && m.top_k < V;
+    m.use_p = m.top_p < 1.0f && m.top_p > 0.0f;
+    m.filt = !m.greedy && (m.use_k || m.use_p);
+    m.want = m.use_k ? (m.top_k < MAX_CAND ? m.top_k : MAX_CAND) : MAX_CAND;   // entries to collect
+    m.whole_sum = !m.greedy && !m.use_k;         // the sum of weights ranges over the whole row
+    return m;
+}
+__device__ __forceinline__ void part_range(int V, int part, int* lo, int* n) {
+    const int per = (V + SP_PARTS - 1) / SP_PARTS;
+    *lo = part * per;
+    int k = V - *lo;
+    *n = k > per ? per : (k > 0 ? k : 0);
+}
+// the row's maximum from the pieces' (every wave computes it for itself)
+__device__ __forceinline__ float sp_row_max(const float* __restrict__ rowf) {
+    return wave_max(rowf[SP_OFF_MAX + (threadIdx.x & 63)]);
+}
+
+// The pieces' maxima, for every row; also clears what the later kernels add to.
+__global__ __launch_bounds__(SP_THREADS) void sp_max_kernel(const float* __restrict__ logits, long ld,
+                                                            float* __restrict__ scratch, int V, int clear) {
     __shared__ float red_v[16];
     __shared__ int red_i[16];
     const int b = blockIdx.y, part = blockIdx.x;
-    if (params[b * 4] != 0.f) return;                       // only rows that take the argmax
-    const int per = (V + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
-    const int lo = part * per;
-    int n = V - lo;
-    if (n > per) n = per;
+    float* rowf = scratch + (size_t)b * SP_ROW_WORDS;
+    if (clear) {
+        constexpr int SHARE = SP_HIST_WORDS / SP_PARTS;
+        for (int i = threadIdx.x; i < SHARE; i += blockDim.x) reinterpret_cast<uint32_t*>(rowf)[SP_OFF_H0 + part * SHARE + i] = 0;
+        if (part == 0 && threadIdx.x == 0) reinterpret_cast<uint32_t*>(rowf)[SP_OFF_NCAND] = 0;
+    }
+    int lo, n;
+    part_range(V, part, &lo, &n);
     float mx = -INFINITY;
-    int idx = 0;
+    int idx = 0x7fffffff;
     if (n > 0) {
         block_argmax(logits + (size_t)b * ld + lo, n, 1.0f, red_v, red_i, &mx, &idx);
         idx += lo;
-    } else {
-        idx = 0x7fffffff;
     }
     if (threadIdx.x == 0) {
-        part_v[b * ARGMAX_PARTS + part] = mx;
-        part_i[b * ARGMAX_PARTS + part] = idx;
+        rowf[SP_OFF_MAX + part] = mx;
+        reinterpret_cast<int*>(rowf)[SP_OFF_IDX + part] = idx;
+    }
+}
+
+// Calls f(i, x[i] * mult) for the piece's elements, a thread's in rising order, with eight loads
+// asked for before the first is used.
+template <typename F>
+__device__ __forceinline__ void for_piece(const float* __restrict__ x, int n, float mult, F f) {
+    constexpr int U = 8;
+    for (int i0 = threadIdx.x; i0 < n; i0 += blockDim.x * U) {
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * blockDim.x;
+            v[u] = x[i < n ? i : n - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int i = i0 + u * blockDim.x;
+            if (i < n) f(i, v[u] * mult);
+        }
+    }
+}
+
+__device__ __forceinline__ float weight_of(float v, float mx) { return v == -INFINITY ? 0.f : expf(v - mx); }
+
+// The pieces' sums of exp(v - max), for rows whose sum ranges over the whole row.
+__global__ __launch_bounds__(SP_THREADS) void sp_sum_kernel(const float* __restrict__ logits, long ld,
+                                                            const float* __restrict__ params,
+                                                            float* __restrict__ scratch, int V) {
+    __shared__ float red[16];
+    const int b = blockIdx.y, part = blockIdx.x;
+    const RowMode m = row_mode(params, b, V);
+    if (!m.whole_sum) return;
+    float* rowf = scratch + (size_t)b * SP_ROW_WORDS;
+    const float mx = sp_row_max(rowf) * m.inv_t;
+    int lo, n;
+    part_range(V, part, &lo, &n);
+    float s = 0.f;
+    for_piece(logits + (size_t)b * ld + lo, n, m.inv_t, [&](int, float v) { s += weight_of(v, mx); });
+    s = block_sum(s, red);
+    if (threadIdx.x == 0) rowf[SP_OFF_SUM + part] = s;
+}
+
+// From a histogram of `bins` digits (a multiple of 256 * 4; all threads of a 256-thread
+// workgroup call): the digit that holds the krem-th largest entry, and how many of that digit's
+// entries are still wanted.  sh: 2 words, arr: 256 words of LDS.
+__device__ void sp_pick_digit(const uint32_t* __restrict__ hist, int bins, uint32_t krem, uint32_t* digit,
+                              uint32_t* krem_out, uint32_t* arr, uint32_t* sh) {
+    const int per = bins / SP_THREADS;                    // 8 or 4 digits a thread, consecutive
+    uint32_t c[8];
+    uint32_t local = 0;
+    {
+        const uint4 a = *reinterpret_cast<const uint4*>(hist + threadIdx.x * per);
+        const uint4 d = per == 8 ? *reinterpret_cast<const uint4*>(hist + threadIdx.x * per + 4) : uint4{0, 0, 0, 0};
+        c[0] = a.x; c[1] = a.y; c[2] = a.z; c[3] = a.w; c[4] = d.x; c[5] = d.y; c[6] = d.z; c[7] = d.w;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) local += c[i];
+    if (threadIdx.x == 0) {
+        sh[0] = 0;
+        sh[1] = krem;
+    }
+    // entries in the digits above this thread's: the total less the running count up to this thread
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    uint32_t run = local;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t t = __shfl_up(run, o, 64);
+        if (lane >= o) run += t;
+    }
+    if (lane == 63) arr[w] = run;
+    __syncthreads();
+    uint32_t total = 0;
+    for (int i = 0; i < SP_THREADS / 64; ++i) {
+        if (i < w) run += arr[i];
+        total += arr[i];
+    }
+    const uint32_t above = total - run;
+    if (above < krem && krem <= above + local) {          // one thread's digits hold the krem-th largest
+        uint32_t cum = above;
+        for (int i = per - 1; i >= 0; --i) {
+            if (cum + c[i] >= krem) {
+                sh[0] = threadIdx.x * per + i;
+                sh[1] = krem - cum;
+                break;
+            }
+            cum += c[i];
+        }
+    }
+    __syncthreads();
+    *digit = sh[0];
+    *krem_out = sh[1];
+    __syncthreads();
+}
+
+// The prefix that earlier rounds of the selection fixed: key bits above `shift` (ROUND 1: the
+// first digit, ROUND 2: the first two, ROUND 3: all three, the threshold key itself).
+template <int ROUND>
+__device__ void sp_prefix(const uint32_t* __restrict__ row, uint32_t want, uint32_t* prefix, uint32_t* arr,
+                          uint32_t* sh) {
+    uint32_t krem = want, d;
+    *prefix = 0;
+    if (ROUND >= 1) {
+        sp_pick_digit(row + SP_OFF_H0, 2048, krem, &d, &krem, arr, sh);
+        *prefix = d << 21;
+    }
+    if (ROUND >= 2) {
+        sp_pick_digit(row + SP_OFF_H1, 2048, krem, &d, &krem, arr, sh);
+        *prefix |= d << 10;
+    }
+    if (ROUND >= 3) {
+        sp_pick_digit(row + SP_OFF_H2, 1024, krem, &d, &krem, arr, sh);
+        *prefix |= d;
+    }
+}
+
+// One round of the selection: the histogram of this round's digit over the entries whose key
+// agrees with the digits found so far.
+template <int ROUND>
+__global__ __launch_bounds__(SP_THREADS) void sp_hist_kernel(const float* __restrict__ logits, long ld,
+                                                             const float* __restrict__ params,
+                                                             float* __restrict__ scratch, int V) {
+    __shared__ uint32_t h[2048];
+    __shared__ uint32_t arr[SP_THREADS];
+    __shared__ uint32_t sh[2];
+    const int b = blockIdx.y, part = blockIdx.x;
+    const RowMode m = row_mode(params, b, V);
+    if (!m.filt) return;
+    uint32_t* row = reinterpret_cast<uint32_t*>(scratch + (size_t)b * SP_ROW_WORDS);
+    uint32_t prefix;
+    sp_prefix<ROUND>(row, (uint32_t)m.want, &prefix, arr, sh);
+    constexpr int BINS = ROUND == 2 ? 1024 : 2048;
+    constexpr int SHIFT = ROUND == 0 ? 21 : (ROUND == 1 ? 10 : 0);          // this round's digit
+    constexpr int ABOVE = ROUND == 0 ? 32 : (ROUND == 1 ? 21 : 10);         // bits from here up are fixed
+    for (int i = threadIdx.x; i < BINS; i += blockDim.x) h[i] = 0;
+    __syncthreads();
+    int lo, n;
+    part_range(V, part, &lo, &n);
+    for_piece(logits + (size_t)b * ld + lo, n, m.inv_t, [&](int, float v) {
+        const uint32_t key = ordered_key(v);
+        if (ROUND == 0 || (key >> (ABOVE & 31)) == (prefix >> (ABOVE & 31))) atomicAdd(&h[(key >> SHIFT) & (BINS - 1)], 1u);
+    });
+    __syncthreads();
+    constexpr int OFF = ROUND == 0 ? SP_OFF_H0 : (ROUND == 1 ? SP_OFF_H1 : SP_OFF_H2);
+    for (int i = threadIdx.x; i < BINS; i += blockDim.x)
+        if (h[i]) atomicAdd(&row[OFF + i], h[i]);
+}
+
+// The entries at or above the threshold key (the want-th largest value and its ties), in any
+// order; at most MAX_CAND are kept.
+__global__ __launch_bounds__(SP_THREADS) void sp_collect_kernel(const float* __restrict__ logits, long ld,
+                                                                const float* __restrict__ params,
+                                                                float* __restrict__ scratch, int V) {
+    __shared__ uint32_t arr[SP_THREADS];
+    __shared__ uint32_t sh[2];
+    const int b = blockIdx.y, part = blockIdx.x;
+    const RowMode m = row_mode(params, b, V);
+    if (!m.filt) return;
+    float* rowf = scratch + (size_t)b * SP_ROW_WORDS;
+    uint32_t* row = reinterpret_cast<uint32_t*>(rowf);
+    uint32_t thr;
+    sp_prefix<3>(row, (uint32_t)m.want, &thr, arr, sh);
+    int lo, n;
+    part_range(V, part, &lo, &n);
+    for_piece(logits + (size_t)b * ld + lo, n, m.inv_t, [&](int i, float v) {
+        if (ordered_key(v) >= thr) {
+            const uint32_t at = atomicAdd(&row[SP_OFF_NCAND], 1u);
+            if (at < MAX_CAND) {
+                rowf[SP_OFF_CV + at] = v;
+                reinterpret_cast<int*>(rowf)[SP_OFF_CI + at] = lo + i;
+            }
+        }
+    });
+}
+
+// Running sums over the workgroup's threads in thread order: the sum up to and including this
+// thread's value is returned, the sum before it goes to *excl (a thread's *excl is bit for bit
+// its predecessor's result, so the threads' intervals tile [0, total) exactly); wtot: 16 words of LDS.
+__device__ float block_running_sum(float v, float* wtot, float* excl, float* total) {
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    float s = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float t = __shfl_up(s, o, 64);
+        if (lane >= o) s += t;
+    }
+    float ex = __shfl_up(s, 1, 64);
+    if (lane == 0) ex = 0.f;
+    __syncthreads();
+    if (lane == 63) wtot[w] = s;
+    __syncthreads();
+    float before = 0.f, tot = 0.f;
+    for (int i = 0; i < nw; ++i) {
+        if (i == w) before = tot;
+        tot += wtot[i];
+    }
+    *total = tot;
+    *excl = lane == 0 ? before : before + ex;
+    return before + s;
+}
+
+// The pieces' sums: their total (in a fixed order), the piece that holds `target` with what
+// remains of it inside that piece, and the last piece with any weight.  Every wave computes it.
+__device__ __forceinline__ float sp_parts_total(const float* __restrict__ rowf) {
+    return wave_sum(rowf[SP_OFF_SUM + (threadIdx.x & 63)]);
+}
+
+// Bitonic sort of the first `span` (a power of two, at most 1024) (key, payload) pairs in LDS;
+// all threads of the workgroup call; before(a, pa, c, pc): (a, pa) goes first.
+template <typename K, typename P, typename F>
+__device__ void sort_pairs(K* key, P* pay, int span, F before) {
+    for (int size = 2; size <= span; size <<= 1)
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            const int i = threadIdx.x, j = i ^ stride;
+            if (j > i && j < span) {
+                const bool up = (i & size) == 0;
+                const K a = key[i], c = key[j];
+                const P pa = pay[i], pc = pay[j];
+                const bool wrong = up ? before(c, pc, a, pa) : before(a, pa, c, pc);
+                if (wrong) {
+                    key[i] = c;
+                    key[j] = a;
+                    pay[i] = pc;
+                    pay[j] = pa;
+                }
+            }
+            __syncthreads();
+        }
+}
+
+// One workgroup of 1024 threads per row decides.
+__global__ __launch_bounds__(SAMPLE_THREADS) void sp_final_kernel(const float* __restrict__ logits, long ld,
+                                                                  const float* __restrict__ params,
+                                                                  int* __restrict__ out, int V,
+                                                                  float* __restrict__ scratch) {
+    __shared__ float cv[MAX_CAND];
+    __shared__ int ci[MAX_CAND];
+    __shared__ float ce[MAX_CAND];
+    __shared__ float wtot[16];
+    __shared__ float chunk[4 * SAMPLE_THREADS];
+    __shared__ float sh_f[2];
+    __shared__ int sh_i[2];
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const RowMode m = row_mode(params, b, V);
+    float* rowf = scratch + (size_t)b * SP_ROW_WORDS;
+    if (m.greedy) {                                           // the pieces' winners; ties go to the lowest index
+        if (tid < 64) {
+            float v = rowf[SP_OFF_MAX + tid];
+            int i = reinterpret_cast<const int*>(rowf)[SP_OFF_IDX + tid];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ov = __shfl_xor(v, o, 64);
+                const int oi = __shfl_xor(i, o, 64);
+                if (ov > v || (ov == v && oi < i)) {
+                    v = ov;
+                    i = oi;
+                }
+            }
+            if (tid == 0) out[b] = i;
+        }
+        return;
+    }
+    const float mx = sp_row_max(rowf) * m.inv_t;
+    bool whole_row = !m.filt;
+    if (m.filt) {
+        uint32_t n = reinterpret_cast<const uint32_t*>(rowf)[SP_OFF_NCAND];
+        if (n > MAX_CAND) n = MAX_CAND;
+        // by falling value (ties: rising index), for the thresholds
+        cv[tid] = tid < (int)n ? rowf[SP_OFF_CV + tid] : -INFINITY;
+        ci[tid] = tid < (int)n ? reinterpret_cast<const int*>(rowf)[SP_OFF_CI + tid] : 0x7fffffff;
+        int span = 2;                                  // the power of two that holds the entries
+        while (span < (int)n) span <<= 1;
+        __syncthreads();
+        sort_pairs(cv, ci, span, [](float a, int ia, float c, int ic) { return a > c || (a == c && ia < ic); });
+        float kth = -INFINITY;
+        if (m.use_k && m.want <= (int)n) kth = cv[m.want - 1];
+        float e = (tid < (int)n && cv[tid] >= kth) ? weight_of(cv[tid], mx) : 0.f;
+        float sum, before;
+        const float run = block_running_sum(e, wtot, &before, &sum);    // in the order of falling value
+        if (!m.use_k) sum = sp_parts_total(rowf);                       // nothing dropped yet: the whole row's sum
+        if (m.use_p) {
+            // the smallest prefix of the sorted weights whose mass reaches top_p * sum; every weight
+            // at or above the last one taken stays.  Not reached within the collected entries: nothing is dropped.
+            const float goal = m.top_p * sum;
+            if (tid == 0) sh_f[0] = 0.f;
+            __syncthreads();
+            if (e > 0.f && run >= goal && before < goal) sh_f[0] = e;      // at most one thread
+            __syncthreads();
+            const float thr = sh_f[0];
+            if (thr == 0.f && !m.use_k) whole_row = true;
+            if (e < thr) e = 0.f;
+        }
+        if (!whole_row) {
+            // by rising index, for the draw: the first kept index whose running sum exceeds u * sum
+            ce[tid] = e;
+            __syncthreads();
+            sort_pairs(ci, ce, span, [](int ia, float, int ic, float) { return ia < ic; });
+            e = ce[tid];
+            float total;
+            const float r2 = block_running_sum(e, wtot, &before, &total);
+            const float target = m.u * total;
+            if (tid == 0) {
+                sh_i[0] = -1;
+                sh_i[1] = -1;
+            }
+            __syncthreads();
+            if (e > 0.f) {
+                if (target < r2 && target >= before) sh_i[0] = ci[tid];      // the intervals tile: one thread
+                atomicMax(&sh_i[1], ci[tid]);                                // rounding at the very end: the last kept index
+            }
+            __syncthreads();
+            if (tid == 0)
+                out[b] = sh_i[0] >= 0 ? sh_i[0] : (sh_i[1] >= 0 ? sh_i[1] : reinterpret_cast<const int*>(rowf)[SP_OFF_IDX]);
+            return;
+        }
+        __syncthreads();                               // (the staging memory is used again below)
+    }
+    // The draw over the whole row: the piece that holds u * sum, then that piece's elements.
+    {
+        if (tid < 64) {                          // a piece per lane
+            const float ps = rowf[SP_OFF_SUM + tid];
+            float incl = ps;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const float t = __shfl_up(incl, o, 64);
+                if (tid >= o) incl += t;
+            }
+            float excl = __shfl_up(incl, 1, 64);
+            if (tid == 0) excl = 0.f;
+            const float total = __shfl(incl, 63, 64);
+            const float target = m.u * total;
+            const unsigned long long holds = __ballot(ps > 0.f && target < incl && target >= excl);
+            const unsigned long long any = __ballot(ps > 0.f);
+            int part;
+            float rem;
+            if (holds) {
+                part = __ffsll((long long)holds) - 1;
+                rem = target - __shfl(excl, part, 64);
+            } else {                             // rounding at the very end: the last piece with any weight, all of it
+                part = any ? 63 - __clzll((long long)any) : 0;
+                rem = INFINITY;
+            }
+            if (tid == 0) {
+                sh_i[0] = part;
+                sh_f[0] = rem;
+            }
+        }
+        __syncthreads();
+        const int part = sh_i[0];
+        float rem = sh_f[0];
+        int lo, n;
+        part_range(V, part, &lo, &n);
+        const float* x = logits + (size_t)b * ld + lo;
+        if (tid == 0) sh_i[1] = -1;
+        int last_pos = -1;                       // (thread 0 keeps it) the last index of the piece with any weight
+        for (int c0 = 0; c0 < n; c0 += 4 * SAMPLE_THREADS) {
+            // 4096 elements at a time: loaded side by side, then four in a row per thread
+            float v[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int i = c0 + tid + k * SAMPLE_THREADS;
+                v[k] = x[i < n ? i : n - 1];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int i = c0 + tid + k * SAMPLE_THREADS;
+                chunk[tid + k * SAMPLE_THREADS] = i < n ? weight_of(v[k] * m.inv_t, mx) : 0.f;
+            }
+            __syncthreads();
+            float w4[4], s4 = 0.f;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                w4[k] = chunk[tid * 4 + k];
+                s4 += w4[k];
+            }
+            float total, before;
+            const float run = block_running_sum(s4, wtot, &before, &total);
+            if (s4 > 0.f && rem < run && rem >= before) {             // this thread's four hold the target
+                float c = before;
+                int pick = -1, last_k = -1;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    c += w4[k];
+                    if (w4[k] > 0.f) {
+                        last_k = k;
+                        if (pick < 0 && rem < c) pick = k;
+                    }
+                }
+                if (pick < 0) pick = last_k;     // (the four's own sum rounds differently: their last weight)
+                sh_i[1] = lo + c0 + tid * 4 + pick;
+            }
+            // the chunk's last index with any weight, should nothing hold the target
+            {
+                int mine = -1;
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (w4[k] > 0.f) mine = c0 + tid * 4 + k;
+                __syncthreads();
+                if (tid == 0) sh_i[0] = -1;
+                __syncthreads();
+                if (mine >= 0) atomicMax(&sh_i[0], mine);
+                __syncthreads();
+                if (sh_i[0] >= 0) last_pos = sh_i[0];
+            }
+            if (sh_i[1] >= 0) break;             // (uniform: read after a barrier)
+            rem -= total;
+        }
+        if (tid == 0) out[b] = sh_i[1] >= 0 ? sh_i[1] : (last_pos >= 0 ? lo + last_pos : V - 1);
     }
 }
 
@@ -127,9 +607,7 @@ __global__ __launch_bounds__(256) void argmax_parts_kernel(const float* __restri
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits, long ld,
                                                                 float* __restrict__ work, long ldw,
                                                                 const float* __restrict__ params,
-                                                                int* __restrict__ out, int V,
-                                                                const float* __restrict__ part_v,
-                                                                const int* __restrict__ part_i) {
+                                                                int* __restrict__ out, int V) {
     __shared__ float red[16];
     __shared__ float red_v[16];
     __shared__ int red_i[16];
@@ -152,23 +630,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     float mx;
     int amax;
     if (temperature == 0.f) {
-        if (part_v) {                                         // the pieces' winners; ties go to the lowest index
-            if (tid < 64) {
-                float v = part_v[b * ARGMAX_PARTS + tid];
-                int i = part_i[b * ARGMAX_PARTS + tid];
-#pragma unroll
-                for (int o = 32; o > 0; o >>= 1) {
-                    const float ov = __shfl_xor(v, o, 64);
-                    const int oi = __shfl_xor(i, o, 64);
-                    if (ov > v || (ov == v && oi < i)) {
-                        v = ov;
-                        i = oi;
-                    }
-                }
-                if (tid == 0) out[b] = i;
-            }
-            return;
-        }
         block_argmax(x, V, 1.0f, red_v, red_i, &mx, &amax);
         if (tid == 0) out[b] = amax;
         return;
@@ -289,22 +750,37 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
     if (tid == 0) out[b] = sh_result;
 }
 
-// scratch: B * 64 floats followed by B * 64 ints for the greedy rows' first pass, or null.
+// scratch: agave_sample_scratch_words() words per row, or null.  With it, rows of a large
+// vocabulary are shared among workgroups.  kinds says what the rows need, so that launches
+// nothing needs are left out: bit 0: some row draws with a temperature; bit 1: some row has
+// top-k or top-p.  (A row decides for itself from params; a set bit that no row needs costs a
+// launch, a missing one gives a wrong draw.)
 extern "C" int agave_sample(const float* logits, long ld, float* work, long ldw, const float* params, int* out,
-                            int B, int V, float* scratch, hipStream_t stream) {
+                            int B, int V, float* scratch, int kinds, hipStream_t stream) {
     AGAVE_CHECK(B >= 0 && V > 0, "sample: bad sizes B=%d V=%d", B, V);
     AGAVE_CHECK(ld >= V && ldw >= V, "sample: a row stride is below the vocabulary");
     AGAVE_CHECK(logits && work && params && out, "sample: null buffer");
     if (B == 0) return 0;
-    float* part_v = nullptr;
-    int* part_i = nullptr;
     if (scratch && V >= 4096 && B <= 65535) {
-        part_v = scratch;
-        part_i = reinterpret_cast<int*>(scratch + (size_t)B * ARGMAX_PARTS);
-        argmax_parts_kernel<<<dim3(ARGMAX_PARTS, B), 256, 0, stream>>>(logits, ld, params, part_v, part_i, V);
-        AGAVE_LAUNCH_CHECK("argmax_parts");
+        const dim3 grid(SP_PARTS, B);
+        sp_max_kernel<<<grid, SP_THREADS, 0, stream>>>(logits, ld, scratch, V, (kinds & 2) ? 1 : 0);
+        AGAVE_LAUNCH_CHECK("sample (maxima)");
+        if (kinds & 1) {
+            sp_sum_kernel<<<grid, SP_THREADS, 0, stream>>>(logits, ld, params, scratch, V);
+            AGAVE_LAUNCH_CHECK("sample (sums)");
+        }
+        if (kinds & 2) {
+            sp_hist_kernel<0><<<grid, SP_THREADS, 0, stream>>>(logits, ld, params, scratch, V);
+            sp_hist_kernel<1><<<grid, SP_THREADS, 0, stream>>>(logits, ld, params, scratch, V);
+            sp_hist_kernel<2><<<grid, SP_THREADS, 0, stream>>>(logits, ld, params, scratch, V);
+            sp_collect_kernel<<<grid, SP_THREADS, 0, stream>>>(logits, ld, params, scratch, V);
+            AGAVE_LAUNCH_CHECK("sample (selection)");
+        }
+        sp_final_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, ld, params, out, V, scratch);
+        AGAVE_LAUNCH_CHECK("sample (draw)");
+        return 0;
     }
-    sample_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, ld, work, ldw, params, out, V, part_v, part_i);
+    sample_kernel<<<B, SAMPLE_THREADS, 0, stream>>>(logits, ld, work, ldw, params, out, V);
     AGAVE_LAUNCH_CHECK("sample");
     return 0;
 }

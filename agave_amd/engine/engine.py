@@ -236,8 +236,9 @@ class Engine:
             sample_ops.repeat_penalty(logits, ids, cu_t, pen)
         work = self.workspace.get("sample_work", b, self.spec.vocab_size, torch.float32)
         out = self._sampled_all()[:b]
-        scratch = self.workspace.get("sample_scratch", b, 128, torch.float32).view(-1)
-        sample_ops.sample(logits, work, step.floats_dev.view(b, 4), out, scratch)
+        scratch = self.workspace.get("sample_scratch", b, sample_ops.scratch_words(), torch.float32).view(-1)
+        sample_ops.sample(logits, work, step.floats_dev.view(b, 4), out, scratch,
+                          kinds=sample_ops.kinds_of(rows, self.spec.vocab_size))
         self._result_turn = 1 - getattr(self, "_result_turn", 0)
         hosts = getattr(self, "_result_hosts", None)
         if hosts is None:

@@ -1,13 +1,15 @@
 """Faces of the sampling kernels."""
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import kernels, library
 from .kernels import _I, _L, _P
 
 kernels.register_signatures("sampling", {
-    "agave_sample": [_P, _L, _P, _L, _P, _P, _I, _I, _P, _P],
+    "agave_sample": [_P, _L, _P, _L, _P, _P, _I, _I, _P, _I, _P],
     "agave_repeat_penalty": [_P, _L, _P, _P, _P, _I, _I, _P],
     "agave_gather_tokens": [_P, _P, _P, _I, _I, _P],
 })
@@ -21,12 +23,37 @@ def _logits(logits: torch.Tensor) -> int:
     return logits.stride(0)
 
 
+KIND_TEMPERATURE = 1     # some row draws with a temperature
+KIND_FILTER = 2          # some row has top-k or top-p
+KIND_ALL = 3
+
+
+def scratch_words() -> int:
+    """float32 words of scratch per row that let rows of a large vocabulary be shared among workgroups."""
+    lib = kernels.lib("sampling")
+    lib.agave_sample_scratch_words.restype = ctypes.c_int
+    lib.agave_sample_scratch_words.argtypes = []
+    return int(lib.agave_sample_scratch_words())
+
+
+def kinds_of(rows, vocab: int) -> int:
+    """What a batch's rows (objects with temperature, top_k, top_p) need of the sampler."""
+    kinds = 0
+    for r in rows:
+        if r.temperature > 0:
+            kinds |= KIND_TEMPERATURE
+            if 0 < r.top_k < vocab or 0.0 < r.top_p < 1.0:
+                kinds |= KIND_FILTER
+    return kinds
+
+
 def sample(logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: torch.Tensor,
-           scratch: torch.Tensor = None) -> None:
+           scratch: torch.Tensor = None, kinds: int = KIND_ALL) -> None:
     """out[b] = a token drawn from row b.  ``params`` float32 [rows, 4] = temperature, top_k,
     top_p, u; temperature 0 takes the argmax (first index on ties).  ``work``: float32 scratch
-    of the logits' shape.  ``scratch`` (128 float32 per row) lets greedy rows of a large vocabulary be
-    searched by 64 workgroups each."""
+    of the logits' shape.  ``scratch`` (``scratch_words()`` float32 per row) lets rows of a large
+    vocabulary be shared among 64 workgroups each; ``kinds`` then says what the rows need
+    (``kinds_of``), so that kernels no row needs are not launched."""
     ld = _logits(logits)
     b, v = logits.shape
     if work.dtype != torch.float32 or work.shape != logits.shape or work.stride(1) != 1 or not work.is_cuda:
@@ -35,11 +62,15 @@ def sample(logits: torch.Tensor, work: torch.Tensor, params: torch.Tensor, out: 
         raise TypeError(f"sample: params must be contiguous float32 [{b}, 4] on the GPU")
     if out.dtype != torch.int32 or out.numel() != b or not out.is_contiguous() or not out.is_cuda:
         raise TypeError(f"sample: out must be {b} contiguous int32 on the GPU")
-    if scratch is not None and (scratch.dtype != torch.float32 or scratch.numel() < 128 * b or not scratch.is_cuda
-                                or not scratch.is_contiguous()):
-        raise TypeError(f"sample: scratch must be {128 * b} contiguous float32 on the GPU")
+    if scratch is not None:
+        need = scratch_words() * b
+        if (scratch.dtype != torch.float32 or scratch.numel() < need or not scratch.is_cuda
+                or not scratch.is_contiguous() or scratch.data_ptr() % 16 != 0):
+            raise TypeError(f"sample: scratch must be {need} contiguous float32 on the GPU, 16-byte aligned")
+    if kinds not in (0, 1, 2, 3):
+        raise ValueError("sample: kinds is a mask of KIND_TEMPERATURE and KIND_FILTER")
     library.call(kernels.lib("sampling"), "agave_sample", logits.data_ptr(), ld, work.data_ptr(), work.stride(0),
-                 params.data_ptr(), out.data_ptr(), b, v, kernels.ptr(scratch), kernels.stream())
+                 params.data_ptr(), out.data_ptr(), b, v, kernels.ptr(scratch), int(kinds), kernels.stream())
 
 
 def repeat_penalty(logits: torch.Tensor, ids: torch.Tensor, cu: torch.Tensor, penalty: torch.Tensor) -> None:
