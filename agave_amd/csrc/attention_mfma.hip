@@ -325,6 +325,9 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
     const int slots = (G - chunk * 16 < 16) ? G - chunk * 16 : 16;
     const int t = blockIdx.z, split = blockIdx.x;
+    // the token's sequence and position are asked for first: the page ids wait for them
+    const int b = a.seq_is_token ? t : a.tok_seq[t];
+    const int p = a.tok_pos[t];
     // FUSED: the first rows of the q/k work are requested before anything else (wave w takes query
     // head w of the chunk; the wave after the last head takes the key and value rows, in case
     // this workgroup turns out to be the one that writes them)
@@ -347,11 +350,9 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
             for (int k = 0; k < NV; ++k) vreg0[k] = vsrc0[lane + 64 * k];
         }
     }
-    const int b = a.seq_is_token ? t : a.tok_seq[t];
     const int col0 = split * a.pages_per_split + wave;
-    long pg0 = -1;
+    int pg0 = -1;                             // (kept as loaded: widening it here would wait for the load)
     if (a.table_from_reach && col0 < a.width) pg0 = a.table[(size_t)b * a.width + col0];
-    const int p = a.tok_pos[t];
     const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
     const int first = lo / AGAVE_PAGE, last = p / AGAVE_PAGE;
     const int page_lo = first + split * a.pages_per_split;
@@ -387,9 +388,9 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
         const int col = page_lo + wave + 4 * i - first;
         pg_pre[i] = (a.table_from_reach && i < n_my && col < a.width) ? a.table[(size_t)b * a.width + col] : -1;
     }
-    auto page_id = [&](int i) -> long {          // i-th page of this wave
+    auto page_id = [&](int i) -> int {           // i-th page of this wave (page ids fit 31 bits)
         const int pi = page_lo + wave + 4 * i;
-        long pg;
+        int pg;
         if (a.table_from_reach) {
             const int col = pi - first;
             if (i == 0) {
@@ -404,7 +405,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
             }
             if (pg >= a.n_pages) pg = -1;
         } else {
-            pg = page_of(a, b, pi);
+            pg = (int)page_of(a, b, pi);
         }
         return pg;
     };
@@ -424,7 +425,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
 
     // units: half pages, in order; the next unit's K and V are fetched while this one is used
     int cur_page = 0;
-    long pg = n_my > 0 ? page_id(0) : -1;
+    int pg = n_my > 0 ? page_id(0) : -1;
     bool have = n_my > 0 && pg >= 0;
     if (have) {
         kp = (const u32x4_t*)(a.k_pages + ((size_t)pg * a.nkv + kvh) * k_stride);
@@ -517,7 +518,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
         bool n_have = n_page < n_my;
         const u32x4_t* nvp = vp;
         if (n_have && half == 1) {
-            const long npg = page_id(n_page);
+            const int npg = page_id(n_page);
             if (npg < 0) {
                 n_have = false;
             } else {
