@@ -13,6 +13,8 @@ kernels.register_signatures("gemm_mfma", {
     "agave_embed_scale_packed": [_P, _P, _F, _P, _I, _I, _I, _P],
     "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _I, _P],
     "agave_gemm_skinny_slices": [_I, _I, _I],
+    "agave_gemm_tiled_slices": [_I, _I, _I],
+    "agave_gemm_tiled_in_slices": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
     "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P, _L, _P],
 })
 
@@ -67,6 +69,38 @@ def slices_for(m: int, n_out: int, k: int) -> int:
             fn = kernels.lib("gemm_mfma").agave_gemm_skinny_slices
             got = _slices[key] = int(fn(m, n_out, k))
     return got
+
+
+def tiled_slices_for(m: int, n_out: int, k: int) -> int:
+    """The same for a product of many tokens: more than one where the tiles would leave many
+    compute units idle and the columns are many."""
+    key = (m, n_out, k)
+    got = _slices.get(key)
+    if got is None:
+        got = 1
+        if m > SKINNY_MAX_M and m * n_out * 4 * 4 <= TILED_SLICES_MAX_BYTES:
+            got = int(kernels.lib("gemm_mfma").agave_gemm_tiled_slices(m, n_out, k))
+        _slices[key] = got
+    return got
+
+
+TILED_SLICES_MAX_BYTES = 512 << 20       # what the slices of one product may take
+
+
+def tiled_slices(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int) -> None:
+    """out[s] = the sums over the s-th run of columns of x[M, K] @ W^T for M > 64; out is float32
+    [tiled_slices_for(M, n_out, K), M, n_out] and its slices add up to the product."""
+    if not (x.is_cuda and packed.is_cuda and out.is_cuda):
+        raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
+    if not _x_ok(x):
+        raise ValueError("packed product: input must be 16-byte aligned bfloat16 rows with K and the row stride multiples of 8")
+    m, k = x.shape
+    if out.dtype != torch.float32 or out.dim() != 3 or out.shape[1:] != (m, n_out) or not out.is_contiguous():
+        raise ValueError(f"partial sums must be a contiguous float32 [slices, {m}, {n_out}] tensor")
+    if packed.numel() != ((n_out + 15) // 16) * ((k + 31) // 32) * 512:
+        raise ValueError("packed product: the packed weight does not fit these sizes")
+    library.call(kernels.lib("gemm_mfma"), "agave_gemm_tiled_in_slices", x.data_ptr(), x.stride(0), packed.data_ptr(),
+                 out.data_ptr(), m, n_out, k, out.shape[0], kernels.stream())
 
 
 def skinny_slices(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int) -> None:

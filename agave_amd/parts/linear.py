@@ -56,12 +56,13 @@ class Linear:
         n = x.shape[0]
         if slices_ok and out is None and self.packed is not None and not self.interleave_ff:
             from ..ops import gemm_mfma, library
-            slices = gemm_mfma.slices_for(n, self.out_features, self.in_features)
+            many = n > gemm_mfma.SKINNY_MAX_M
+            slices = (gemm_mfma.tiled_slices_for if many else gemm_mfma.slices_for)(n, self.out_features, self.in_features)
             if slices > 1 and gemm_mfma._x_ok(x):
                 out = self.env.workspace.get((tag or self.name) + "_slices", slices * n, self.out_features,
                                              torch.float32).view(slices, n, self.out_features)
                 library.profile.label = self.name
-                gemm_mfma.skinny_slices(x, self.packed, out, self.out_features)
+                (gemm_mfma.tiled_slices if many else gemm_mfma.skinny_slices)(x, self.packed, out, self.out_features)
                 library.profile.label = None
                 return out
         if out is None:

@@ -583,6 +583,30 @@ def test_gemm_tiled(G, m, n, k, out_dtype):
     assert float((out.cpu().double() - ref).abs().max()) <= tol
 
 
+@pytest.mark.parametrize("m,n,k", [(2048, 2560, 10240),     # 160 tiles of 128 x 256: three slices
+                                   (4096, 2560, 10240),     # 160 tiles of 256 x 256: three slices
+                                   (2000, 2552, 10248),     # the same tiles, ragged edges
+                                   (2048, 2560, 2048),      # few columns: one product
+                                   (300, 200, 4096)])       # small tiles: one product
+def test_gemm_tiled_in_slices(G, m, n, k):
+    """A product of many tokens whose tiles fill the compute units badly comes as 32-bit slices
+    that add up to it, for a reader that adds them."""
+    z = G.tiled_slices_for(m, n, k)
+    assert z == (3 if k >= 10240 and m >= 2000 else 1)
+    if z == 1:
+        return
+    g = torch.Generator().manual_seed(m + n + k)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    packed = G.pack_weight(w.to(DEV))
+    out = torch.full((z, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    G.tiled_slices(x.to(DEV), packed, out, n)
+    ref = x.to(DEV).double() @ w.to(DEV).double().T
+    got = out.double().sum(0)
+    assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max()) * math.sqrt(k / 64)
+    assert float(out[0].abs().max()) > 0 and float(out[z - 1].abs().max()) > 0
+
+
 @pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40), (1024, 5120, 1000), (2048, 10236, 64)])
 def test_gemm_tiled_geglu(G, m, ff, k):
     g = torch.Generator().manual_seed(ff + m)
