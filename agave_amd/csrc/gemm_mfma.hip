@@ -846,42 +846,42 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
 }
 
 // A product of many tokens whose reader adds 32-bit slices up (the residual kernel does): when
-// the tiles fill the 256 compute units' rounds badly (160 tiles of 128 x 256 for 2,048 tokens and
+// its 128 x 256 tiles fill the 256 compute units' rounds badly (160 tiles for 2,048 tokens and
 // 2,560 rows leave 96 of them idle for the whole product), each tile's columns are shared among
 // z workgroups, each of which leaves its sums in a slice of its own.  In units of one tile's
 // time the product then takes rounds(tiles * z) / z, and every slice beyond the first costs its
-// bytes, written here and read by whoever adds them: some 0.07 of a 128 x 256 tile's time at 160
-// tiles and 10,240 columns (measured), in proportion to the tiles and inversely to the columns.
-struct TiledCut { int pick, z; };
-static TiledCut cut_tiled_slices(int M, int N, int K) {
+// bytes, written here and read by whoever adds them: some 0.07 of a tile's time at 160 tiles and
+// 10,240 columns (measured: down at 2,048 tokens takes 114 us in three slices instead of 136, and
+// the kernel that adds them 8 us more), in proportion to the tiles and inversely to the columns.
+// Products that run in 256 x 256 tiles are left alone: sliced, they were slower (measured at
+// 4,096 and 8,192 tokens, by 4 %).
+static int cut_tiled_slices(int M, int N, int K) {
     const long NB = (N + 15) / 16;
     const long rows16 = (NB + 15) / 16, rows8 = (NB + 7) / 8;
     const long t256 = (M + 255) / 256;
-    const long wgs[2] = {rows16 * t256, rows8 * t256};
-    TiledCut cut = {-1, 1};
-    int pick = wgs[0] >= 160 ? 0 : (wgs[1] >= 160 ? 1 : -1);
-    if (pick < 0) return cut;                              // smaller tiles: the product shares its columns out itself
-    const long t = wgs[pick];
+    if (rows16 * t256 >= 160 || rows8 * t256 < 160) return 1;      // 256 x 256 tiles, or smaller ones than 128 x 256
+    const long t = rows8 * t256;
     auto rounds = [](long g) { return (double)((g + 255) / 256); };
-    const double slice_cost = 0.07 * (10240.0 / K) * ((double)t / 160.0) * (pick == 0 ? 0.25 : 1.0);
-    const int n_stage = pick == 0 ? (K + 31) / 32 : (K + 63) / 64;
+    const double slice_cost = 0.07 * (10240.0 / K) * ((double)t / 160.0);
+    const int n_stage = (K + 63) / 64;
     double best = rounds(t);
+    int z_best = 1;
     for (int z = 2; z <= 4; ++z) {
         if (n_stage / z < 16) break;
         const double cost = rounds(t * z) / z + (z - 1) * slice_cost;
         if (cost < 0.93 * best) {
             best = cost;
-            cut = {pick, z};
+            z_best = z;
         }
     }
-    return cut;
+    return z_best;
 }
 
 // How many 32-bit slices a product of M > 64 tokens is best computed in by a caller that can
 // add them up (1: as one product).
 extern "C" int agave_gemm_tiled_slices(int M, int N, int K) {
     if (M <= 64 || N <= 0 || K <= 0 || K % 8 != 0) return 1;
-    return cut_tiled_slices(M, N, K).z;
+    return cut_tiled_slices(M, N, K);
 }
 
 // Y: 32-bit [z][M][N], z = agave_gemm_tiled_slices(M, N, K) > 1; slice s gets the sums over the
@@ -892,13 +892,10 @@ extern "C" int agave_gemm_tiled_in_slices(const void* X, long ldx, const void* W
     AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
                 "gemm_tiled_in_slices: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
     AGAVE_CHECK(ldx >= K && ldx < (1L << 22), "gemm_tiled_in_slices: bad row stride %ld", ldx);
-    const TiledCut cut = cut_tiled_slices(M, N, K);
-    AGAVE_CHECK(z > 1 && z == cut.z, "gemm_tiled_in_slices: %d slices asked for, %d planned", z, cut.z);
+    const int planned = cut_tiled_slices(M, N, K);
+    AGAVE_CHECK(z > 1 && z == planned, "gemm_tiled_in_slices: %d slices asked for, %d planned", z, planned);
     const int KB = (K + 31) / 32, NB = (N + 15) / 16;
-    const long stride = (long)M * N;
-    int rc;
-    if (cut.pick == 0) rc = launch_tiled<4, 1, 4, 0, float, 8, 256, true>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, stride);
-    else rc = launch_tiled<2, 2, 3, 0, float, 8, 256, false>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, stride);
+    const int rc = launch_tiled<2, 2, 3, 0, float, 8, 256, false>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, (long)M * N);
     if (rc != 0) return rc;
     AGAVE_LAUNCH_CHECK("gemm_tiled_in_slices");
     return 0;
