@@ -676,6 +676,57 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
     }
 }
 
+// The same merge for many rows and few splits (a prompt whose blocks of positions were shared
+// among workgroups): a wave per (token, head), four elements a lane at a time, every load asked
+// for before the first is used.
+#define COMBINE_ROWS_MAX_SPLITS 4
+__global__ __launch_bounds__(256) void attn_combine_rows_kernel(const float* __restrict__ part_o,
+                                                                const float* __restrict__ part_ml,
+                                                                bf16* __restrict__ out, long ldo, int nh, int hd,
+                                                                int splits, long rows) {
+    const int lane = threadIdx.x & 63;
+    const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const long t = r / nh;
+    const int head = (int)(r % nh);
+    const size_t slot0 = (size_t)r * splits;
+    float ms[COMBINE_ROWS_MAX_SPLITS], ls[COMBINE_ROWS_MAX_SPLITS];
+#pragma unroll
+    for (int sp = 0; sp < COMBINE_ROWS_MAX_SPLITS; ++sp) {
+        const int s2 = sp < splits ? sp : splits - 1;
+        ms[sp] = part_ml[(slot0 + s2) * 2];
+        ls[sp] = part_ml[(slot0 + s2) * 2 + 1];
+    }
+    for (int d0 = lane * 4; d0 < hd; d0 += 256) {
+        float4 v[COMBINE_ROWS_MAX_SPLITS];
+#pragma unroll
+        for (int sp = 0; sp < COMBINE_ROWS_MAX_SPLITS; ++sp) {
+            const int s2 = sp < splits ? sp : splits - 1;
+            v[sp] = *reinterpret_cast<const float4*>(part_o + (slot0 + s2) * hd + d0);
+        }
+        float m = -INFINITY;
+#pragma unroll
+        for (int sp = 0; sp < COMBINE_ROWS_MAX_SPLITS; ++sp)
+            if (sp < splits) m = fmaxf(m, ms[sp]);
+        float l = 0.f;
+        float4 acc = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int sp = 0; sp < COMBINE_ROWS_MAX_SPLITS; ++sp) {
+            const float f = (sp < splits && ms[sp] != -INFINITY) ? __expf(ms[sp] - m) : 0.f;
+            l += ls[sp] * f;
+            acc.x += v[sp].x * f;
+            acc.y += v[sp].y * f;
+            acc.z += v[sp].z * f;
+            acc.w += v[sp].w * f;
+        }
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        uint2 u;
+        u.x = f32x2_to_bf16x2(acc.x * inv, acc.y * inv);
+        u.y = f32x2_to_bf16x2(acc.z * inv, acc.w * inv);
+        *reinterpret_cast<uint2*>(out + (size_t)t * ldo + (size_t)head * hd + d0) = u;
+    }
+}
+
 // ------------------------------------------------------------------ prefill: 64 positions x QT heads per workgroup
 // grid (block of positions, kv head * head chunks, sequence).  The four waves are hw heads
 // wide and 4/hw tiles of 16 positions deep; a wave takes QT heads of its tile (slot j of tile t
@@ -742,7 +793,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int 
         }
     };
 
-    fetch(page_first, 0);
+    if (page_first <= page_last) fetch(page_first, 0);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     for (int pi = page_first; pi <= page_last; ++pi) {
@@ -797,7 +848,11 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     const int b = blockIdx.z;
     const int t0 = a.cu[b], n_new = a.cu[b + 1] - t0;
     const int blk_len = (NWV / hw) * 16;                         // positions a workgroup covers
-    const int blk0 = blockIdx.x * blk_len;
+    // a.splits workgroups share a block of positions: each takes a run of the block's pages and
+    // leaves partial results, which attn_combine_kernel merges (a prompt of a few thousand tokens
+    // has too few blocks to fill the compute units otherwise)
+    const int split = blockIdx.x % a.splits;
+    const int blk0 = (blockIdx.x / a.splits) * blk_len;
     if (blk0 >= n_new) return;                                   // the whole workgroup leaves
     const int tile0 = blk0 + (wave / hw) * 16;                   // first step-token of this wave's tile
     const int gh = chunk * hw + wave % hw;                       // this wave's head within the group
@@ -830,7 +885,12 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     const int p_blk0 = a.tok_pos[t0 + blk0];
     const int blk_n = (n_new - blk0 < blk_len) ? n_new - blk0 : blk_len;
     const int lo_blk = a.window > 0 ? (p_blk0 - a.window + 1 > 0 ? p_blk0 - a.window + 1 : 0) : 0;
-    const int page_first = lo_blk / AGAVE_PAGE, page_last = (p_blk0 + blk_n - 1) / AGAVE_PAGE;
+    int page_first = lo_blk / AGAVE_PAGE, page_last = (p_blk0 + blk_n - 1) / AGAVE_PAGE;
+    if (a.splits > 1) {
+        const int per = (page_last - page_first + a.splits) / a.splits;
+        page_first += split * per;
+        if (page_last > page_first + per - 1) page_last = page_first + per - 1;     // (may leave no page at all)
+    }
 
     // The ids of the pages this workgroup goes through, looked up once: a lookup inside the loop
     // is two dependent loads from memory a page, and waiting for them also waits for the next
@@ -853,7 +913,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
         }
     };
 
-    fetch(page_first, 0);
+    if (page_first <= page_last) fetch(page_first, 0);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     for (int pi = page_first; pi <= page_last; ++pi) {
@@ -941,6 +1001,23 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     const int head = kvh * G + gh;
+    if (a.splits > 1) {
+        // sums as they stand, with the reference they are relative to (in natural logarithms, as the combine pass reads it)
+        if (g == 0 && col_ok) {
+            const size_t ps = ((size_t)(t0 + tile0 + j) * a.nh + head) * a.splits + split;
+            a.part_ml[ps * 2 + 0] = m_ref * 0.6931471805599453f;
+            a.part_ml[ps * 2 + 1] = l;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int row = 4 * g + e;
+            if (tile0 + row >= n_new) continue;
+            float* dst = a.part_o + (((size_t)(t0 + tile0 + row) * a.nh + head) * a.splits + split) * hd;
+#pragma unroll
+            for (int d = 0; d < HDT; ++d) dst[16 * d + j] = o[d][e];
+        }
+        return;
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
         const int row = 4 * g + e;                                // slot (position) this lane's values belong to
@@ -1047,14 +1124,36 @@ extern "C" int agave_attn_decode_fused(const void* q, long ldq, const void* k, l
     return launch_decode<true>(a, f, N, stream);
 }
 
+// How many workgroups should share a block of positions' pages in a prefill of these sizes (1:
+// none).  page_span: the most pages a block of positions reaches back over.  More than one only
+// for the streamlined kernel (head sizes 64, 128, 256) with eight waves, when its blocks leave
+// more than a third of the 256 compute units idle and every share still has four pages.
+extern "C" int agave_attn_prefill_splits(int n_seqs, int max_new, int nh, int nkv, int hd, int page_span) {
+    if (n_seqs <= 0 || max_new <= 32 || nkv <= 0 || nh % nkv != 0 || !(hd == 64 || hd == 128 || hd == 256)) return 1;
+    const int G = nh / nkv;
+    const int hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
+    const int blk_len = (8 / hw) * 16;
+    const long wgs = (long)((max_new + blk_len - 1) / blk_len) * nkv * ((G + hw - 1) / hw) * n_seqs;
+    int s = (int)(256 / (wgs > 0 ? wgs : 1));
+    if (wgs > 170) s = 1;
+    if (s > 4) s = 4;
+    while (s > 1 && page_span / s < 4) --s;
+    return s < 1 ? 1 : s;
+}
+
+// splits > 1 (only what agave_attn_prefill_splits gives): part_o [N][nh][splits][hd] and part_ml
+// [N][nh][splits][2], 32-bit, take the partial results.
 extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long ldo, const void* k_pages,
                                        const void* v_pages, const int* table, int width, const int* base,
                                        int n_pages, const int* tok_seq, const int* tok_pos, const int* cu, int n_seqs,
                                        int max_new, int N, int nh, int nkv, int hd, float scale, int window,
-                                       hipStream_t stream) {
-    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, nullptr, nullptr, (const uint4*)k_pages, (const uint4*)v_pages,
-               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, 1, 0, 0, 0};
+                                       float* part_o, float* part_ml, int splits, hipStream_t stream) {
+    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
+               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, splits, 0, 0, 0};
     if (check_common("attn_prefill_mfma", a, N)) return -1;
+    AGAVE_CHECK(splits >= 1 && splits <= 4, "attn_prefill_mfma: %d splits", splits);
+    AGAVE_CHECK(splits == 1 || (part_o && part_ml && max_new > 32 && (hd == 64 || hd == 128 || hd == 256)),
+                "attn_prefill_mfma: splits need the partial buffers and the eight-wave kernel's sizes");
     AGAVE_CHECK(cu && n_seqs > 0 && max_new > 0, "attn_prefill_mfma: needs the sequences' token ranges");
     AGAVE_CHECK(n_seqs <= 65535, "attn_prefill_mfma: %d sequences exceed the grid limit", n_seqs);
     if (N == 0) return 0;
@@ -1070,7 +1169,7 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
     const int wg_heads = qt_heads * hw, blk_len = (nwv / hw) * 16;
     const int chunks = (G + wg_heads - 1) / wg_heads;
     AGAVE_CHECK(nkv * chunks <= 65535, "attn_prefill_mfma: too many head chunks");
-    dim3 grid((max_new + blk_len - 1) / blk_len, nkv * chunks, n_seqs);
+    dim3 grid((max_new + blk_len - 1) / blk_len * splits, nkv * chunks, n_seqs);
     // two pages (K and V tiles) in LDS
     const size_t lds = (size_t)2 * (4 * ((hd + 31) / 32) + (hd / 16) * 2) * 64 * sizeof(uint4);
     static bool raised = false;
@@ -1101,5 +1200,14 @@ extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long 
     else if (hd <= 128) attn_prefill_mfma_kernel<8, 2><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else attn_prefill_mfma_kernel<16, 1><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     AGAVE_LAUNCH_CHECK("attn_prefill_mfma");
+    if (splits > 1) {
+        AGAVE_CHECK((long)N * nh < (1L << 31), "attn_prefill_mfma: too many (token, head) pairs for the combine pass");
+        const long rows = (long)N * nh;
+        if (ldo % 4 == 0 && ((uintptr_t)out % 8) == 0 && splits <= COMBINE_ROWS_MAX_SPLITS)
+            attn_combine_rows_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, stream>>>(part_o, part_ml, a.out, a.ldo, nh, hd, splits, rows);
+        else
+            attn_combine_kernel<<<N * nh, hd >= 256 ? 256 : (hd >= 128 ? 128 : 64), 0, stream>>>(part_o, part_ml, a.out, a.ldo, nh, hd, splits);
+        AGAVE_LAUNCH_CHECK("attn_combine");
+    }
     return 0;
 }

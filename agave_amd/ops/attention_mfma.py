@@ -13,7 +13,9 @@ kernels.register_signatures("attention_mfma", {
                                _I, _P],
     "agave_attn_decode_fused": [_P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I,
                                 _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _P],
-    "agave_attn_prefill_mfma": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "agave_attn_prefill_mfma": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
+                                _I, _P],
+    "agave_attn_prefill_splits": [_I, _I, _I, _I, _I, _I],
 })
 
 TARGET_WORKGROUPS = 256      # workgroups (of 4 waves) a decode launch aims for: one per compute unit
@@ -57,10 +59,19 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
                      1 if step.n_seqs == n else 0, 1 if getattr(step, "tables_start_at_reach", False) else 0,
                      kernels.stream())
     else:
+        # a prompt with few blocks of positions: several workgroups share a block's pages
+        splits = int(lib.agave_attn_prefill_splits(step.n_seqs, step.max_new, n_heads, n_kv, head_dim,
+                                                   step.page_span(window)))
+        part_o = part_ml = None
+        if splits > 1:
+            ws = step.workspace
+            part_o = ws.get("attn_part_o", n * n_heads * splits, head_dim, torch.float32)
+            part_ml = ws.get("attn_part_ml", n * n_heads * splits, 2, torch.float32)
         library.call(lib, "agave_attn_prefill_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
                      k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width, base.data_ptr(), n_pages,
                      step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), step.cu_dev.data_ptr(), step.n_seqs,
-                     step.max_new, n, n_heads, n_kv, head_dim, scale, w, kernels.stream())
+                     step.max_new, n, n_heads, n_kv, head_dim, scale, w, kernels.ptr(part_o), kernels.ptr(part_ml),
+                     splits, kernels.stream())
 
 
 FUSED_HEAD_DIMS = (64, 128, 256)

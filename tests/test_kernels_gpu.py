@@ -550,6 +550,20 @@ def test_attn_mfma_long_sequences_split_over_workgroups(K, decode):
     assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,lens,window", [(4, 2, 128, [1500], None), (4, 2, 128, [1500], 1024),
+                                                   (8, 4, 256, [700, 300], None), (2, 2, 64, [1100, 64, 1], 600)])
+def test_attn_mfma_prefill_blocks_shared_among_workgroups(K, nh, nkv, hd, lens, window):
+    """A prompt with few blocks of positions: several workgroups share a block's pages and a
+    second pass merges what they leave."""
+    from agave_amd.ops import attention_mfma, kernels
+    step = _FakeStep(lens, lambda L: 0, window)
+    lib = kernels.lib("attention_mfma")
+    assert lib.agave_attn_prefill_splits(len(lens), max(lens), nh, nkv, hd, step.page_span(window)) > 1
+    got, ref, _ = _mfma_attn_case(K, nh, nkv, hd, lens, window, 0.3 * (16 / hd) ** 0.5, False, seed=7)
+    assert torch.isfinite(got).all()
+    assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("decode", [True, False])
 def test_attn_mfma_far_key_and_window_edge(K, decode):
     got, ref, vs = _mfma_attn_case(K, 2, 1, 32, [700], None, 0.5, decode, seed=1, boost=3)
