@@ -42,7 +42,7 @@ def kinds_of(rows, vocab: int) -> int:
     for r in rows:
         if r.temperature > 0:
             kinds |= KIND_TEMPERATURE
-            if 0 < r.top_k < vocab or 0.0 < r.top_p < 1.0:
+            if 0 < min(r.top_k, 1 << 20) < vocab or 0.0 < r.top_p < 1.0:     # (top_k travels capped at 2^20)
                 kinds |= KIND_FILTER
     return kinds
 
