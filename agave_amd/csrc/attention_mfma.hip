@@ -350,7 +350,11 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
             for (int k = 0; k < NV; ++k) vreg0[k] = vsrc0[lane + 64 * k];
         }
     }
-    const int col0 = split * a.pages_per_split + wave;
+    // A wave takes half pages (units of 32 keys): wave w the half w % 2 of the pages
+    // page_lo + w / 2, + 2, + 4, ... of the workgroup's range, so that four waves share two pages
+    // at a time and a range of 2 pages is one unit, one round trip to memory, for every wave.
+    const int half = wave & 1, wpage = wave >> 1;
+    const int col0 = split * a.pages_per_split + wpage;
     int pg0 = -1;                             // (kept as loaded: widening it here would wait for the load)
     if (a.table_from_reach && col0 < a.width) pg0 = a.table[(size_t)b * a.width + col0];
     const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
@@ -378,18 +382,20 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     float m_ref = -INFINITY, l = 0.f;
 
     constexpr size_t k_stride = (size_t)4 * KS * 64, v_stride = (size_t)HDT * 2 * 64;   // uint4 per (page, kv head)
-    const int n_my = (page_hi >= page_lo + wave) ? (page_hi - page_lo - wave) / 4 + 1 : 0; // pages this wave takes
+    // (the second half of the token's own page holds no key yet when the position lies in its first half)
+    const int my_hi = (half == 1 && page_hi == last && p % AGAVE_PAGE < 32) ? page_hi - 1 : page_hi;
+    const int n_my = (my_hi >= page_lo + wpage) ? (my_hi - page_lo - wpage) / 2 + 1 : 0;   // pages this wave takes
     // the ids of this wave's first pages are fetched together, ahead of any use: a lookup in the
     // loop would stand between every two pages
-    constexpr int PG_AHEAD = 8;
+    constexpr int PG_AHEAD = 10;
     int pg_pre[PG_AHEAD];
 #pragma unroll
     for (int i = 1; i < PG_AHEAD; ++i) {
-        const int col = page_lo + wave + 4 * i - first;
+        const int col = page_lo + wpage + 2 * i - first;
         pg_pre[i] = (a.table_from_reach && i < n_my && col < a.width) ? a.table[(size_t)b * a.width + col] : -1;
     }
     auto page_id = [&](int i) -> int {           // i-th page of this wave (page ids fit 31 bits)
-        const int pi = page_lo + wave + 4 * i;
+        const int pi = page_lo + wpage + 2 * i;
         int pg;
         if (a.table_from_reach) {
             const int col = pi - first;
@@ -412,18 +418,18 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     frag16 kb[2][KS], vb[HDT];
     const u32x4_t* kp = nullptr;
     const u32x4_t* vp = nullptr;
-    auto load_k = [&](int half) {
+    auto load_k = [&]() {
 #pragma unroll
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) kb[kt][ks].r = kp[((2 * half + kt) * KS + ks) * 64 + lane];
     };
-    auto load_v = [&](int half) {
+    auto load_v = [&]() {
 #pragma unroll
         for (int d = 0; d < HDT; ++d) vb[d].r = vp[(d * 2 + half) * 64 + lane];
     };
 
-    // units: half pages, in order; the next unit's K and V are fetched while this one is used
+    // units: this wave's half of its pages, in order; the next unit's K and V are fetched while this one is used
     int cur_page = 0;
     int pg = n_my > 0 ? page_id(0) : -1;
     bool have = n_my > 0 && pg >= 0;
@@ -434,10 +440,10 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     // FUSED: the token's own key and value go into the page of position p, by the workgroup that
     // reads it; the wave whose first page that is waits with its loads until the row is there
     const bool writer = FUSED && f.k_raw != nullptr && page_lo <= last && page_hi == last;
-    const bool early = !(writer && page_lo + wave == last);
+    const bool early = !(writer && page_lo + wpage == last);
     if (have && early) {
-        load_k(0);
-        load_v(0);
+        load_k();
+        load_v();
     }
     if constexpr (FUSED) {
         float* ybuf = lds + (size_t)4 * slots * hd + 4 * 16 * 2 + (size_t)wave * hd;
@@ -499,12 +505,11 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
         }
     }
     if (have && !early) {
-        load_k(0);
-        load_v(0);
+        load_k();
+        load_v();
     }
-    int half = 0;
     while (have) {
-        const int pi = page_lo + wave + 4 * cur_page;
+        const int pi = page_lo + wpage + 2 * cur_page;
         const int key0 = pi * AGAVE_PAGE + 32 * half;             // first key of this unit
         // S^T for the unit's two key tiles
         f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0;
@@ -514,10 +519,10 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
             st1 = mfma_16x16x32(kb[1][ks], qf[ks], st1);
         }
         // where the next unit lies, and its keys (the K registers are free now)
-        int n_half = half ^ 1, n_page = cur_page + (half == 1);
+        const int n_page = cur_page + 1;
         bool n_have = n_page < n_my;
         const u32x4_t* nvp = vp;
-        if (n_have && half == 1) {
+        if (n_have) {
             const int npg = page_id(n_page);
             if (npg < 0) {
                 n_have = false;
@@ -526,7 +531,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
                 nvp = (const u32x4_t*)(a.v_pages + ((size_t)npg * a.nkv + kvh) * v_stride);
             }
         }
-        if (n_have) load_k(n_half);
+        if (n_have) load_k();
         // scores -> probabilities against the running reference
         float s[8];
 #pragma unroll
@@ -572,8 +577,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
 #pragma unroll
         for (int d = 0; d < HDT; ++d) o[d] = mfma_16x16x32(pf, vb[d], o[d]);
         vp = nvp;
-        if (n_have) load_v(n_half);
-        half = n_half;
+        if (n_have) load_v();
         cur_page = n_page;
         have = n_have;
     }
