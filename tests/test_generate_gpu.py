@@ -96,6 +96,38 @@ def test_temperature_sampling_is_seeded_and_independent_of_batch_mates(model_b):
         toks.append(got)
 
 
+def test_sampling_kinds_mixed_in_a_batch_with_a_large_vocabulary(tmp_path):
+    """A vocabulary of 5,003 takes the sampler that shares a row among workgroups: greedy,
+    temperature, top-k and top-p requests in one batch, each following the plain rule for the u
+    of its own stream."""
+    from agave_amd import Engine, SamplingParams
+    cfg = dict(P.tiny_config("A"), vocab_size=5003)
+    w = P.random_weights(cfg, 5)
+    folder = U.write_model(str(tmp_path), cfg, w)
+    eng = Engine.from_folder(folder, dtype="float32", max_slots=4, max_context=64)
+    prompts = [U.random_tokens(n, 5003, 200 + i) for i, n in enumerate((3, 9, 17, 6))]
+    sps = [SamplingParams(max_tokens=6, temperature=0.0, ignore_eos=True),
+           SamplingParams(max_tokens=6, temperature=0.9, seed=4, ignore_eos=True),
+           SamplingParams(max_tokens=6, temperature=1.1, top_k=7, seed=5, ignore_eos=True),
+           SamplingParams(max_tokens=6, temperature=0.8, top_k=50, top_p=0.7, seed=6, ignore_eos=True)]
+    got = [r.tokens for r in eng.generate(prompts, sps)]
+    assert got == [r.tokens for r in eng.generate(prompts, sps, max_batch=3)]
+    for i, sp in enumerate(sps):
+        rng = np.random.default_rng([sp.seed if sp.seed is not None else 0, i])
+        toks = list(prompts[i])
+        for tok in got[i]:
+            u = float(rng.random(dtype=np.float32)) if sp.temperature > 0 else 0.0
+            logits = P.forward(cfg, w, toks)[-1].float()
+            want = P.sample_token(logits, sp.temperature, sp.top_k, sp.top_p, u)
+            if tok != want:
+                # a draw that falls within rounding of an interval's edge may go to the neighbour
+                wts = P.sample_distribution(logits, sp.temperature, sp.top_k, sp.top_p)
+                cdf = torch.cumsum(wts, 0) / wts.sum()
+                edge = min(abs(float(cdf[tok]) - u), abs(float(cdf[tok - 1]) - u) if tok else 1.0)
+                assert float(wts[tok]) > 0 and edge < 1e-4, (i, tok, want)
+            toks.append(tok)
+
+
 def test_command_line_json(model_a):
     cfg, w, folder = model_a
     prompt = [2] + U.random_tokens(6, 512, 110)
