@@ -168,3 +168,20 @@ def test_repeat_penalty_is_not_run_ahead():
     be = AheadBackend(max_slots=1)
     generate(be, [[7, 8]], SamplingParams(max_tokens=3, repeat_penalty=1.3))
     assert be.max_in_flight == 0 and [s["gen"][0] for s in be.steps] == [[], [9], [9, 10]]
+
+
+def test_the_sampler_is_told_what_the_rows_need():
+    """Which of the sampler's kernels a batch needs is decided on the host, from the rows'
+    options, exactly as a row decides for itself on the device."""
+    from agave_amd.ops import sampling as S
+
+    class Row:
+        def __init__(self, temperature, top_k=0, top_p=1.0):
+            self.temperature, self.top_k, self.top_p = temperature, top_k, top_p
+    vocab = 5000
+    assert S.kinds_of([Row(0.0), Row(0.0, 40, 0.5)], vocab) == 0                    # greedy rows need neither
+    assert S.kinds_of([Row(0.0), Row(0.7)], vocab) == S.KIND_TEMPERATURE
+    assert S.kinds_of([Row(0.7, top_k=vocab)], vocab) == S.KIND_TEMPERATURE          # top-k of the whole row is none
+    assert S.kinds_of([Row(0.7, top_p=1.0), Row(0.7, top_k=0)], vocab) == S.KIND_TEMPERATURE
+    assert S.kinds_of([Row(0.7, top_k=3)], vocab) == S.KIND_ALL
+    assert S.kinds_of([Row(0.0), Row(1.2, top_p=0.9)], vocab) == S.KIND_ALL
