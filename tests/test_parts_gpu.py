@@ -233,6 +233,37 @@ def test_gated_ffn_part(dtype, hidden, inter, rows):
     check(y, P.geglu(x, t["f.g"], t["f.u"], t["f.d"]), dtype, "feed-forward")
 
 
+def test_gated_ffn_at_a_prompts_length_comes_in_slices_that_the_residual_kernel_adds():
+    """The benchmark model's feed-forward at 2,048 tokens: the down product's tiles would leave
+    many compute units idle, so it comes as 32-bit slices; summed, and added to the residual
+    stream by the norm kernel, they give what the formula gives (the plain formula runs on the
+    GPU here, in 64-bit: it is a hundred GFLOP)."""
+    from agave_amd.config.spec import GatedFfnSpec, NormSpec
+    from agave_amd.parts import GatedFfn, add_pending_and_norm, lookup
+    hidden, inter, rows = 2560, 10240, 2048
+    spec = GatedFfnSpec(kind="gated_dense", hidden=hidden, intermediate=inter, activation="gelu_tanh",
+                        gate_proj="f.g", up_proj="f.u", down_proj="f.d")
+    t = {"f.g": rnd((inter, hidden), 60, 0.02), "f.u": rnd((inter, hidden), 61, 0.02), "f.d": rnd((hidden, inter), 62, 0.02)}
+    b = Bench("bfloat16")
+    part = GatedFfn(spec, weights_of(t, GatedFfn.tensor_needs(spec), "bfloat16"), b.env)
+    x = rnd((rows, hidden), 63, 1.0)
+    y = part.forward(x.to(torch.bfloat16).to(DEV), None)
+    assert y.dim() == 3 and y.shape[0] > 1 and y.dtype == torch.float32
+    ref = P.geglu(x.to(DEV), t["f.g"].to(DEV), t["f.u"].to(DEV), t["f.d"].to(DEV)).cpu()
+    check(y.sum(0), ref, "bfloat16", "feed-forward in slices")
+    # the norm kernel adds the slices to the residual stream and normalises the sum
+    nspec = NormSpec("rmsnorm", hidden, 1e-6, "n.w", True)
+    norm = lookup("norm", "rmsnorm")(nspec, weights_of({"n.w": rnd((hidden,), 64, 0.1)}, lookup("norm", "rmsnorm").tensor_needs(nspec),
+                                                        "bfloat16"), b.env)
+    h0 = rnd((rows, hidden), 65, 1.0).float()
+    h = h0.clone().to(DEV)
+    out = torch.empty(rows, hidden, dtype=torch.bfloat16, device=DEV)
+    add_pending_and_norm(h, (y, None), norm, out)
+    want_h = h0.double() + ref
+    check(h, want_h, "bfloat16", "residual stream after the slices")
+    check(out, P.rms_norm(want_h, rnd((hidden,), 64, 0.1), 1e-6, add_one=True), "bfloat16", "norm of the sum")
+
+
 def test_gated_ffn_refuses_unknown_activation():
     from agave_amd.config.spec import GatedFfnSpec
     from agave_amd.parts import GatedFfn
