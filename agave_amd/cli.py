@@ -4,9 +4,10 @@ Options keep the reference's names and meanings where it has them (``src/main.zi
 ``-n/--max-tokens`` (512), ``-t/--temperature`` (0 = greedy), ``--top-p`` (1.0), ``--top-k``
 (0 = off), ``--repeat-penalty`` (1.0), ``--seed``, ``--ctx-size`` (0 = the model's full
 context; default min(model, 4096), ``:345, 1096-1113``), ``--prefill-batch-size``, ``--json``,
-``--model-info``, ``-q/--quiet``, ``-V/--verbose``, ``-v/--version``.  The reference's
-options for its server, other backends, quantised caches, vision, speculative decoding and
-grammars have no counterpart here.  There is no tokenizer in this library: a prompt is a list
+``--model-info``, ``--profile``, ``-q/--quiet``, ``-V/--verbose``, ``-d/--debug``, ``-v/--version``,
+``--backend`` (only ``auto`` and ``rocm`` exist here).  The reference's options for its server,
+quantised caches, vision, speculative decoding, its single-dispatch kernel and grammars have no
+counterpart here.  There is no tokenizer in this library: a prompt is a list
 of token ids ("2 17 5" or "2,17,5"), and the output is token ids.
 
 Added: ``--prompt-file`` (one request per line), ``--dtype``, ``--max-batch``, ``--ignore-eos``,
@@ -52,6 +53,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("-q", "--quiet", action="store_true", help="suppress stats (raw output only)")
     ap.add_argument("-V", "--verbose", action="store_true", help="show technical details")
     ap.add_argument("-v", "--version", action="store_true", help="print version and exit")
+    ap.add_argument("-d", "--debug", action="store_true",
+                    help="debug output (the token ids that are fed, per-request details); implies --verbose")
+    ap.add_argument("--backend", default="auto",
+                    help="compute backend: auto or rocm (the reference's other backends do not exist here) [default: auto]")
     # not in the reference
     ap.add_argument("--prompt-file", help="file with one prompt (token ids) per line; runs them as batches")
     ap.add_argument("--prompt-ids", help="token ids of the prompt (same as the positional)")
@@ -91,6 +96,10 @@ def main(argv: Optional[List[str]] = None) -> int:
         ap.error("--top-p must be in (0, 1]")
     if args.repeat_penalty <= 0:
         ap.error("--repeat-penalty must be > 0")
+    if args.backend not in ("auto", "rocm"):
+        ap.error(f"--backend {args.backend}: this library runs on rocm (one MI355X) only")
+    if args.debug:
+        args.verbose = True
     quiet = args.quiet or args.json
 
     if args.random_weights:
@@ -134,6 +143,9 @@ def main(argv: Optional[List[str]] = None) -> int:
     if bos is not None and not args.no_bos:
         prompts = [p if (p and p[0] == bos) else [bos] + p for p in prompts]   # src/main.zig:2199-2208
 
+    if args.debug and not quiet:
+        for i, p in enumerate(prompts):
+            print(f"[debug] request {i}: {len(p)} prompt token ids: {' '.join(map(str, p))}", file=sys.stderr)
     params = SamplingParams(max_tokens=args.max_tokens, temperature=args.temperature, top_k=args.top_k,
                             top_p=args.top_p, repeat_penalty=args.repeat_penalty, seed=args.seed,
                             ignore_eos=args.ignore_eos)

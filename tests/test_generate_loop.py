@@ -185,3 +185,21 @@ def test_the_sampler_is_told_what_the_rows_need():
     assert S.kinds_of([Row(0.7, top_p=1.0), Row(0.7, top_k=0)], vocab) == S.KIND_TEMPERATURE
     assert S.kinds_of([Row(0.7, top_k=3)], vocab) == S.KIND_ALL
     assert S.kinds_of([Row(0.0), Row(1.2, top_p=0.9)], vocab) == S.KIND_ALL
+
+
+def test_command_line_options_follow_the_reference():
+    """src/main.zig:325-382: names, short forms and defaults of the options this library has."""
+    from agave_amd.cli import build_parser, parse_ids
+    ap = build_parser()
+    a = ap.parse_args(["m"])
+    assert (a.max_tokens, a.temperature, a.top_p, a.top_k, a.repeat_penalty, a.seed) == (512, 0.0, 1.0, 0, 1.0, None)
+    assert a.ctx_size is None and a.backend == "auto" and not (a.json or a.quiet or a.verbose or a.debug or a.profile)
+    a = ap.parse_args(["m", "2 17 5", "-n", "9", "-t", "0.8", "--top-p", "0.9", "--top-k", "40", "--repeat-penalty", "1.1",
+                       "--seed", "3", "--ctx-size", "0", "--prefill-batch-size", "512", "--json", "--model-info", "-q", "-V",
+                       "-d", "--profile", "--backend", "rocm"])
+    assert (a.max_tokens, a.temperature, a.top_p, a.top_k, a.repeat_penalty, a.seed) == (9, 0.8, 0.9, 40, 1.1, 3)
+    assert a.ctx_size == 0 and a.prefill_batch_size == 512 and a.json and a.model_info and a.quiet and a.verbose
+    assert a.debug and a.profile and a.backend == "rocm" and a.prompt == "2 17 5"
+    assert parse_ids("2, 17  5") == [2, 17, 5]
+    with pytest.raises(SystemExit):
+        parse_ids("hello")
