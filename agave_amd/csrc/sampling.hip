@@ -11,6 +11,12 @@
 #include "common_impl.h"
 #include <math.h>
 
+// No multiplication in this file is fused with a following addition: the scaled logit x * 1/T is
+// rounded by itself, so that it has the same bits in every kernel here.  Fused into the subtraction
+// of the maximum it would differ in its last bit from place to place, and an entry whose weight has
+// to equal a threshold that another kernel found (the largest weight, say) would fall below it.
+#pragma clang fp contract(off)
+
 #define SAMPLE_THREADS 1024
 #define MAX_CAND 1024
 
@@ -125,7 +131,8 @@ __device__ void block_argmax(const float* __restrict__ x, int n, float mult, flo
 #define SP_OFF_MAX 0                          // float[64]: the pieces' maxima
 #define SP_OFF_IDX 64                         // int[64]: lowest index holding each
 #define SP_OFF_SUM 128                        // float[64]: the pieces' sums of weights
-#define SP_OFF_NCAND 192                      // uint: collected entries
+#define SP_OFF_NCAND 192                      // uint: collected entries above the threshold value
+#define SP_OFF_NTIE 193                       // uint: entries that equal it
 #define SP_OFF_H0 256                         // uint[2048]: histogram of key bits 31..21
 #define SP_OFF_H1 (SP_OFF_H0 + 2048)          // uint[2048]: bits 20..10 under the first digit
 #define SP_OFF_H2 (SP_OFF_H1 + 2048)          // uint[1024]: bits 9..0 under the first two
@@ -178,7 +185,7 @@ __global__ __launch_bounds__(SP_THREADS) void sp_max_kernel(const float* __restr
     if (clear) {
         constexpr int SHARE = SP_HIST_WORDS / SP_PARTS;
         for (int i = threadIdx.x; i < SHARE; i += blockDim.x) reinterpret_cast<uint32_t*>(rowf)[SP_OFF_H0 + part * SHARE + i] = 0;
-        if (part == 0 && threadIdx.x == 0) reinterpret_cast<uint32_t*>(rowf)[SP_OFF_NCAND] = 0;
+        if (part == 0 && threadIdx.x < 2) reinterpret_cast<uint32_t*>(rowf)[SP_OFF_NCAND + threadIdx.x] = 0;
     }
     int lo, n;
     part_range(V, part, &lo, &n);
@@ -290,7 +297,7 @@ __device__ void sp_pick_digit(const uint32_t* __restrict__ hist, int bins, uint3
 // first digit, ROUND 2: the first two, ROUND 3: all three, the threshold key itself).
 template <int ROUND>
 __device__ void sp_prefix(const uint32_t* __restrict__ row, uint32_t want, uint32_t* prefix, uint32_t* arr,
-                          uint32_t* sh) {
+                          uint32_t* sh, uint32_t* wanted_of_last = nullptr) {
     uint32_t krem = want, d;
     *prefix = 0;
     if (ROUND >= 1) {
@@ -305,6 +312,7 @@ __device__ void sp_prefix(const uint32_t* __restrict__ row, uint32_t want, uint3
         sp_pick_digit(row + SP_OFF_H2, 1024, krem, &d, &krem, arr, sh);
         *prefix |= d;
     }
+    if (wanted_of_last) *wanted_of_last = krem;         // entries still wanted among those with the last digit found
 }
 
 // One round of the selection: the histogram of this round's digit over the entries whose key
@@ -339,8 +347,9 @@ __global__ __launch_bounds__(SP_THREADS) void sp_hist_kernel(const float* __rest
         if (h[i]) atomicAdd(&row[OFF + i], h[i]);
 }
 
-// The entries at or above the threshold key (the want-th largest value and its ties), in any
-// order; at most MAX_CAND are kept.
+// The entries above the threshold key (the want-th largest value; fewer than want of them),
+// in any order, then the entries that equal it, as many as still fit MAX_CAND: what is left out
+// then equals what was taken.
 __global__ __launch_bounds__(SP_THREADS) void sp_collect_kernel(const float* __restrict__ logits, long ld,
                                                                 const float* __restrict__ params,
                                                                 float* __restrict__ scratch, int V) {
@@ -351,13 +360,15 @@ __global__ __launch_bounds__(SP_THREADS) void sp_collect_kernel(const float* __r
     if (!m.filt) return;
     float* rowf = scratch + (size_t)b * SP_ROW_WORDS;
     uint32_t* row = reinterpret_cast<uint32_t*>(rowf);
-    uint32_t thr;
-    sp_prefix<3>(row, (uint32_t)m.want, &thr, arr, sh);
+    uint32_t thr, ties_wanted;
+    sp_prefix<3>(row, (uint32_t)m.want, &thr, arr, sh, &ties_wanted);
+    const uint32_t n_above = (uint32_t)m.want - ties_wanted;        // entries above the threshold value
     int lo, n;
     part_range(V, part, &lo, &n);
     for_piece(logits + (size_t)b * ld + lo, n, m.inv_t, [&](int i, float v) {
-        if (ordered_key(v) >= thr) {
-            const uint32_t at = atomicAdd(&row[SP_OFF_NCAND], 1u);
+        const uint32_t key = ordered_key(v);
+        if (key >= thr) {
+            const uint32_t at = key > thr ? atomicAdd(&row[SP_OFF_NCAND], 1u) : n_above + atomicAdd(&row[SP_OFF_NTIE], 1u);
             if (at < MAX_CAND) {
                 rowf[SP_OFF_CV + at] = v;
                 reinterpret_cast<int*>(rowf)[SP_OFF_CI + at] = lo + i;
@@ -421,6 +432,80 @@ __device__ void sort_pairs(K* key, P* pay, int span, F before) {
         }
 }
 
+// Goes through x[0..n) in index order, 4096 elements at a time (loaded side by side, then four
+// in a row per thread), with the weight exp(v - mx) of every element whose scaled value v is
+// at least kth and whose weight is at least thr (others weigh nothing).  Returns the first
+// index whose running sum of weights exceeds rem, or -1 if none does; *sum gets the weights'
+// sum up to where the walk ended (all of them when nothing was found), *last_pos the last index
+// seen with any weight (-1: none).  All 1024 threads of the workgroup call; chunk: 4096 floats
+// of LDS, wtot: 16, sh: 2 ints.  The result is the same in every thread.
+__device__ int weights_walk(const float* __restrict__ x, int n, float inv_t, float mx, float kth, float thr, float rem,
+                            float* chunk, float* wtot, int* sh, float* sum, int* last_pos) {
+    const int tid = threadIdx.x;
+    float acc = 0.f;
+    int last = -1;
+    __syncthreads();
+    if (tid == 0) sh[1] = -1;
+    __syncthreads();
+    for (int c0 = 0; c0 < n; c0 += 4 * SAMPLE_THREADS) {
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int i = c0 + tid + k * SAMPLE_THREADS;
+            v[k] = x[i < n ? i : n - 1];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int i = c0 + tid + k * SAMPLE_THREADS;
+            const float sv = v[k] * inv_t;
+            float w = (i < n && sv >= kth) ? weight_of(sv, mx) : 0.f;
+            if (w < thr) w = 0.f;
+            chunk[tid + k * SAMPLE_THREADS] = w;
+        }
+        __syncthreads();
+        float w4[4], s4 = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            w4[k] = chunk[tid * 4 + k];
+            s4 += w4[k];
+        }
+        float total, before;
+        const float run = block_running_sum(s4, wtot, &before, &total);
+        if (s4 > 0.f && rem < run && rem >= before) {             // this thread's four hold the target
+            float c = before;
+            int pick = -1, last_k = -1;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                c += w4[k];
+                if (w4[k] > 0.f) {
+                    last_k = k;
+                    if (pick < 0 && rem < c) pick = k;
+                }
+            }
+            if (pick < 0) pick = last_k;         // (the four's own sum rounds differently: their last weight)
+            sh[1] = c0 + tid * 4 + pick;
+        }
+        // the chunk's last index with any weight, should nothing hold the target
+        int mine = -1;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (w4[k] > 0.f) mine = c0 + tid * 4 + k;
+        __syncthreads();
+        if (tid == 0) sh[0] = -1;
+        __syncthreads();
+        if (mine >= 0) atomicMax(&sh[0], mine);
+        __syncthreads();
+        if (sh[0] >= 0) last = sh[0];
+        if (sh[1] >= 0) break;                   // (uniform: read after a barrier)
+        rem -= total;
+        acc += total;
+    }
+    *sum = acc;
+    *last_pos = last;
+    return sh[1];
+}
+
 // One workgroup of 1024 threads per row decides.
 __global__ __launch_bounds__(SAMPLE_THREADS) void sp_final_kernel(const float* __restrict__ logits, long ld,
                                                                   const float* __restrict__ params,
@@ -456,7 +541,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sp_final_kernel(const float* _
     const float mx = sp_row_max(rowf) * m.inv_t;
     bool whole_row = !m.filt;
     if (m.filt) {
-        uint32_t n = reinterpret_cast<const uint32_t*>(rowf)[SP_OFF_NCAND];
+        uint32_t n = reinterpret_cast<const uint32_t*>(rowf)[SP_OFF_NCAND] + reinterpret_cast<const uint32_t*>(rowf)[SP_OFF_NTIE];
+        const bool overflow = n > MAX_CAND;
         if (n > MAX_CAND) n = MAX_CAND;
         // by falling value (ties: rising index), for the thresholds
         cv[tid] = tid < (int)n ? rowf[SP_OFF_CV + tid] : -INFINITY;
@@ -470,7 +556,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sp_final_kernel(const float* _
         float e = (tid < (int)n && cv[tid] >= kth) ? weight_of(cv[tid], mx) : 0.f;
         float sum, before;
         const float run = block_running_sum(e, wtot, &before, &sum);    // in the order of falling value
-        if (!m.use_k) sum = sp_parts_total(rowf);                       // nothing dropped yet: the whole row's sum
+        if (!m.use_k) {
+            sum = sp_parts_total(rowf);                                 // nothing dropped yet: the whole row's sum
+        } else if (overflow && m.use_p) {
+            // entries that tie with the last collected one were left out: the sum of what top-k keeps
+            // is taken from the row itself
+            int none_i;
+            weights_walk(logits + (size_t)b * ld, V, m.inv_t, mx, kth, 0.f, INFINITY, chunk, wtot, sh_i, &sum, &none_i);
+        }
         if (m.use_p) {
             // the smallest prefix of the sorted weights whose mass reaches top_p * sum; every weight
             // at or above the last one taken stays.  Not reached within the collected entries: nothing is dropped.
@@ -482,6 +575,21 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sp_final_kernel(const float* _
             const float thr = sh_f[0];
             if (thr == 0.f && !m.use_k) whole_row = true;
             if (e < thr) e = 0.f;
+        }
+        if (!whole_row && overflow) {
+            // More entries than the collection holds tie with its last one (a thousand equal
+            // logits): the thresholds above are still exact, because what was left out equals what
+            // was taken; the draw then walks the whole row with them, once for the sum and once
+            // for the place (slow, and rare).
+            const float kth_v = kth;
+            const float thr_w = m.use_p ? sh_f[0] : 0.f;
+            const float* x = logits + (size_t)b * ld;
+            float total, part_sum;
+            int last_pos;
+            weights_walk(x, V, m.inv_t, mx, kth_v, thr_w, INFINITY, chunk, wtot, sh_i, &total, &last_pos);
+            const int at = weights_walk(x, V, m.inv_t, mx, kth_v, thr_w, m.u * total, chunk, wtot, sh_i, &part_sum, &last_pos);
+            if (tid == 0) out[b] = at >= 0 ? at : (last_pos >= 0 ? last_pos : V - 1);
+            return;
         }
         if (!whole_row) {
             // by rising index, for the draw: the first kept index whose running sum exceeds u * sum
@@ -540,66 +648,14 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sp_final_kernel(const float* _
         }
         __syncthreads();
         const int part = sh_i[0];
-        float rem = sh_f[0];
+        const float rem = sh_f[0];
         int lo, n;
         part_range(V, part, &lo, &n);
-        const float* x = logits + (size_t)b * ld + lo;
-        if (tid == 0) sh_i[1] = -1;
-        int last_pos = -1;                       // (thread 0 keeps it) the last index of the piece with any weight
-        for (int c0 = 0; c0 < n; c0 += 4 * SAMPLE_THREADS) {
-            // 4096 elements at a time: loaded side by side, then four in a row per thread
-            float v[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int i = c0 + tid + k * SAMPLE_THREADS;
-                v[k] = x[i < n ? i : n - 1];
-            }
-            __syncthreads();
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int i = c0 + tid + k * SAMPLE_THREADS;
-                chunk[tid + k * SAMPLE_THREADS] = i < n ? weight_of(v[k] * m.inv_t, mx) : 0.f;
-            }
-            __syncthreads();
-            float w4[4], s4 = 0.f;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                w4[k] = chunk[tid * 4 + k];
-                s4 += w4[k];
-            }
-            float total, before;
-            const float run = block_running_sum(s4, wtot, &before, &total);
-            if (s4 > 0.f && rem < run && rem >= before) {             // this thread's four hold the target
-                float c = before;
-                int pick = -1, last_k = -1;
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    c += w4[k];
-                    if (w4[k] > 0.f) {
-                        last_k = k;
-                        if (pick < 0 && rem < c) pick = k;
-                    }
-                }
-                if (pick < 0) pick = last_k;     // (the four's own sum rounds differently: their last weight)
-                sh_i[1] = lo + c0 + tid * 4 + pick;
-            }
-            // the chunk's last index with any weight, should nothing hold the target
-            {
-                int mine = -1;
-#pragma unroll
-                for (int k = 0; k < 4; ++k)
-                    if (w4[k] > 0.f) mine = c0 + tid * 4 + k;
-                __syncthreads();
-                if (tid == 0) sh_i[0] = -1;
-                __syncthreads();
-                if (mine >= 0) atomicMax(&sh_i[0], mine);
-                __syncthreads();
-                if (sh_i[0] >= 0) last_pos = sh_i[0];
-            }
-            if (sh_i[1] >= 0) break;             // (uniform: read after a barrier)
-            rem -= total;
-        }
-        if (tid == 0) out[b] = sh_i[1] >= 0 ? sh_i[1] : (last_pos >= 0 ? lo + last_pos : V - 1);
+        float piece_sum;
+        int last_pos;
+        const int at = weights_walk(logits + (size_t)b * ld + lo, n, m.inv_t, mx, -INFINITY, 0.f, rem, chunk, wtot, sh_i,
+                                    &piece_sum, &last_pos);
+        if (tid == 0) out[b] = at >= 0 ? lo + at : (last_pos >= 0 ? lo + last_pos : V - 1);
     }
 }
 
@@ -664,9 +720,16 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
         if (tid == 0) n_cand = 0;
         for (int i = tid; i < MAX_CAND; i += blockDim.x) cand[i] = 0.f;
         __syncthreads();
+        // first what lies above the 1024th largest weight (fewer than 1024 entries), then its equals
+        // as far as there is room: which of them are left out does not matter, they are all the same
         for (int i = tid; i < V; i += blockDim.x) {
             const float e = w[i];
-            if (e > 0.f && ordered_key(e) >= min_key) {
+            if (e > 0.f && ordered_key(e) > min_key) cand[atomicAdd(&n_cand, 1u)] = e;
+        }
+        __syncthreads();
+        for (int i = tid; i < V; i += blockDim.x) {
+            const float e = w[i];
+            if (e > 0.f && ordered_key(e) == min_key) {
                 const uint32_t at = atomicAdd(&n_cand, 1u);
                 if (at < MAX_CAND) cand[at] = e;
             }

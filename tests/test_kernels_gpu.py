@@ -345,6 +345,36 @@ def test_sample_rows_are_independent_and_mixed(S):
     assert together == [P.sample_token(lg[i], *params[i]) for i in range(4)]
 
 
+@pytest.mark.parametrize("vocab", [3001, 4096, 40013])
+@pytest.mark.parametrize("temperature,top_k,top_p", [(0.8, 0, 0.01), (1.7, 5000, 0.01), (1.0, 1000, 1.0),
+                                                      (0.8, 0, 0.9), (1.3, 1024, 0.7), (1.0, 900, 0.5)])
+def test_sample_with_more_equal_logits_than_the_filter_collects(S, vocab, temperature, top_k, top_p):
+    """Some hundred logits above a plateau of far more than a thousand equal ones: the 1024 largest
+    end inside the plateau, all of which stays or goes together, and the draw has to range over
+    entries that the filter could not collect.  top_p = 0.01 keeps the maximum alone: its weight,
+    which is exactly 1, has to equal the threshold wherever it is computed again."""
+    g = torch.Generator().manual_seed(vocab + top_k)
+    logits = torch.randn(vocab, generator=g) * 2.0
+    plateau = float(torch.sort(logits, descending=True).values[700])
+    logits[::3] = plateau                                  # vocab / 3 equal entries below about 470 others
+    w = P.sample_distribution(logits, temperature, top_k, top_p)
+    cdf = torch.cumsum(w, 0) / w.sum()
+    support = torch.nonzero(w > 0).view(-1).tolist()
+    picks = support if len(support) <= 48 else [support[i] for i in range(0, len(support), len(support) // 48)]
+    picks = sorted(set(picks + support[-2:]))
+    us, want = [], []
+    for i in picks:
+        lo = float(cdf[i - 1]) if i > 0 else 0.0
+        hi = float(cdf[i])
+        if hi - lo < 1e-5:
+            continue
+        us.append((lo + hi) / 2)
+        want.append(i)
+    assert us
+    got = _sample(S, logits.view(1, -1).repeat(len(us), 1), [[temperature, top_k, top_p, u] for u in us])
+    assert got == want
+
+
 def test_sample_frequencies_follow_softmax(S):
     lg = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]])
     n = 4000
