@@ -521,7 +521,7 @@ class _FakeStep:
         return span
 
 
-def _mfma_attn_case(K, nh, nkv, hd, lens, window, scale, decode, seed=0, boost=None):
+def _mfma_attn_case(K, nh, nkv, hd, lens, window, scale, decode, seed=0, boost=None, last_row_only=False):
     """Keys and values go into packed pages through the q/k kernel (no norm, no rotation); then
     either every position is a query (prefill) or only each sequence's last one (decode)."""
     from agave_amd.ops import attention_mfma
@@ -556,9 +556,27 @@ def _mfma_attn_case(K, nh, nkv, hd, lens, window, scale, decode, seed=0, boost=N
     q_sel = torch.cat([q[p0:] for q, p0 in zip(qs, step.pos0)]).reshape(-1, nh * hd).to(DEV)
     out = torch.full_like(q_sel, float("nan"))
     attention_mfma.attention(q_sel, out, kp, vp, table, base, step, nh, nkv, hd, scale, window)
-    refs = [P.attention_core(q.double(), k.double(), v.double(), scale, window)[p0:]
-            for q, k, v, p0 in zip(qs, ks, vs, step.pos0)]
-    return out.cpu().double().view(-1, nh, hd), torch.cat(refs), vs
+    if last_row_only and not decode:
+        refs = []                                           # the caller checks rows of its choice
+    elif last_row_only:
+        refs = [_last_row_attention(q.double(), k.double(), v.double(), scale, window) for q, k, v in zip(qs, ks, vs)]
+    else:
+        refs = [P.attention_core(q.double(), k.double(), v.double(), scale, window)[p0:]
+                for q, k, v, p0 in zip(qs, ks, vs, step.pos0)]
+    return out.cpu().double().view(-1, nh, hd), (torch.cat(refs) if refs else (qs, ks)), vs
+
+
+def _last_row_attention(q, k, v, scale, window):
+    """The last position's attention alone, as a library softmax over its keys: what the whole
+    table of scores would cost too much for at tens of thousands of keys.  q [L, nh, hd], k, v [L, nkv, hd]."""
+    L, nh, _ = q.shape
+    group = nh // k.shape[1]
+    first = max(0, L - window) if window is not None else 0
+    out = torch.empty(1, nh, v.shape[-1], dtype=torch.float64)
+    for h in range(nh):
+        scores = (k[first:, h // group] @ q[L - 1, h]) * scale
+        out[0, h] = torch.softmax(scores, 0) @ v[first:, h // group]
+    return out
 
 
 @pytest.mark.parametrize("decode", [True, False])
@@ -578,6 +596,36 @@ def test_attn_mfma_long_sequences_split_over_workgroups(K, decode):
     assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
     got, ref, _ = _mfma_attn_case(K, 4, 2, 128, [2500, 1031], 1024, 0.05, decode, seed=4)
     assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,lens,window", [(8, 4, 256, [20000, 9001, 100], None), (8, 4, 256, [20000, 9001], 1024),
+                                                   (5, 1, 80, [33000], None), (2, 2, 64, [70000, 3], 4097)])
+def test_attn_mfma_decode_over_tens_of_thousands_of_keys(K, nh, nkv, hd, lens, window):
+    """Hundreds of pages a sequence, beside a short one: every share of the pages and their merge,
+    with key 3 made to win in one pass (the furthest key there is) and random scores in the other."""
+    g = torch.Generator().manual_seed(2)
+    q, k, v = (torch.randn(9, n, 8, generator=g).double() for n in (4, 2, 2))
+    for w in (None, 5):                                     # the helper is the plain function's last row
+        assert torch.allclose(_last_row_attention(q, k, v, 0.3, w), P.attention_core(q, k, v, 0.3, w)[-1:], atol=1e-12)
+    got, ref, _ = _mfma_attn_case(K, nh, nkv, hd, lens, window, 0.3 * (16 / hd) ** 0.5, True, seed=11, last_row_only=True)
+    assert torch.isfinite(got).all()
+    assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
+    if window is None:
+        got, ref, vs = _mfma_attn_case(K, nh, nkv, hd, lens, None, 0.5, True, seed=12, boost=3, last_row_only=True)
+        assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
+        assert torch.allclose(got[0, 0], vs[0][3, 0].double(), atol=2e-2)
+
+
+@pytest.mark.parametrize("nh,nkv,hd,L,window", [(4, 2, 128, 20000, None), (8, 4, 256, 9001, 1024), (3, 1, 48, 40000, 5000)])
+def test_attn_mfma_prefill_of_tens_of_thousands_of_tokens(K, nh, nkv, hd, L, window):
+    """A prompt of hundreds of pages in one step; rows at the start, at page edges, in the middle
+    and at the end are compared, each as the last row of the sequence that ends with it."""
+    scale = 0.3 * (16 / hd) ** 0.5
+    got, (qs, ks), vs = _mfma_attn_case(K, nh, nkv, hd, [L], window, scale, False, seed=13, last_row_only=True)
+    assert torch.isfinite(got).all()
+    for r in (0, 63, 64, 1023, 1024, L // 2 + 7, L - 65, L - 1):
+        ref = _last_row_attention(qs[0][:r + 1].double(), ks[0][:r + 1].double(), vs[0][:r + 1].double(), scale, window)
+        assert torch.allclose(got[r:r + 1], ref, atol=2e-2, rtol=2e-2), r
 
 
 @pytest.mark.parametrize("nh,nkv,hd,lens,window", [(4, 2, 128, [1500], None), (4, 2, 128, [1500], 1024),
