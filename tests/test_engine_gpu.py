@@ -148,6 +148,37 @@ def test_long_decoding(engine_of):
         assert g.pool.n_free == g.pool.n_pages
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_context_of_thousands_of_tokens(tmp_path, dtype):
+    """Dozens of pages a sequence and a window that reaches over two dozen of them: the prompt
+    whole, then in three pieces beside a short request, then further tokens one by one; the
+    long dot products of attention over thousands of keys are where a lost page would show."""
+    from agave_amd.engine import Engine
+    cfg = dict(P.tiny_config("C"))
+    cfg["sliding_window"] = 1500
+    weights = P.random_weights(cfg, 5)
+    folder = U.write_model(str(tmp_path / "m"), cfg, weights)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=2, max_context=4224)
+    long_req = U.random_tokens(4200, cfg["vocab_size"], 7)
+    short_req = U.random_tokens(70, cfg["vocab_size"], 8)
+    ref = U.plain_logits(cfg, weights, long_req)
+    check = close(dtype)
+    kw = dict(longer_sums=8.0) if dtype == "float32" else {}
+    check(U.run_whole(eng, long_req[:4100]), ref[:4100], "whole", **kw)
+    slots = [eng.alloc_slot(), eng.alloc_slot()]
+    got = []
+    for lo, hi, slo, shi in ((0, 2048, 0, 30), (2048, 4095, 30, 31), (4095, 4160, 31, 70)):
+        lg = eng.step(slots, [long_req[lo:hi], short_req[slo:shi]], "all").float().cpu()
+        got.append(lg[:hi - lo].clone())
+    eng.free_slot(slots[1])
+    for t in long_req[4160:]:
+        got.append(eng.step(slots[:1], [[t]], "all").float().cpu().clone())
+    eng.free_slot(slots[0])
+    check(torch.cat(got, 0), ref, "pieces, then one by one", **kw)
+    for g in eng.cache.groups:
+        assert g.pool.n_free == g.pool.n_pages
+
+
 def test_prompt_in_pieces(engine_of):
     """Steps of several tokens that start in the middle of a sequence (a prompt that enters in
     pieces): pieces that end on a page's edge, one short of it and one past it, for two
