@@ -675,16 +675,18 @@ def test_gemm_tiled(G, m, n, k, out_dtype):
     assert float((out.cpu().double() - ref).abs().max()) <= tol
 
 
-@pytest.mark.parametrize("m,n,k", [(2048, 2560, 10240),     # 160 tiles of 128 x 256: three slices
-                                   (4096, 2560, 10240),     # 160 tiles of 256 x 256: one product
-                                   (2000, 2552, 10248),     # the same tiles, ragged edges
-                                   (2048, 2560, 2048),      # few columns: one product
-                                   (300, 200, 4096)])       # small tiles: one product
-def test_gemm_tiled_in_slices(G, m, n, k):
+@pytest.mark.parametrize("m,n,k,slices", [
+    (2048, 2560, 10240, 3),     # 160 tiles of 128 x 256: three slices, which run as 240 tiles of 256 x 256
+    (4096, 2560, 10240, 1),     # 160 tiles of 256 x 256: one product
+    (2000, 2552, 10248, 3),     # ragged edges
+    (8192, 640, 10240, 3),      # 160 tiles of 128 x 256 whose slices in 256 x 256 would be 288: they stay 480 of 128 x 256
+    (2048, 2560, 2048, 1),      # few columns: one product
+    (300, 200, 4096, 1)])       # small tiles: one product
+def test_gemm_tiled_in_slices(G, m, n, k, slices):
     """A product of many tokens whose tiles fill the compute units badly comes as 32-bit slices
     that add up to it, for a reader that adds them."""
     z = G.tiled_slices_for(m, n, k)
-    assert z == (3 if k >= 10240 and m <= 2048 else 1)
+    assert z == slices
     if z == 1:
         return
     g = torch.Generator().manual_seed(m + n + k)
