@@ -123,7 +123,10 @@ __device__ void block_argmax(const float* __restrict__ x, int n, float mult, flo
 // radix selection of the value of the (at most 1024) largest entries in three rounds of
 // histograms (11, 11 and 10 bits of the ordered key), and the collection of those entries; last,
 // one workgroup per row decides.  With a filter the kept entries are among the collected ones,
-// which are sorted by value (thresholds) and then by index (the draw).  Without one the piece that
+// which are sorted by value (thresholds) and then by index (the draw).  Entries above the value
+// of the 1024th largest are collected first and its equals behind them as far as there is room, so
+// that a plateau of equal logits can only leave out its own kind; if it does, the thresholds are
+// still exact and the draw walks the whole row with them.  Without a filter the piece that
 // holds u * sum is found from the pieces' sums and only that piece is read again.
 // Words of scratch per row:
 #define SP_PARTS 64
