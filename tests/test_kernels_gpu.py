@@ -375,6 +375,35 @@ def test_sample_with_more_equal_logits_than_the_filter_collects(S, vocab, temper
     assert got == want
 
 
+def test_sample_random_parameters_ties_and_masked_halves(S):
+    """A sweep of random rows and parameters, some rows with a seventh of their entries equal and
+    some with their upper half at -inf, six rows a batch with mixed kinds; every draw must be the
+    plain rule's (a u within 1e-4 of an interval's edge may go to the neighbour)."""
+    rng = np.random.default_rng(0)
+    checked = 0
+    for trial in range(48):
+        vocab = int(rng.choice([4096, 5003, 40013]))
+        g = torch.Generator().manual_seed(trial)
+        lg = torch.randn(6, vocab, generator=g) * float(rng.choice([0.5, 2.0, 6.0]))
+        if trial % 3 == 0:
+            lg[:, ::7] = lg[:, 3:4]
+        if trial % 4 == 0:
+            lg[:, vocab // 2:] = float("-inf")
+        params = [[float(rng.choice([0.0, 0.3, 0.8, 1.0, 1.7])), int(rng.choice([0, 0, 1, 5, 40, 1000, 1024, 5000])),
+                   float(rng.choice([1.0, 1.0, 0.95, 0.7, 0.3, 0.01])), float(rng.random())] for _ in range(6)]
+        got = _sample(S, lg, params)
+        for b, (t, k, p, u) in enumerate(params):
+            want = P.sample_token(lg[b], t, k, p, u)
+            if got[b] != want:
+                w = P.sample_distribution(lg[b], t, k, p)
+                assert t > 0 and float(w[got[b]]) > 0, (trial, b, params[b], got[b], want)
+                cdf = torch.cumsum(w, 0) / w.sum()
+                edges = [float(cdf[got[b]])] + ([float(cdf[got[b] - 1])] if got[b] else [])
+                assert min(abs(e - u) for e in edges) < 1e-4, (trial, b, params[b], got[b], want)
+            checked += 1
+    assert checked == 48 * 6
+
+
 def test_sample_frequencies_follow_softmax(S):
     lg = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]])
     n = 4000
