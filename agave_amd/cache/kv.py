@@ -140,6 +140,40 @@ class KVCache:
             plans.append(GroupPlan(base, rows))
         return pos0, plans
 
+    def check_pieces(self, slots: Sequence[int], pieces: Sequence[Sequence[int]]) -> None:
+        """Raise, changing nothing, unless a step that is run as several steps one after another
+        fits as a whole.  ``pieces[j][i]`` is the number of tokens that ``slots[i]`` brings in
+        the j-th of them (0: it takes no part).  Every sequence must stay within the context, and
+        in every group the pages held at the fullest moment must be there: a windowed group
+        gives pages back between the pieces, a group that needs all keys does not."""
+        if len(set(slots)) != len(slots):
+            raise CacheError("a slot appears twice in one step")
+        lengths = []
+        for i, s in enumerate(slots):
+            self.slots.check(s)
+            cur = self.slots.length[s]
+            total = sum(int(p[i]) for p in pieces)
+            if cur + total > self.max_context:
+                raise CacheError(f"slot {s}: {cur} + {total} positions exceed the context of {self.max_context}")
+            lengths.append(cur)
+        for g in self.groups:
+            held = [set(g.held(s)) for s in slots]
+            there = g.pool.n_free + sum(len(h) for h in held)
+            lens = list(lengths)
+            for piece in pieces:
+                for i, n in enumerate(piece):
+                    if n > 0:
+                        held[i].update(range(lens[i] // PAGE, (lens[i] + n - 1) // PAGE + 1))
+                need = sum(len(h) for h in held)
+                if need > there:
+                    raise OutOfPages(f"step needs {need - there} more cache pages of group {g.key} than the "
+                                     f"{g.pool.n_free} that are free of {g.pool.n_pages}")
+                for i, n in enumerate(piece):
+                    if n > 0:
+                        lens[i] += n
+                        keep_from = g._first_needed(lens[i])
+                        held[i] = {x for x in held[i] if x >= keep_from}
+
     def commit_step(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
         for s, n in zip(slots, n_new):
             self.slots.length[s] += n

@@ -101,6 +101,25 @@ class GroupKey:
     head_dim: int
 
 
+def pages_in_reach(window: Optional[int], max_context: int, max_new: int = 1) -> int:
+    """Most pages one sequence holds in a group while a step brings it up to ``max_new`` tokens,
+    for sequences of at most ``max_context`` positions.  A group that needs all keys holds the
+    whole context.  A window of W reaches back W - 1 positions from the step's first token, so
+    the step spans W + max_new - 1 positions, which touch at most one page more than they fill."""
+    full = (max_context + PAGE - 1) // PAGE
+    if window is None:
+        return full
+    return min(full, (window + max_new - 1 + PAGE - 2) // PAGE + 1)
+
+
+def pool_pages(window: Optional[int], max_slots: int, max_context: int, piece: int) -> int:
+    """Pages a group's pool needs so that ``max_slots`` sequences of up to ``max_context``
+    positions always fit when no step brings a sequence more than ``piece`` tokens: all keys of
+    every sequence for a group without a window, only the window's reach plus the step's own
+    tokens for a windowed one (what the reference's ring of W rows per sliding layer bounds)."""
+    return max_slots * pages_in_reach(window, max_context, max(1, min(piece, max_context)))
+
+
 class GroupPages:
     """The pages of one group: for every slot a map from page index (position // 64) to
     page id."""
@@ -119,11 +138,7 @@ class GroupPages:
     def table_width(self, max_context: int, max_new: int = 1) -> int:
         """Columns that a step's table needs at most for sequences up to ``max_context``
         positions when a step brings up to ``max_new`` tokens per sequence."""
-        full = (max_context + PAGE - 1) // PAGE
-        if self.key.window is None:
-            return full
-        reach = (self.key.window + max_new - 1 + PAGE - 2) // PAGE + 1
-        return min(full, reach)
+        return pages_in_reach(self.key.window, max_context, max_new)
 
     def plan(self, slot: int, pos0: int, n_new: int) -> Tuple[int, List[int]]:
         """Make sure pages exist for positions ``pos0 .. pos0+n_new-1`` and return

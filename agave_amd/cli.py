@@ -22,9 +22,6 @@ import sys
 import time
 from typing import List, Optional
 
-DEFAULT_CTX = 4096          # src/main.zig:107
-
-
 def parse_ids(text: str) -> List[int]:
     parts = [p for p in re.split(r"[\s,]+", text.strip()) if p]
     try:
@@ -107,21 +104,15 @@ def main(argv: Optional[List[str]] = None) -> int:
         with open(args.random_weights) as f:
             write_random_model(json.load(f), args.seed or 0, args.model)
 
-    from .config import load_config
     from .engine import Engine
     from .engine.generate import GenerationStats
     from .sampling import SamplingParams
 
-    _, cfg = load_config(args.model)
-    model_ctx = getattr(cfg, "max_position_embeddings", DEFAULT_CTX)
-    if args.ctx_size is None:
-        ctx = min(model_ctx, DEFAULT_CTX)
-    elif args.ctx_size == 0:
-        ctx = model_ctx
-    else:
-        ctx = args.ctx_size
+    if args.ctx_size is not None and args.ctx_size < 0:
+        ap.error("--ctx-size must be >= 0")
     t0 = time.perf_counter()
-    engine = Engine.from_folder(args.model, dtype=args.dtype, max_slots=max(1, args.max_batch), max_context=ctx)
+    engine = Engine.from_folder(args.model, dtype=args.dtype, max_slots=max(1, args.max_batch),
+                                max_context=args.ctx_size)     # None: min(model, 4096); 0: the model's
     load_ms = (time.perf_counter() - t0) * 1e3
     if args.model_info:
         info = model_info(engine)

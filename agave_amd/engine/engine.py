@@ -18,14 +18,17 @@ import os
 
 import torch
 
-from ..cache import PAGE, GroupKey, KVCache
+from ..cache import PAGE, GroupKey, KVCache, pool_pages
 from ..config import find_architecture, read_config_json
 from ..config.spec import ModelSpec
 from ..parts import BuildEnv, Workspace
 from ..weights import Checkpoint, DictWeightSource, RandomWeightSource, WeightSource
 from .graphs import DecodeGraphs, span_bucket
 from .model import Model, tensor_needs
-from .step import Step, StepPlanner, Want
+from .step import Step, StepPlanner, Want, resolve_want, split_pieces
+
+DEFAULT_CONTEXT = 4096      # the reference's default context (src/main.zig:107, 1100-1113)
+DEFAULT_PIECE = 4096        # tokens a sequence brings at most in one run of the model
 
 _DTYPES = {"float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
            "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
@@ -52,10 +55,16 @@ def require_gpu(device=None) -> torch.device:
 class Engine:
     def __init__(self, spec: ModelSpec, weights, *, dtype="bfloat16", max_slots: int = 8,
                  max_context: Optional[int] = None, cache_tokens: Optional[int] = None,
-                 device=None, config=None):
-        """``max_context``: longest sequence a slot may hold (default: the model's).
+                 prefill_piece: Optional[int] = None, device=None, config=None):
+        """``max_context``: longest sequence a slot may hold; None: the smaller of the model's
+        context and 4096, 0: the model's whole context (the reference's ``--ctx-size``,
+        ``src/main.zig:1100-1113``, ``src/models/gemma3.zig:164-166``).
         ``cache_tokens``: positions the cache holds over all live sequences, each counted
-        rounded up to a multiple of 64 (default: ``max_slots * max_context``)."""
+        rounded up to a multiple of 64 (default: ``max_slots * max_context``).
+        ``prefill_piece``: most tokens of one sequence that the model runs at a time (default
+        4096); a longer prompt enters in pieces.  Layers with a window keep only the window's
+        reach plus one piece per sequence, so their share of the cache does not grow with
+        the context."""
         self.device = require_gpu(device)
         self.dtype = parse_dtype(dtype)
         self.spec = spec
@@ -71,20 +80,26 @@ class Engine:
         self.workspace = Workspace(self.device)
         self.env = BuildEnv(self.dtype, self.device, self.workspace)
         self.model = Model(spec, weights, self.env)
-        self.max_context = int(max_context) if max_context else int(spec.max_context)
+        if max_context is None:
+            self.max_context = min(int(spec.max_context), DEFAULT_CONTEXT)
+        else:
+            self.max_context = int(max_context) if int(max_context) > 0 else int(spec.max_context)
         if self.max_context < 1:
             raise ValueError("max_context must be positive")
-        per_seq = (self.max_context + PAGE - 1) // PAGE
-        if cache_tokens is None:
-            n_pages = max_slots * per_seq
-        else:
-            n_pages = max(1, (int(cache_tokens) + PAGE - 1) // PAGE)
+        self.max_piece = min(self.max_context, int(prefill_piece) if prefill_piece else DEFAULT_PIECE)
+        if self.max_piece < 1:
+            raise ValueError("prefill_piece must be positive")
         kv_needs = self.model.kv_needs()
-        pages: Dict[GroupKey, int] = {key: n_pages for key in set(kv_needs.values())}
+        pages: Dict[GroupKey, int] = {}
+        for key in set(kv_needs.values()):
+            # what max_slots sequences can hold at most; fewer if the caller bounds the live positions
+            pages[key] = pool_pages(key.window, max_slots, self.max_context, self.max_piece)
+            if cache_tokens is not None:
+                pages[key] = min(pages[key], max(1, (int(cache_tokens) + PAGE - 1) // PAGE))
         self.cache = KVCache(kv_needs, self.model.state_needs(), max_slots, pages, self.dtype, self.device,
                              self.max_context)
         self.planner = StepPlanner(self.cache, spec.vocab_size, self.device, self.workspace)
-        self.prefill_chunk = 0          # > 0: prompts enter in pieces of at most this many tokens
+        self.prefill_chunk = 0          # > 0: prompts enter in pieces of at most this many tokens (at most max_piece)
         self.use_graphs = os.environ.get("AGAVE_AMD_NO_GRAPHS", "") not in ("1", "true", "yes")
         self.graphs = DecodeGraphs(self)
         self._decode_widths = [g.table_width(self.max_context, 1) for g in self.cache.groups]
@@ -163,7 +178,54 @@ class Engine:
         return self._run(slots, tokens, want)[0]
 
     def _run(self, slots, tokens, want, carry=None, floats=None):
-        """Plan, run and commit one step; (logits, step)."""
+        """Run one step of the caller's; (logits, the last planned step).  A step in which a
+        sequence brings more tokens than a piece holds runs as several steps of the model, the
+        last of which holds every sequence; the logits come back in the caller's order."""
+        piece = min(self.max_piece, int(self.prefill_chunk)) if int(self.prefill_chunk or 0) > 0 else self.max_piece
+        n_new = [len(t) for t in tokens]
+        if n_new and max(n_new) > piece and len(slots) == len(tokens) and min(n_new) >= 1:
+            return self._run_in_pieces(slots, tokens, want, piece, floats)
+        return self._run_one(slots, tokens, want, carry, floats)
+
+    def _run_in_pieces(self, slots, tokens, want, piece, floats):
+        n_new = [len(t) for t in tokens]
+        wanted = resolve_want(want, n_new)
+        pieces = split_pieces(n_new, piece)
+        self.cache.check_pieces(list(slots), pieces)       # all or nothing, before the first piece runs
+        # where every wanted row of the caller's order comes from: (piece, row among that piece's wanted rows)
+        first_row = [0]
+        for w in wanted:
+            first_row.append(first_row[-1] + len(w))
+        total = first_row[-1]
+        done = [0] * len(slots)
+        result = None
+        gathered = None
+        for j, counts in enumerate(pieces):
+            idx = [i for i, c in enumerate(counts) if c > 0]
+            sub_tokens = [tokens[i][done[i]:done[i] + counts[i]] for i in idx]
+            sub_want, dest = [], []
+            for i in idx:
+                lo, hi = done[i], done[i] + counts[i]
+                places = [(k, x - lo) for k, x in enumerate(wanted[i]) if lo <= x < hi]
+                sub_want.append([x for _, x in places])
+                dest += [first_row[i] + k for k, _ in places]
+            last = j == len(pieces) - 1
+            logits, step = self._run_one([slots[i] for i in idx], sub_tokens, sub_want, None, floats if last else None)
+            for i in idx:
+                done[i] += counts[i]
+            if logits is None:
+                continue
+            if last and len(dest) == total:
+                result = logits                             # everything wanted lies in the last piece, in order
+            else:
+                if gathered is None:
+                    gathered = self.workspace.get("logits_gathered", total, self.spec.vocab_size, torch.float32)
+                gathered.index_copy_(0, torch.tensor(dest, dtype=torch.int64, device=self.device), logits)
+                result = gathered
+        return (result if total else None), step
+
+    def _run_one(self, slots, tokens, want, carry=None, floats=None):
+        """Plan, run and commit one step of the model; (logits, step)."""
         step = self.planner.plan(slots, tokens, want, decode_widths=self._decode_widths if self.use_graphs else None,
                                  carry=carry, floats=floats)
         if carry is not None:
@@ -210,16 +272,6 @@ class Engine:
             if any(r.repeat_penalty != 1.0 for r in rows):
                 raise ValueError("launch_step: the repeat penalty needs the tokens on the host; no carry")
             tokens = [[0]] * b
-        chunk = int(self.prefill_chunk or 0)
-        if chunk > 0 and max(len(t) for t in tokens) > chunk:
-            # the reference feeds a prompt in chunks (src/models/gemma3.zig:385-391); only the
-            # last piece of each sequence needs logits
-            tokens = [list(t) for t in tokens]
-            while max(len(t) for t in tokens) > chunk:
-                idx = [i for i, t in enumerate(tokens) if len(t) > chunk]
-                self.step([slots[i] for i in idx], [tokens[i][:chunk] for i in idx], "none")
-                for i in idx:
-                    tokens[i] = tokens[i][chunk:]
         params = np.asarray([[r.temperature, float(min(r.top_k, 1 << 20)), r.top_p, r.u] for r in rows],
                             dtype=np.float32)
         logits, step = self._run(slots, tokens, "last", carry=carry, floats=params)

@@ -97,6 +97,25 @@ def resolve_want(want: Want, n_new: Sequence[int]) -> List[List[int]]:
     return out
 
 
+def split_pieces(n_new: Sequence[int], piece: int) -> List[List[int]]:
+    """How a step whose sequences bring ``n_new[i]`` tokens runs when no sequence may bring more
+    than ``piece`` at a time: while a sequence has more than ``piece`` tokens left, those that do
+    run their next ``piece`` tokens together; the last step holds every sequence with what it
+    has left (at least one token, at most ``piece``).  Returns the token counts of each step in
+    turn (0: the sequence takes no part in it).  The reference feeds a prompt in chunks the same
+    way, one sequence at a time (``src/models/gemma3.zig:385-391``)."""
+    if piece < 1:
+        raise StepError("a step's pieces hold at least one token")
+    left = [int(n) for n in n_new]
+    out: List[List[int]] = []
+    while max(left) > piece:
+        now = [piece if n > piece else 0 for n in left]
+        out.append(now)
+        left = [n - k for n, k in zip(left, now)]
+    out.append(left)
+    return out
+
+
 class StepPlanner:
     """Turns (slots, tokens, want) into a :class:`Step`: checks the request, takes cache
     pages, and uploads the step's description in one copy."""

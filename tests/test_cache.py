@@ -154,3 +154,70 @@ def test_table_width():
     g = GroupPages(GroupKey(1024, 1, 8), 64, 2)
     assert g.table_width(4096) == 17 and g.table_width(512) == 8
     assert GroupPages(GroupKey(None, 1, 8), 64, 2).table_width(4096) == 64
+
+
+def test_pool_sizes_follow_each_group_reach():
+    from agave_amd.cache import pages_in_reach, pool_pages
+    # all keys: the whole context of every slot
+    assert pool_pages(None, 8, 131072, 4096) == 8 * 2048
+    # a window of 1024 and pieces of 4096: 1024 + 4095 positions touch at most 81 + 1 pages
+    assert pages_in_reach(1024, 131072, 4096) == (1024 + 4096 - 1 + 62) // 64 + 1 == 81
+    assert pool_pages(1024, 8, 131072, 4096) == 8 * 81
+    # never more than the context itself, and a piece is never longer than the context
+    assert pool_pages(1024, 8, 4096, 4096) == 8 * 64 and pool_pages(1024, 3, 512, 99999) == 3 * 8
+    # decoding only: the window's reach
+    assert pages_in_reach(1024, 131072, 1) == 17 and pages_in_reach(16, 64, 1) == 1
+    # every alignment of a step inside its pages fits the bound, and one alignment reaches it
+    for window, piece in ((16, 1), (70, 5), (100, 130), (1024, 64)):
+        bound = pages_in_reach(window, 10 ** 6, piece)
+        spans = []
+        for pos0 in range(0, 4 * 64 + window):
+            lo = max(0, pos0 - window + 1) // PAGE
+            spans.append((pos0 + piece - 1) // PAGE - lo + 1)
+        assert max(spans) == bound
+
+
+def test_published_sizes_fit_one_gpu_at_the_whole_context():
+    """Gemma 3 27B at 131,072 positions and 8 slots: the windowed layers' share does not grow
+    with the context."""
+    from agave_amd.cache import pool_pages
+    layers, pattern, nkv, hd, window = 62, 6, 16, 128, 1024
+    n_window = sum(1 for i in range(layers) if (i + 1) % pattern)
+    page_bytes = 2 * 64 * nkv * hd * 2                       # K and V, bfloat16
+    full = (layers - n_window) * pool_pages(None, 8, 131072, 4096) * page_bytes
+    win = n_window * pool_pages(window, 8, 131072, 4096) * page_bytes
+    assert n_window == 52 and full == 10 * 16384 * page_bytes
+    assert win == 52 * 8 * 81 * page_bytes and (full + win) / 2 ** 30 < 100
+    same_as_full = layers * pool_pages(None, 8, 131072, 4096) * page_bytes
+    assert same_as_full / 2 ** 30 > 490
+
+
+def test_a_step_in_pieces_is_checked_as_a_whole():
+    from agave_amd.engine.step import split_pieces
+    assert split_pieces([5, 300, 128, 129], 128) == [[0, 128, 0, 128], [0, 128, 0, 0], [5, 44, 128, 1]]
+    assert split_pieces([7], 128) == [[7]] and split_pieces([256], 128) == [[128], [128]]
+    W = 70
+    full, win = GroupKey(None, 1, 8), GroupKey(W, 1, 8)
+    # the windowed pool holds the window's reach plus a piece of 128 for two slots, no more
+    from agave_amd.cache import pool_pages
+    n_win = pool_pages(W, 2, 2048, 128)
+    c = KVCache({0: win, 1: full}, {}, 2, {win: n_win, full: 40}, torch.float32, None, 2048)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    with pytest.raises(OutOfPages):
+        c.check_pieces([a, b], [[1500, 900]])                  # as one piece the windowed pool is too small
+    pieces = split_pieces([1500, 900], 128)
+    c.check_pieces([a, b], pieces)
+    for counts in pieces:                                      # and the pieces do run, one after another
+        idx = [i for i, n in enumerate(counts) if n]
+        c.plan_step([[a, b][i] for i in idx], [counts[i] for i in idx])
+        c.commit_step([[a, b][i] for i in idx], [counts[i] for i in idx])
+    assert c.length(a) == 1500 and c.length(b) == 900
+    with pytest.raises(CacheError, match="context"):
+        c.check_pieces([a], split_pieces([600], 128))
+    # a group that needs all keys counts every piece: 24 of its 40 pages are held, 1100 positions need 18
+    c.free_slot(b)
+    b = c.alloc_slot()
+    free_before = [g.pool.n_free for g in c.groups]
+    with pytest.raises(OutOfPages):
+        c.check_pieces([b], split_pieces([1100], 128))
+    assert [g.pool.n_free for g in c.groups] == free_before and c.length(b) == 0

@@ -334,3 +334,92 @@ def test_sizes_that_fit_no_fast_kernel(tmp_path, dtype):
     outs = U.run_batched(eng, [toks, toks[:70], toks[:9]], (90, 69, 1))
     for o, n in zip(outs, (130, 70, 9)):
         close(dtype)(o, ref[:n], f"batched, {n} tokens")
+
+
+def test_default_arguments_bound_the_context_and_each_group_s_pool(tmp_path):
+    """An engine built with nothing but the folder takes the smaller of the model's context and
+    4096 (the reference's default), 0 takes the model's, and each group's storage is as large as
+    its reach says: the whole context for layers that need all keys, the window plus a piece for
+    the others."""
+    from agave_amd.cache import PAGE, pool_pages
+    from agave_amd.engine import Engine
+    cfg = dict(P.tiny_config("C"), max_position_embeddings=131072)
+    folder = U.write_model(str(tmp_path / "m"), cfg, P.random_weights(cfg, 1))
+    eng = Engine.from_folder(folder)
+    assert eng.max_context == 4096 and eng.max_slots == 8 and eng.dtype == torch.bfloat16
+    assert Engine.from_folder(folder, max_context=1000, max_slots=1).max_context == 1000
+    del eng
+    eng = Engine.from_folder(folder, max_context=0, max_slots=3, prefill_piece=512)
+    assert eng.max_context == 131072 and eng.max_piece == 512
+    kinds = cfg["layer_types"]
+    for key, k_store, v_store, group in zip(eng.cache.group_keys, eng.cache.k_store, eng.cache.v_store, eng.cache.groups):
+        n_mem = sum(1 for t in kinds if (t == "sliding_attention") == (key.window is not None))
+        want = pool_pages(key.window, 3, 131072, 512)
+        assert want == (3 * 2048 if key.window is None else 3 * ((70 + 511 + 62) // 64 + 1))
+        assert group.pool.n_pages == want and k_store.shape[:2] == (n_mem, want) and v_store.shape[:2] == (n_mem, want)
+    nkv, hd = cfg["num_key_value_heads"], cfg["head_dim"]
+    per_page = nkv * PAGE * (64 + hd) * 2            # bfloat16; K rows of 48 are padded to whole tiles of 32 columns
+    assert eng.cache.bytes() == per_page * (2 * 3 * 2048 + 3 * 3 * 11)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_through_a_small_window_pool(tmp_path, dtype):
+    """One call brings a prompt of 4,200 tokens and a short one while the windowed layers' pool
+    holds five pages a sequence: the engine runs the call in pieces, gives pages back between
+    them, and returns the wanted rows of all pieces in the caller's order."""
+    from agave_amd.engine import Engine
+    cfg = dict(P.tiny_config("C"))
+    weights = P.random_weights(cfg, 6)
+    folder = U.write_model(str(tmp_path / "m"), cfg, weights)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=2, max_context=4224, prefill_piece=128)
+    win = [g for g in eng.cache.groups if g.key.window is not None][0]
+    assert win.pool.n_pages == 2 * 5
+    long_req = U.random_tokens(4200, cfg["vocab_size"], 9)
+    short_req = U.random_tokens(131, cfg["vocab_size"], 10)
+    ref_long, ref_short = U.plain_logits(cfg, weights, long_req), U.plain_logits(cfg, weights, short_req)
+    want_long = [0, 127, 128, 1000, 1001, 4095, 4096, 4199]
+    want_short = [5, 130]
+    check = close(dtype)
+    kw = dict(longer_sums=8.0) if dtype == "float32" else {}
+    slots = [eng.alloc_slot(), eng.alloc_slot()]
+    got = eng.step(slots, [long_req, short_req], [want_long, want_short]).float().cpu()
+    check(got[:len(want_long)], ref_long[want_long], "long request", **kw)
+    check(got[len(want_long):], ref_short[want_short], "short request", **kw)
+    assert len(win.held(slots[0])) <= 5 and eng.kv_seq_len(slots[0]) == 4200
+    # a call that cannot fit is refused before any piece has run
+    from agave_amd.cache import CacheError
+    with pytest.raises(CacheError):
+        eng.step(slots, [long_req[:200], short_req], "last")
+    assert eng.kv_seq_len(slots[0]) == 4200 and eng.kv_seq_len(slots[1]) == 131
+    for s in slots:
+        eng.free_slot(s)
+    # everything wanted in the last piece: the common case of a prompt whose last logits are wanted
+    slot = eng.alloc_slot()
+    got = eng.step([slot], [long_req[:1000]], "last").float().cpu()
+    check(got, ref_long[999:1000], "last row", **kw)
+    eng.free_slot(slot)
+    for g in eng.cache.groups:
+        assert g.pool.n_free == g.pool.n_pages
+
+
+def test_the_27b_sizes_at_the_whole_context_fit_the_gpu():
+    """Gemma 3 27B's own configuration with random weights, 8 slots of 131,072 positions: the
+    windowed layers' pool does not grow with the context, so the cache is some 100 GB and the engine
+    constructs; a short batch then runs through tables that are 2,048 pages wide."""
+    import bench
+    from agave_amd.cache import pool_pages
+    from agave_amd.engine import Engine
+    eng = Engine.from_random(bench.GEMMA3_27B, seed=0, dtype="bfloat16", max_slots=8, max_context=131072)
+    page = 2 * 16 * 64 * 128 * 2
+    want = page * (10 * pool_pages(None, 8, 131072, 4096) + 52 * pool_pages(1024, 8, 131072, 4096))
+    assert eng.cache.bytes() == want and want / 2 ** 30 < 100
+    slots = [eng.alloc_slot(), eng.alloc_slot()]
+    v = eng.vocab_size
+    a = eng.step(slots, [U.random_tokens(70, v, 1), U.random_tokens(3, v, 2)], "last").clone()
+    b = eng.step(slots, [[5], [7]], "last").clone()
+    assert a.shape == (2, v) and bool(torch.isfinite(a).all()) and bool(torch.isfinite(b).all())
+    assert float((a[0] - a[1]).abs().max()) > 0
+    for s in slots:
+        eng.free_slot(s)
+    del eng
+    torch.cuda.empty_cache()
