@@ -10,7 +10,7 @@ quantised caches, vision, speculative decoding, its single-dispatch kernel and g
 counterpart here.  There is no tokenizer in this library: a prompt is a list
 of token ids ("2 17 5" or "2,17,5"), and the output is token ids.
 
-Added: ``--prompt-file`` (one request per line), ``--dtype``, ``--max-batch``, ``--ignore-eos``,
+Added: ``--prompt-file`` (one request per line), ``--dtype``, ``--max-batch``, ``--ignore-eos``, ``--cast-weights``,
 ``--random-weights CONFIG.json`` (write a random model folder at <model> first).
 """
 from __future__ import annotations
@@ -61,6 +61,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-batch", type=int, default=8, help="sequences per batch [default: 8]")
     ap.add_argument("--ignore-eos", action="store_true", help="do not stop at end-of-sequence ids")
     ap.add_argument("--no-bos", action="store_true", help="do not prepend the begin-of-sequence id")
+    ap.add_argument("--cast-weights", action="store_true",
+                    help="cast matrices that the checkpoint stores in 32-bit to the engine's dtype (default: they stay 32-bit)")
     ap.add_argument("--random-weights", metavar="CONFIG.json",
                     help="first write random weights for this configuration into <model> (uses --seed)")
     return ap
@@ -112,6 +114,7 @@ def main(argv: Optional[List[str]] = None) -> int:
         ap.error("--ctx-size must be >= 0")
     t0 = time.perf_counter()
     engine = Engine.from_folder(args.model, dtype=args.dtype, max_slots=max(1, args.max_batch),
+                                keep_stored_precision=not args.cast_weights,
                                 max_context=args.ctx_size)     # None: min(model, 4096); 0: the model's
     load_ms = (time.perf_counter() - t0) * 1e3
     if args.model_info:

@@ -453,6 +453,32 @@ extern "C" int agave_geglu(int dtype, const void* gate, long ldg, const void* up
     return 0;
 }
 
+// ------------------------------------------------------------------ rows of the residual stream, as they are
+// out[i] = h[rows[i]] (rows null: h[i]) in out's element type: what a model without a final norm
+// hands to its output matrix.
+template <typename TO>
+__global__ void gather_rows_kernel(const float* __restrict__ h, const int* __restrict__ rows, TO* __restrict__ out,
+                                   long ldo, int e) {
+    const int i = blockIdx.x;
+    const float* src = h + (size_t)(rows ? rows[i] : i) * e;
+    for (int c = threadIdx.x; c < e; c += blockDim.x) st(out + (size_t)i * ldo + c, src[c]);
+}
+
+extern "C" int agave_gather_rows(int dtype_out, const float* h, const int* rows, void* out, long ldo, int n_rows, int e,
+                                 hipStream_t stream) {
+    AGAVE_CHECK(n_rows >= 0 && e > 0 && ldo >= e, "gather_rows: bad sizes rows=%d e=%d stride=%ld", n_rows, e, ldo);
+    AGAVE_CHECK(h != nullptr && out != nullptr, "gather_rows: null tensor");
+    if (n_rows == 0) return 0;
+    if (dtype_out == AGAVE_F32)
+        gather_rows_kernel<float><<<n_rows, 256, 0, stream>>>(h, rows, (float*)out, ldo, e);
+    else if (dtype_out == AGAVE_BF16)
+        gather_rows_kernel<bf16><<<n_rows, 256, 0, stream>>>(h, rows, (bf16*)out, ldo, e);
+    else
+        AGAVE_CHECK(false, "gather_rows: unknown dtype %d", dtype_out);
+    AGAVE_LAUNCH_CHECK("gather_rows");
+    return 0;
+}
+
 // ------------------------------------------------------------------ casts
 template <typename TI, typename TO>
 __global__ void cast_kernel(const TI* __restrict__ in, TO* __restrict__ out, long n) {

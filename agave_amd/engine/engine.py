@@ -55,7 +55,8 @@ def require_gpu(device=None) -> torch.device:
 class Engine:
     def __init__(self, spec: ModelSpec, weights, *, dtype="bfloat16", max_slots: int = 8,
                  max_context: Optional[int] = None, cache_tokens: Optional[int] = None,
-                 prefill_piece: Optional[int] = None, device=None, config=None):
+                 prefill_piece: Optional[int] = None, keep_stored_precision: bool = True, device=None,
+                 config=None):
         """``max_context``: longest sequence a slot may hold; None: the smaller of the model's
         context and 4096, 0: the model's whole context (the reference's ``--ctx-size``,
         ``src/main.zig:1100-1113``, ``src/models/gemma3.zig:164-166``).
@@ -64,7 +65,11 @@ class Engine:
         ``prefill_piece``: most tokens of one sequence that the model runs at a time (default
         4096); a longer prompt enters in pieces.  Layers with a window keep only the window's
         reach plus one piece per sequence, so their share of the cache does not grow with
-        the context."""
+        the context.
+        ``keep_stored_precision``: in a bfloat16 engine a matrix that the checkpoint stores in
+        32-bit stays in 32-bit (its products then run on the plain multiply-add kernel, far from
+        the matrix cores' speed; a line on standard error says how many do); False casts such
+        matrices to bfloat16 at load.  Half precision is always cast to the engine's type."""
         self.device = require_gpu(device)
         self.dtype = parse_dtype(dtype)
         self.spec = spec
@@ -78,8 +83,13 @@ class Engine:
             needed += ["gemm_mfma", "attention_mfma"]
         library.ensure_built(needed)
         self.workspace = Workspace(self.device)
-        self.env = BuildEnv(self.dtype, self.device, self.workspace)
+        self.env = BuildEnv(self.dtype, self.device, self.workspace, keep_stored_precision=bool(keep_stored_precision))
         self.model = Model(spec, weights, self.env)
+        if self.env.kept_32bit:
+            kept = self.env.kept_32bit
+            library._log(f"{len(kept)} weight matrices are stored in 32-bit and stay so ({', '.join(sorted(set(kept)))}): "
+                         f"their products run on the plain multiply-add kernel, not on the matrix cores; "
+                         f"keep_stored_precision=False (--cast-weights) casts them to bfloat16")
         if max_context is None:
             self.max_context = min(int(spec.max_context), DEFAULT_CONTEXT)
         else:

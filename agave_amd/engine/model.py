@@ -36,10 +36,9 @@ class Model:
         self.spec = spec
         self.env = env
         table = weights.get(spec.embed_weight)
-        if env.dtype == torch.float32 and table.dtype != torch.float32:
-            table = table.to(torch.float32)
-        if table.dtype not in (torch.float32, torch.bfloat16):
-            raise TypeError(f"embedding table has unsupported element type {table.dtype}")
+        keep = env.weight_dtype(table.dtype)
+        if table.dtype != keep:
+            table = table.to(keep)
         self.embed_table: Optional[torch.Tensor] = table.to(env.device).contiguous()
         self.blocks = [lookup("block", layer.kind)(layer, weights, env) for layer in spec.layers]
         self.final_norm = (lookup("norm", spec.final_norm.kind)(spec.final_norm, weights, env)
@@ -104,10 +103,7 @@ class Model:
         if step.n_want == 0:
             return None
         x = ws.get("final_normed", step.n_want, self.spec.hidden, self.env.dtype)
-        if self.final_norm is not None:
-            add_pending_and_norm(h, pending, self.final_norm, x, rows=step.want_rows)
-        else:
-            raise NotImplementedError("a model without a final norm is not supported")
+        add_pending_and_norm(h, pending, self.final_norm, x, rows=step.want_rows)   # no final norm: the rows as they are
         logits = ws.get("logits", step.n_want, self.spec.vocab_size, torch.float32)
         self.head.forward(x, out=logits)
         return logits

@@ -26,6 +26,7 @@ _SIGNATURES = {
                                   _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
         "agave_cast": [_I, _P, _I, _P, _L, _P],
+        "agave_gather_rows": [_I, _P, _P, _P, _L, _I, _I, _P],
     },
     "gemm": {
         "agave_gemm_plain": [_I, _P, _L, _I, _P, _L, _I, _P, _L, _I, _I, _I, _P],
@@ -228,6 +229,20 @@ def geglu(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor) -> None:
         raise ValueError("geglu: gate, up and out must agree in shape and dtype")
     n, ff = gate.shape
     library.call(lib("elementwise"), "agave_geglu", dt(gate), ptr(gate), ldg, ptr(up), ldu, ptr(out), ldo, n, ff, stream())
+
+
+def gather_rows(h: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor) -> None:
+    """out[i] = h[rows[i]] (all rows in order if ``rows`` is None), rounded to out's element type;
+    ``h`` is the 32-bit residual stream.  The caller vouches that the row numbers lie inside ``h``."""
+    _dev(h, rows, out)
+    if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
+        raise ValueError("gather_rows: the source must be a contiguous float32 [rows, hidden] tensor")
+    n = h.shape[0] if rows is None else rows.numel()
+    _i32(rows, "rows")
+    ldo = _rows(out, "out")
+    if out.shape != (n, h.shape[1]):
+        raise ValueError(f"gather_rows: out must be [{n}, {h.shape[1]}], got {tuple(out.shape)}")
+    library.call(lib("elementwise"), "agave_gather_rows", dt(out), ptr(h), ptr(rows), ptr(out), ldo, n, h.shape[1], stream())
 
 
 def cast(src: torch.Tensor, dst: torch.Tensor) -> None:

@@ -7,8 +7,11 @@ the kinds that the layer's spec names.
 
 Interfaces (duck-typed; the classes below document them):
 
-* norm:        ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, fields ``gain`` (float32
-               on the device, any "+1" folded in) and ``eps``; the residual kernels take those.
+* norm:        ``tensor_needs(spec)``, ``__init__(spec, weights, env)``, field ``size``,
+               ``apply(x, out, rows=None)`` (out = norm of the 32-bit rows x, or of the chosen ones),
+               ``add_to(h, branch)`` (h += norm(branch)) and ``add_and_norm(h, pending, out, rows=None)``,
+               which :class:`agave_amd.parts.norm.Norm` composes of the two; blocks and the model's end
+               only ever call the last.
 * position:    ``__init__(spec, env)``, ``fused_rotation() -> (inv_freq | None, pos_scale)`` when the
                q/k kernel can apply it (a rotation of pairs, or nothing), else ``apply(q, k, step)``:
                in place on the normalised rows q [N, heads*head_dim] and k [N, kv_heads*head_dim]
@@ -23,7 +26,7 @@ Interfaces (duck-typed; the classes below document them):
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional
 
 import torch
@@ -35,6 +38,20 @@ class BuildEnv:
     dtype: torch.dtype                 # torch.float32 or torch.bfloat16: activations and cache
     device: torch.device
     workspace: "Workspace"
+    keep_stored_precision: bool = True   # a matrix stored in 32-bit stays so in a bfloat16 engine
+    kept_32bit: List[str] = field(default_factory=list)    # names of the products that therefore miss the matrix cores
+
+    def weight_dtype(self, stored: torch.dtype) -> torch.dtype:
+        """The element type a matrix (or the embedding table) stored as ``stored`` is held in.  A
+        32-bit engine widens everything (exactly).  A bfloat16 engine keeps bfloat16, casts half
+        precision to bfloat16, and keeps 32-bit storage unless it was told to cast that too."""
+        if stored not in (torch.float32, torch.bfloat16, torch.float16):
+            raise TypeError(f"a weight matrix must hold floats (bfloat16, float16 or float32), got {stored}")
+        if self.dtype == torch.float32:
+            return torch.float32
+        if stored == torch.float32 and self.keep_stored_precision:
+            return torch.float32
+        return self.dtype
 
 
 class Workspace:

@@ -6,8 +6,9 @@
 
 ``prenorm`` is the same without the two post norms.  A block never adds its last branch
 itself: it returns it as *pending* ``(branch, norm | None)``, and whoever runs next (the
-next block's first norm, or the model's end) adds it in the same kernel that computes the
-next norm, so the residual stream is read and written once per sublayer.
+next block's first norm, or the model's end) hands it to the norm that comes next
+(``norm.add_and_norm``), which adds it and computes itself, in one kernel where the kinds of
+norm allow it, so that the residual stream is read and written once per sublayer.
 """
 from __future__ import annotations
 
@@ -16,23 +17,22 @@ from typing import List, Optional, Tuple
 import torch
 
 from ..config.spec import LayerSpec
-from ..ops import kernels
 from ..weights.loader import TensorNeed
 from .base import BuildEnv, lookup, register
-
-Pending = Optional[Tuple[torch.Tensor, Optional[object]]]
+from .norm import Pending, add_branch, rows_as_they_are
 
 
 def add_pending_and_norm(h: torch.Tensor, pending: Pending, norm, out: Optional[torch.Tensor],
                          rows: Optional[torch.Tensor] = None) -> None:
-    """h += post(branch) for a pending branch, then out = norm(h) if asked."""
-    branch, post = pending if pending is not None else (None, None)
-    if rows is not None and branch is not None:
-        kernels.residual_norm(h, branch, post.gain if post else None, post.eps if post else 0.0, None, None, 0.0)
-        branch = None
-    kernels.residual_norm(h, branch, post.gain if (branch is not None and post) else None,
-                          post.eps if (branch is not None and post) else 0.0,
-                          out, norm.gain if out is not None else None, norm.eps if out is not None else 0.0, rows)
+    """h += post(branch) for a pending branch, then out = norm(h) if asked: the norm that comes
+    next does it (``norm`` None: the branch is added and the rows are handed on as they are)."""
+    if norm is None:
+        if out is not None:
+            rows_as_they_are(h, pending, out, rows)
+        else:
+            add_branch(h, pending)
+    else:
+        norm.add_and_norm(h, pending, out, rows)
 
 
 class SandwichBlock:
@@ -71,12 +71,12 @@ class SandwichBlock:
     def forward(self, h: torch.Tensor, pending: Pending, step, memory: int, writes: bool) -> Pending:
         n = h.shape[0]
         x = self.env.workspace.get("normed", n, self.hidden, self.env.dtype)
-        add_pending_and_norm(h, pending, self.pre_mixer, x)
+        self.pre_mixer.add_and_norm(h, pending, x)
         a = self.mixer.forward(x, step, memory, writes)
         pending = (a, self.post_mixer)
         if self.ffn is None:
             return pending
-        add_pending_and_norm(h, pending, self.pre_ffn, x)
+        self.pre_ffn.add_and_norm(h, pending, x)
         f = self.ffn.forward(x, step)
         return (f, self.post_ffn)
 

@@ -1,10 +1,11 @@
 """A linear map y = W x with W stored row-major [out, in] (``src/backend/backend.zig:474, 481``).
 
-The weight stays in the element type it was stored in, unless the engine runs in 32-bit, in
-which case bfloat16 weights are widened (exactly).  The kernel is chosen by the types: 32-bit
-anything goes through the plain multiply-add kernel; bfloat16 activations with bfloat16
-weights go through the matrix-core kernels, which fall back to the plain kernel for shapes
-they refuse.
+The weight's element type is the build environment's choice (``BuildEnv.weight_dtype``): a
+32-bit engine widens everything (exactly); a bfloat16 engine keeps bfloat16, casts half
+precision to bfloat16, and keeps a matrix that was stored in 32-bit as it is unless told to cast
+it.  The kernel is chosen by the types: 32-bit anything goes through the plain multiply-add
+kernel; bfloat16 activations with bfloat16 weights go through the matrix-core kernels, which
+fall back to the plain kernel for shapes they refuse.
 """
 from __future__ import annotations
 
@@ -26,8 +27,9 @@ class Linear:
         for w in weights:
             if w.dim() != 2:
                 raise ValueError(f"{name}: weight must be a matrix, got {tuple(w.shape)}")
-            if env.dtype == torch.float32 and w.dtype != torch.float32:
-                w = w.to(torch.float32)
+            keep = env.weight_dtype(w.dtype)
+            if w.dtype != keep:
+                w = w.to(keep)
             ws.append(w)
         if len({w.shape[1] for w in ws}) != 1:
             raise ValueError(f"{name}: stacked weights must agree in input size")
@@ -45,6 +47,8 @@ class Linear:
             from ..ops import gemm_mfma
             self.packed = gemm_mfma.pack_weight(self.weight, interleave_ff=interleave_ff)
             self.weight = None      # only the packed copy is kept
+        elif env.dtype == torch.bfloat16 and self.weight.dtype == torch.float32:
+            env.kept_32bit.append(name)
         self.interleave_ff = interleave_ff if self.packed is not None else 0
 
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,

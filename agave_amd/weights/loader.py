@@ -1,33 +1,49 @@
 """Resolving a model's tensors by name, with one error that lists everything wrong.
 
 Reference: the reference looks tensors up lazily on every forward and fails at the first
-missing one (``error.MissingTensor``, ``src/models/gemma3.zig:352, 450``).  Here every part
-of the model states the tensors it needs (name and shape); all of them are checked before
-anything is read, and a single :class:`WeightError` lists the missing names, the names the
-checkpoint holds that no part asked for, and the shapes that do not fit.
+missing one (``error.MissingTensor``, ``src/models/gemma3.zig:352, 450``), and maps a stored
+element type it does not know to ``.unknown`` (``src/format/safetensors.zig:1605-1616``: F32,
+F16 and BF16 are the floating-point types it takes).  Here every part of the model states the
+tensors it needs (name, shape, and whether it holds floats or integers); all of them are
+checked before anything is read, and a single :class:`WeightError` lists the missing names, the
+names the checkpoint holds that no part asked for, the shapes that do not fit and the tensors
+stored in an element type that their use does not take.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, Iterable, List, Sequence, Tuple
+from typing import Dict, Iterable, List, Optional, Sequence, Tuple
 
 import torch
 
 from .safetensors_io import Checkpoint
 
 
+FLOAT_STORAGE = ("BF16", "F16", "F32")                       # what a matrix or vector of floats may be stored as
+INT_STORAGE = ("I64", "I32", "I16", "I8", "U8")              # what an integer table may be stored as
+_STORAGE_OF = {torch.bfloat16: "BF16", torch.float16: "F16", torch.float32: "F32", torch.float64: "F64",
+               torch.int64: "I64", torch.int32: "I32", torch.int16: "I16", torch.int8: "I8", torch.uint8: "U8",
+               torch.bool: "BOOL"}
+
+
 @dataclass(frozen=True)
 class TensorNeed:
     name: str
     shape: Tuple[int, ...]
+    kind: str = "float"         # "float": a matrix or vector of floats; "int": an integer table
+
+    def accepts(self, stored: str) -> bool:
+        return stored in (FLOAT_STORAGE if self.kind == "float" else INT_STORAGE)
 
 
 class WeightError(ValueError):
     def __init__(self, missing: Sequence[str], unexpected: Sequence[str],
-                 wrong_shape: Sequence[Tuple[str, Tuple[int, ...], Tuple[int, ...]]], where: str = ""):
+                 wrong_shape: Sequence[Tuple[str, Tuple[int, ...], Tuple[int, ...]]], where: str = "",
+                 wrong_dtype: Sequence[Tuple[str, str, str]] = ()):
         self.missing = list(missing)
         self.unexpected = list(unexpected)
         self.wrong_shape = list(wrong_shape)
+        self.wrong_dtype = list(wrong_dtype)            # (name, stored as, kind needed)
         lines = [f"weights of {where or 'the model'} do not fit its configuration:"]
         if self.missing:
             lines.append(f"  missing ({len(self.missing)}): " + ", ".join(self.missing))
@@ -36,30 +52,42 @@ class WeightError(ValueError):
         if self.wrong_shape:
             lines.append(f"  wrong shape ({len(self.wrong_shape)}): " + ", ".join(
                 f"{n} is {list(got)}, needs {list(want)}" for n, got, want in self.wrong_shape))
+        if self.wrong_dtype:
+            lines.append(f"  wrong element type ({len(self.wrong_dtype)}): " + ", ".join(
+                f"{n} is stored as {got}, needs one of {'/'.join(FLOAT_STORAGE if kind == 'float' else INT_STORAGE)}"
+                for n, got, kind in self.wrong_dtype))
         super().__init__("\n".join(lines))
 
 
-def check_tensors(have: Dict[str, Tuple[int, ...]], needs: Iterable[TensorNeed], where: str = "") -> None:
-    """Raise one :class:`WeightError` if ``have`` (name -> shape) and ``needs`` differ."""
+def check_tensors(have: Dict[str, Tuple[int, ...]], needs: Iterable[TensorNeed], where: str = "",
+                  stored: Optional[Dict[str, str]] = None) -> None:
+    """Raise one :class:`WeightError` if ``have`` (name -> shape) and ``needs`` differ, or if
+    ``stored`` (name -> the container's name of the element type) holds a type that a tensor's
+    use does not take."""
     needs = list(needs)
     wanted = {n.name for n in needs}
     missing = [n.name for n in needs if n.name not in have]
     unexpected = sorted(n for n in have if n not in wanted)
     wrong = [(n.name, tuple(have[n.name]), tuple(n.shape)) for n in needs
              if n.name in have and tuple(have[n.name]) != tuple(n.shape)]
-    if missing or unexpected or wrong:
-        raise WeightError(missing, unexpected, wrong, where)
+    bad_type = []
+    if stored is not None:
+        bad_type = [(n.name, stored[n.name], n.kind) for n in needs
+                    if n.name in stored and not n.accepts(stored[n.name])]
+    if missing or unexpected or wrong or bad_type:
+        raise WeightError(missing, unexpected, wrong, where, bad_type)
 
 
 class WeightSource:
     """What the model builder reads tensors from: a checked checkpoint."""
 
     def __init__(self, checkpoint: Checkpoint, needs: Iterable[TensorNeed]):
-        check_tensors({n: checkpoint.shape(n) for n in checkpoint.names()}, needs, checkpoint.model_dir)
+        check_tensors({n: checkpoint.shape(n) for n in checkpoint.names()}, needs, checkpoint.model_dir,
+                      stored={n: checkpoint.stored_dtype(n) for n in checkpoint.names()})
         self._ckpt = checkpoint
 
     def get(self, name: str) -> torch.Tensor:
-        """CPU tensor in its kept dtype (bfloat16, float32 or int32)."""
+        """CPU tensor in its kept dtype (bfloat16, float16, float32 or int32)."""
         return self._ckpt.read(name)
 
 
@@ -67,11 +95,21 @@ class DictWeightSource:
     """The same over tensors already in memory (tests, random weights without a folder)."""
 
     def __init__(self, tensors: Dict[str, torch.Tensor], needs: Iterable[TensorNeed], where: str = "dict"):
-        check_tensors({n: tuple(t.shape) for n, t in tensors.items()}, needs, where)
+        check_tensors({n: tuple(t.shape) for n, t in tensors.items()}, needs, where,
+                      stored={n: _STORAGE_OF.get(t.dtype, str(t.dtype)) for n, t in tensors.items()})
         self._tensors = tensors
 
     def get(self, name: str) -> torch.Tensor:
         t = self._tensors[name]
-        if t.dtype in (torch.bfloat16, torch.float32, torch.int32):
+        if t.dtype in (torch.bfloat16, torch.float16, torch.float32, torch.int32):
             return t
-        return t.to(torch.float32 if t.is_floating_point() else torch.int32)
+        return narrow_to_int32(t, name)
+
+
+def narrow_to_int32(t: torch.Tensor, name: str) -> torch.Tensor:
+    """An integer table as int32; values that int32 cannot hold are an error, not a wrap-around."""
+    if t.numel() and t.dtype in (torch.int64, torch.uint8, torch.int16, torch.int8):
+        lo, hi = int(t.min()), int(t.max())
+        if lo < -2 ** 31 or hi > 2 ** 31 - 1:
+            raise ValueError(f"tensor {name!r}: values {lo}..{hi} do not fit the 32-bit integers tables are kept in")
+    return t.to(torch.int32)

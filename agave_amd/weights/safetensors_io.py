@@ -9,8 +9,9 @@ The same checks are made here; every failure is a :class:`SafetensorsError` that
 file and what is wrong with it.
 
 Tensors come back as CPU tensors over the mapped file (no copy): bfloat16 stays bfloat16, a
-tensor stored in 32-bit floats stays so, half precision is widened exactly to 32-bit, and
-integer tables become int32.
+tensor stored in 32-bit floats stays so, half precision stays half precision until the part
+that uses it casts it to the engine's element type, and integer tables become int32 (a value
+that does not fit is an error).
 """
 from __future__ import annotations
 
@@ -44,7 +45,9 @@ def kept_dtype(stored: str) -> torch.dtype:
     """The dtype a stored tensor is kept in after loading."""
     if stored == "BF16":
         return torch.bfloat16
-    if stored in ("F32", "F16", "F64"):
+    if stored == "F16":
+        return torch.float16
+    if stored in ("F32", "F64"):
         return torch.float32
     return torch.int32
 
@@ -168,9 +171,13 @@ class Checkpoint:
     def shape(self, name: str) -> Tuple[int, ...]:
         return self.entries[name].shape
 
+    def stored_dtype(self, name: str) -> str:
+        """The container's name of the element type ("BF16", "F32", ...)."""
+        return self.entries[name].dtype
+
     def read(self, name: str) -> torch.Tensor:
-        """The tensor in its kept dtype, on the CPU.  bfloat16 and 32-bit tensors are views
-        of the mapped file; others are converted."""
+        """The tensor in its kept dtype, on the CPU.  bfloat16, half-precision and 32-bit
+        tensors are views of the mapped file; others are converted."""
         e = self.entries[name]
         stored, _ = _STORED[e.dtype]
         if e.end == e.begin:
@@ -180,7 +187,12 @@ class Checkpoint:
             warnings.simplefilter("ignore", UserWarning)     # the mapping is read-only; nothing writes to it
             t = torch.frombuffer(buf, dtype=stored).reshape(e.shape)
         keep = kept_dtype(e.dtype)
-        return t if t.dtype == keep else t.to(keep)
+        if t.dtype == keep:
+            return t
+        if keep == torch.int32:
+            from .loader import narrow_to_int32
+            return narrow_to_int32(t.to(torch.int64) if t.dtype == torch.bool else t, name)
+        return t.to(keep)
 
 
 def write_safetensors(path: str, tensors: Mapping[str, torch.Tensor]) -> None:

@@ -202,32 +202,102 @@ def test_prompt_in_pieces(engine_of):
         close(dtype)(torch.cat(outs[i], 0), U.plain_logits(cfg, weights, r), f"request {i} in pieces")
 
 
-def test_tensors_stored_in_32_bit_stay_so_in_a_bfloat16_engine(tmp_path):
-    """A checkpoint that stores some matrices and the table in 32-bit (values that bfloat16 cannot
-    hold): the bfloat16 engine keeps them in 32-bit and still gives the plain logits."""
+def _save_folder(folder, cfg, stored):
     from safetensors.torch import save_file
     import json, os
-    from agave_amd.engine import Engine
-    cfg = P.tiny_config("B")
-    weights = P.random_weights(cfg, 7, bf16_exact=False)
-    kept32 = [k for k in weights if k.endswith(("embed_tokens.weight", "q_proj.weight", "down_proj.weight",
-                                                "input_layernorm.weight"))]
-    assert kept32 and any((weights[k].bfloat16().float() != weights[k].float()).any() for k in kept32)
-    stored = {k: (v.float() if k in kept32 else v.bfloat16()).contiguous() for k, v in weights.items()}
-    folder = str(tmp_path / "mixed")
     os.makedirs(folder)
-    save_file(stored, os.path.join(folder, "model.safetensors"))
+    save_file({k: v.contiguous() for k, v in stored.items()}, os.path.join(folder, "model.safetensors"))
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(cfg, f)
-    eng = Engine.from_folder(folder, dtype="bfloat16", max_slots=2, max_context=128)
+    return folder
+
+
+def test_tensors_stored_in_32_bit_stay_so_in_a_bfloat16_engine(tmp_path):
+    """A checkpoint that stores some matrices, a norm and the output matrix in 32-bit, with values
+    that bfloat16 cannot hold: the bfloat16 engine keeps them in 32-bit and gives the plain logits.
+    The output matrix is made so that rounding it would show: every row is the same vector of +-1
+    plus a small part of its own, which bfloat16 drops (its steps near 1 are 2^-8 and 2^-7).  What
+    tells the vocabulary's entries apart then lies in the dropped part alone, so the logits minus
+    their mean over the vocabulary are right only if the 32-bit values took part.  An engine on the
+    same tensors rounded to bfloat16 first matches its own plain logits and not the other's."""
+    from agave_amd.engine import Engine
+    cfg = P.tiny_config("C")                       # untied output matrix
+    weights = P.random_weights(cfg, 7, bf16_exact=False)
+    g = torch.Generator().manual_seed(3)
+    sign = (torch.randint(0, 2, (cfg["hidden_size"],), generator=g) * 2 - 1).double()
+    weights["lm_head.weight"] = sign[None, :] + 0.002 * torch.randn(cfg["vocab_size"], cfg["hidden_size"],
+                                                                     generator=g, dtype=torch.float64)
+    kept32 = [k for k in weights if k.endswith(("lm_head.weight", "q_proj.weight", "down_proj.weight",
+                                                "input_layernorm.weight"))]
+    assert any((weights[k].bfloat16().double() != weights[k].float().double()).any() for k in kept32)
+    stored = {k: (v.float() if k in kept32 else v.bfloat16()) for k, v in weights.items()}
+    rounded = {k: v.bfloat16() for k, v in weights.items()}
     toks = U.random_tokens(70, cfg["vocab_size"], 5)
-    as_stored = {k: v.double() for k, v in stored.items()}
-    ref = U.plain_logits(cfg, as_stored, toks)
-    bf16_close(U.run_whole(eng, toks), ref, "mixed storage, whole")
-    bf16_close(U.run_tail(eng, toks, 20), ref, "mixed storage, tail")
-    # the 32-bit values took part: rounding them to bfloat16 first gives visibly other logits than the engine's
+    ref = U.plain_logits(cfg, {k: v.double() for k, v in stored.items()}, toks)
+    ref_rounded = U.plain_logits(cfg, {k: v.double() for k, v in rounded.items()}, toks)
+
+    def centred(x):
+        x = x.double()
+        return x - x.mean(dim=-1, keepdim=True)
+
+    def apart(a, b):
+        """Largest difference of two sets of centred logits, in units of the first one's spread."""
+        return float(((centred(a) - centred(b)).abs().max(dim=-1).values / centred(a).abs().max(dim=-1).values).max())
+
+    def common_close(got, want, what):
+        """The part that all entries of a row share is a sum of +-x_j over the final row x, which
+        cancels to anything between 0 and a dozen: its error is measured against the length of x
+        (about sqrt(hidden)), not against the sum itself."""
+        err = (got.double().mean(-1) - want.mean(-1)).abs().max()
+        assert float(err) < 0.04 * cfg["hidden_size"] ** 0.5, f"{what}: common part off by {float(err):.3f}"
+
+    assert apart(ref, ref_rounded) > 0.5            # the construction works: rounding changes what is compared
+    eng = Engine.from_folder(_save_folder(str(tmp_path / "mixed"), cfg, stored), dtype="bfloat16", max_slots=2,
+                             max_context=128)
     attn0 = eng.model.blocks[0].mixer
     assert attn0.qkv.packed is None and attn0.qkv.weight.dtype == torch.float32
+    assert eng.model.head.packed is None and eng.model.head.weight.dtype == torch.float32
+    assert eng.model.blocks[0].ffn.gate_up.packed is not None          # stored in bfloat16: on the matrix cores
+    whole, tail = U.run_whole(eng, toks), U.run_tail(eng, toks, 20)
+    common_close(whole, ref, "mixed storage, whole")
+    common_close(tail, ref, "mixed storage, tail")
+    assert apart(ref, whole) < 0.1 and apart(ref, tail) < 0.1
+    del eng
+    eng = Engine.from_folder(_save_folder(str(tmp_path / "rounded"), cfg, rounded), dtype="bfloat16", max_slots=2,
+                             max_context=128)
+    assert eng.model.head.packed is not None
+    got = U.run_whole(eng, toks)
+    common_close(got, ref_rounded, "rounded storage")
+    assert apart(ref_rounded, got) < 0.1 and apart(ref, got) > 0.5
+    del eng
+    # told to cast, the engine on the 32-bit folder behaves as the one on the rounded folder
+    eng = Engine.from_folder(str(tmp_path / "mixed"), dtype="bfloat16", max_slots=2, max_context=128,
+                             keep_stored_precision=False)
+    assert eng.model.head.packed is not None and eng.model.blocks[0].mixer.qkv.packed is not None
+    got = U.run_whole(eng, toks)
+    assert apart(ref_rounded, got) < 0.1 and apart(ref, got) > 0.5
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_a_half_precision_folder_is_cast_to_the_engine_s_type(tmp_path, dtype):
+    """Every tensor stored as F16: a bfloat16 engine casts the matrices to bfloat16 and runs them on
+    the matrix cores, a 32-bit engine widens them exactly."""
+    from agave_amd.engine import Engine
+    cfg = P.tiny_config("C")
+    weights = P.random_weights(cfg, 8)
+    stored = {k: v.half() for k, v in weights.items()}
+    eng = Engine.from_folder(_save_folder(str(tmp_path / "half"), cfg, stored), dtype=dtype, max_slots=2,
+                             max_context=128)
+    qkv = eng.model.blocks[0].mixer.qkv
+    if dtype == "bfloat16":
+        assert qkv.packed is not None and eng.model.head.packed is not None and not eng.env.kept_32bit
+    else:
+        assert qkv.weight.dtype == torch.float32
+    toks = U.random_tokens(70, cfg["vocab_size"], 6)
+    as_held = {k: (v.bfloat16() if dtype == "bfloat16" and v.dim() == 2 else v).double() for k, v in stored.items()}
+    ref = U.plain_logits(cfg, as_held, toks)
+    close(dtype)(U.run_whole(eng, toks), ref, "half-precision storage, whole")
+    close(dtype)(U.run_tail(eng, toks, 20), ref, "half-precision storage, tail")
 
 
 @pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "float32"), ("B", "bfloat16")])
@@ -278,6 +348,10 @@ BIG_LAYERS = {
     # the 4B model's layers: width 2560, 8 query and 4 kv heads of 256, 10240 inner columns, window 1024
     "4b": (dict(hidden_size=2560, num_attention_heads=8, num_key_value_heads=4, head_dim=256, query_pre_attn_scalar=256,
                 intermediate_size=10240, sliding_window=1024), 1060, 1015),
+    # the 12B model's: width 3840, 16 query and 8 kv heads of 256, 15360 inner columns (other cuts of the
+    # row blocks among workgroups than the 4B sizes'); a shorter window, as for the 27B sizes
+    "12b": (dict(hidden_size=3840, num_attention_heads=16, num_key_value_heads=8, head_dim=256,
+                 query_pre_attn_scalar=256, intermediate_size=15360, sliding_window=256), 300, 250),
     # the 27B model's: width 5376, 32 query and 16 kv heads of 128, a scale that is not the head size;
     # a shorter window so that the plain implementation stays quick
     "27b": (dict(hidden_size=5376, num_attention_heads=32, num_key_value_heads=16, head_dim=128,
@@ -289,7 +363,8 @@ BIG_LAYERS = {
 @pytest.mark.parametrize("size", sorted(BIG_LAYERS))
 def test_layers_of_the_published_sizes(tmp_path, dtype, size):
     """Two layers with a published model's own sizes (the second one global with its scaled rope) and
-    a small vocabulary: a prompt that ends just short of the window's reach, then steps across it."""
+    a small vocabulary: a prompt that ends just short of the window's reach, then steps across it;
+    then three requests of unequal lengths as one batch whose shorter ones end earlier."""
     from agave_amd.engine import Engine
     sizes, n_all, n_prompt = BIG_LAYERS[size]
     cfg = dict(P.tiny_config("A"), vocab_size=1536, num_hidden_layers=2, sliding_window_pattern=2, rope_theta=1e6,
@@ -298,7 +373,7 @@ def test_layers_of_the_published_sizes(tmp_path, dtype, size):
     cfg.pop("layer_types", None)
     weights = P.random_weights(cfg, 11)
     folder = U.write_model(str(tmp_path / "m"), cfg, weights)
-    eng = Engine.from_folder(folder, dtype=dtype, max_slots=2, max_context=1152)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=3, max_context=1152)
     toks = U.random_tokens(n_all, cfg["vocab_size"], 12)
     ref = U.plain_logits(cfg, weights, toks)
     first = [0, 1, n_prompt // 2, n_prompt - 2, n_prompt - 1]
@@ -308,10 +383,13 @@ def test_layers_of_the_published_sizes(tmp_path, dtype, size):
         got.append(eng.step([slot], [[t]], "last").float().cpu().clone())
     eng.free_slot(slot)
     rows = first + list(range(n_prompt, len(toks)))
-    if dtype == "float32":
-        f32_close(torch.cat(got, 0), ref[rows], f"{size} layers", longer_sums=sizes["intermediate_size"] / 320)
-    else:
-        bf16_close(torch.cat(got, 0), ref[rows], f"{size} layers")
+    kw = dict(longer_sums=sizes["intermediate_size"] / 320) if dtype == "float32" else {}
+    close(dtype)(torch.cat(got, 0), ref[rows], f"{size} layers", **kw)
+    others = [U.random_tokens(n, cfg["vocab_size"], 13 + i) for i, n in enumerate((150, 67))]
+    outs = U.run_batched(eng, [toks] + others, (n_prompt - 9, 120, 3))
+    close(dtype)(outs[0], ref, f"{size} layers, first of a batch", **kw)
+    for i, (r, o) in enumerate(zip(others, outs[1:])):
+        close(dtype)(o, U.plain_logits(cfg, weights, r), f"{size} layers, request {i + 1} of a batch", **kw)
 
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])

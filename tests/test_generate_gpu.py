@@ -240,3 +240,53 @@ def test_steps_launched_ahead_give_the_tokens_of_steps_run_one_by_one(model_b):
         running, cur = following, k
     got.append(b.finish_step(running))
     assert got == ref
+
+
+def test_repeat_penalty_through_the_engine(model_a):
+    """Requests of one batch with different penalties (one without): every token is the plain
+    argmax of the plain logits after the plain penalty over that request's own generated ids.  The
+    prompts end in a token that greedy decoding repeats, so the penalty changes what comes out."""
+    from agave_amd import Engine, SamplingParams
+    cfg, w, folder = model_a
+    eng = Engine.from_folder(folder, dtype="float32", max_slots=3, max_context=64)
+    prompts = [U.random_tokens(n, 512, 400 + i) for i, n in enumerate((7, 12, 3))]
+    penalties = [1.3, 1.0, 2.5]
+    sps = [SamplingParams(max_tokens=14, repeat_penalty=p, ignore_eos=True) for p in penalties]
+    got = [r.tokens for r in eng.generate(prompts, sps)]
+    free = [r.tokens for r in eng.generate(prompts, SamplingParams(max_tokens=14, ignore_eos=True))]
+    for i, (prompt, pen) in enumerate(zip(prompts, penalties)):
+        toks, out = list(prompt), []
+        for _ in range(14):
+            logits = P.apply_repeat_penalty(P.forward(cfg, w, toks)[-1], out, pen)
+            out.append(P.argmax_first(logits))
+            toks.append(out[-1])
+        assert got[i] == out, f"request {i} with penalty {pen}"
+    assert got[1] == free[1]
+    assert got[0] != free[0] or got[2] != free[2], "the penalty changed nothing: the test proves nothing"
+    # the same requests alone and in another order: the ids and rows of a penalty belong to its request
+    again = [r.tokens for r in eng.generate(prompts[::-1], sps[::-1], max_batch=2)]
+    assert again == got[::-1]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_more_kinds_of_decode_steps_than_graphs_are_kept(model_b, dtype):
+    """Twenty requests with twenty different lengths: the batch shrinks by one request every three
+    steps, so twenty kinds of decode step pass by while four graphs are kept.  Old graphs make room,
+    every kind of step is still recorded, and the tokens are those of an engine without graphs."""
+    from agave_amd import Engine, SamplingParams
+    cfg, w, folder = model_b
+    v = cfg["vocab_size"]
+    a = Engine.from_folder(folder, dtype=dtype, max_slots=20, max_context=128)
+    b = Engine.from_folder(folder, dtype=dtype, max_slots=20, max_context=128)
+    a.graphs.max_graphs = 4
+    b.use_graphs = False
+    prompts = [U.random_tokens(1 + (5 * i) % 23, v, 500 + i) for i in range(20)]
+    sps = [SamplingParams(max_tokens=4 + 3 * i, ignore_eos=True) for i in range(20)]
+    ra = a.generate(prompts, sps)
+    rb = b.generate(prompts, sps)
+    assert [r.tokens for r in ra] == [r.tokens for r in rb]
+    assert all(len(r.tokens) == 4 + 3 * i for i, r in enumerate(ra))
+    kept = list(a.graphs._graphs)
+    assert len(kept) <= 4 and a.graphs.evicted >= 14
+    assert sorted(k[0] for k in kept) == [1, 2, 3, 4], kept          # the batch sizes that ran last
+    assert not b.graphs._graphs

@@ -319,10 +319,11 @@ def test_block_part(dtype, kind):
     out = torch.empty((T, hidden), dtype=b.dtype, device=DEV)
     final_gain = rnd((hidden,), 100, 0.2)
 
-    class Final:
-        gain = (final_gain + 1.0).float().to(DEV)
-        eps = 1e-5
-    add_pending_and_norm(h, pending, Final, out)
+    from agave_amd.config.spec import NormSpec
+    final_spec = NormSpec("rmsnorm", hidden, 1e-5, "final", True)
+    final_needs = lookup("norm", "rmsnorm").tensor_needs(final_spec)
+    final = lookup("norm", "rmsnorm")(final_spec, weights_of({"final": final_gain}, final_needs, dtype), b.env)
+    add_pending_and_norm(h, pending, final, out)
 
     a = plain_attention(spec.mixer, t, P.rms_norm(h0, t["n.0"], 1e-5))
     r = h0 + (P.rms_norm(a, t["n.1"], 1e-5) if kind == "sandwich" else a)

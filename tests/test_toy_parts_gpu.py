@@ -309,3 +309,143 @@ def test_toy_model_generates(toy):
         for _ in range(6):
             seq.append(P.argmax_first(plain_toy(w, seq)[-1]))
         assert list(r.tokens) == seq[len(p):]
+
+
+# ---------------------------------------------------------------- another kind of norm, and no final norm
+def define_centred_norm_model():
+    """A norm that subtracts the mean and has a bias, registered from outside, standing before and
+    after sublayers next to the built-in RMS norm, in a model with or without a final norm."""
+    from agave_amd.config import register_architecture
+    from agave_amd.config.registry import Architecture
+    from agave_amd.config.spec import AttentionSpec, GatedFfnSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec, RunEntry
+    from agave_amd.parts import Norm, register
+    from agave_amd.weights.loader import TensorNeed
+
+    class CentredNorm(Norm):
+        """y = (x - mean(x)) / sqrt(var(x) + eps) * g + b"""
+
+        def __init__(self, spec, weights, env):
+            self.g = weights.get(spec.weight).float().to(env.device)
+            self.b = weights.get(spec.weight + "_bias").float().to(env.device)
+            self.eps, self.size = spec.eps, spec.size
+
+        @staticmethod
+        def tensor_needs(spec):
+            return [TensorNeed(spec.weight, (spec.size,)), TensorNeed(spec.weight + "_bias", (spec.size,))]
+
+        def _norm(self, x):
+            x = x.float()
+            x = x - x.mean(-1, keepdim=True)
+            return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + self.eps) * self.g + self.b
+
+        def apply(self, x, out, rows=None):
+            out.copy_(self._norm(x if rows is None else x[rows.long()]).to(out.dtype))
+
+        def add_to(self, h, branch):
+            h += self._norm(branch.sum(0) if branch.dim() == 3 else branch)
+
+    register("norm", "toy_centred", CentredNorm)
+
+    def rms(name):
+        return NormSpec("rmsnorm", HIDDEN, EPS, name, True)
+
+    def centred(name):
+        return NormSpec("toy_centred", HIDDEN, EPS, name)
+
+    def attention(prefix):
+        return AttentionSpec(kind="attention", hidden=HIDDEN, n_heads=HEADS, n_kv_heads=KV, head_dim=HD,
+                             scale=1.0 / math.sqrt(HD), window=None, position=PositionSpec("rope", HD, THETA, 1.0),
+                             q_proj=prefix + "q", k_proj=prefix + "k", v_proj=prefix + "v", o_proj=prefix + "o")
+
+    def dense(prefix):
+        return GatedFfnSpec(kind="gated_dense", hidden=HIDDEN, intermediate=INTER, activation="gelu_tanh",
+                            gate_proj=prefix + "g", up_proj=prefix + "u", down_proj=prefix + "d")
+
+    def spec_of(cfg, names=None):
+        layers = [
+            LayerSpec("sandwich", attention("l0."), dense("l0."), pre_mixer_norm=rms("l0.n0"),
+                      post_mixer_norm=centred("l0.n1"), pre_ffn_norm=centred("l0.n2"), post_ffn_norm=rms("l0.n3")),
+            LayerSpec("prenorm", attention("l1."), dense("l1."), pre_mixer_norm=centred("l1.n0"), pre_ffn_norm=rms("l1.n2")),
+            LayerSpec("sandwich", attention("l2."), dense("l2."), pre_mixer_norm=rms("l2.n0"),
+                      post_mixer_norm=rms("l2.n1"), pre_ffn_norm=rms("l2.n2"), post_ffn_norm=centred("l2.n3")),
+        ]
+        final = {"none": None, "centred": centred("final"), "rms": rms("final")}[cfg["final_norm"]]
+        return ModelSpec(architecture="ToyNormForCausalLM", vocab_size=VOCAB, hidden=HIDDEN, embed_weight="emb",
+                         embed_scale=1.0, layers=layers, order=[RunEntry(i, i) for i in range(3)], final_norm=final,
+                         head_weight="head", max_context=cfg["max_position_embeddings"], eos_token_ids=())
+
+    register_architecture(Architecture("ToyNormForCausalLM", ("toy_norm",), lambda raw: dict(raw), spec_of))
+    return spec_of
+
+
+def plain_centred_norm_model(w, tokens, final) -> torch.Tensor:
+    W = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    ang = P.rope_angles(torch.arange(T, dtype=torch.float64), HD, THETA, 1.0)
+
+    def rms(x, name):
+        return P.rms_norm(x, W[name], EPS)
+
+    def centred(x, name):
+        x = x - x.mean(-1, keepdim=True)
+        return x / torch.sqrt((x * x).mean(-1, keepdim=True) + EPS) * W[name] + W[name + "_bias"]
+
+    def attn(pre, x):
+        q = P.apply_rope((x @ W[pre + "q"].T).view(T, HEADS, HD), ang)
+        k = P.apply_rope((x @ W[pre + "k"].T).view(T, KV, HD), ang)
+        v = (x @ W[pre + "v"].T).view(T, KV, HD)
+        return P.attention_core(q, k, v, 1.0 / math.sqrt(HD), None).reshape(T, -1) @ W[pre + "o"].T
+
+    def ffn(pre, x):
+        return P.geglu(x, W[pre + "g"], W[pre + "u"], W[pre + "d"])
+
+    h = W["emb"][torch.tensor(tokens)]
+    h = h + centred(attn("l0.", rms(h, "l0.n0")), "l0.n1")
+    h = h + rms(ffn("l0.", centred(h, "l0.n2")), "l0.n3")
+    h = h + attn("l1.", centred(h, "l1.n0"))
+    h = h + ffn("l1.", rms(h, "l1.n2"))
+    h = h + rms(attn("l2.", rms(h, "l2.n0")), "l2.n1")
+    h = h + centred(ffn("l2.", rms(h, "l2.n2")), "l2.n3")
+    if final == "centred":
+        h = centred(h, "final")
+    elif final == "rms":
+        h = rms(h, "final")
+    return h @ W["head"].T
+
+
+@pytest.mark.parametrize("final", ["none", "centred", "rms"])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_norm_of_another_form_and_a_model_without_a_final_norm(tmp_path, dtype, final):
+    """The norm kind is registered here; blocks and the model's end reach every norm through the
+    norm part's own interface, so no file of the framework knows of it.  Without a final norm the
+    output matrix takes the wanted rows of the residual stream as they are."""
+    from safetensors.torch import save_file
+    from agave_amd.engine import Engine
+    from agave_amd.engine.model import tensor_needs
+    cfg = {"architectures": ["ToyNormForCausalLM"], "model_type": "toy_norm", "max_position_embeddings": 256,
+           "final_norm": final}
+    spec = define_centred_norm_model()(cfg)
+    g = torch.Generator().manual_seed(11)
+    w = {}
+    for need in tensor_needs(spec):
+        std = 0.1 if len(need.shape) > 1 else 0.3
+        w[need.name] = (torch.randn(need.shape, generator=g) * std).bfloat16().float()
+    w["emb"] = (w["emb"] * 10).bfloat16().float()
+    assert ("final" in w) == (final != "none") and ("final_bias" in w) == (final == "centred")
+    folder = str(tmp_path)
+    save_file({k: v.bfloat16().contiguous() for k, v in w.items()}, os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=3, max_context=192)
+    assert (eng.model.final_norm is None) == (final == "none")
+    toks = U.random_tokens(90, VOCAB, 2)
+    ref = plain_centred_norm_model(w, toks, final)
+    close(U.run_whole(eng, toks), ref, dtype, "whole")
+    close(U.run_tail(eng, toks, 32), ref, dtype, "last 32 one by one")
+    slot = eng.alloc_slot()
+    some = eng.step([slot], [toks], [[3, 50, 89]]).float().cpu()       # chosen rows only
+    eng.free_slot(slot)
+    close(some, ref[[3, 50, 89]], dtype, "chosen rows")
+    reqs = [U.random_tokens(n, VOCAB, 20 + i) for i, n in enumerate((40, 9, 70))]
+    for i, (r, o) in enumerate(zip(reqs, U.run_batched(eng, reqs, (30, 9, 2)))):
+        close(o, plain_centred_norm_model(w, r, final), dtype, f"request {i} of a batch")

@@ -30,7 +30,8 @@ def test_reader_against_the_safetensors_package(tmp_path):
     assert ck.read("a").dtype == torch.bfloat16 and torch.equal(ck.read("a"), t["a"])
     assert ck.read("b").dtype == torch.float32 and torch.equal(ck.read("b"), t["b"])      # 32-bit stays 32-bit
     assert ck.read("c").dtype == torch.int32 and torch.equal(ck.read("c").long(), t["c"])  # tables as int32
-    assert ck.read("d").dtype == torch.float32 and torch.equal(ck.read("d"), t["d"].float())
+    assert ck.read("d").dtype == torch.float16 and torch.equal(ck.read("d"), t["d"])      # cast where it is used
+    assert [ck.stored_dtype(n) for n in "abcd"] == ["BF16", "F32", "I64", "F16"]
     assert ck.read("e").shape == (0, 4)
 
 
@@ -84,6 +85,62 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     with pytest.raises(WeightError, match="missing"):
         WeightSource(Checkpoint(str(tmp_path)), needs)
     check_tensors({"a": (1,)}, [TensorNeed("a", (1,))])
+
+
+def test_element_types_are_checked_in_the_same_error(tmp_path):
+    """A matrix must be stored as BF16, F16 or F32 (what the reference's loader takes as floats,
+    src/format/safetensors.zig:1605-1616); integers, doubles and booleans in its place are listed by
+    name in the one error, beside whatever else is wrong."""
+    from safetensors.torch import save_file
+    raw, needs = _needs("A")
+    w = {k: v.bfloat16() for k, v in P.random_weights(raw, 0).items()}
+    w["model.layers.0.mlp.up_proj.weight"] = torch.zeros(192, 64, dtype=torch.int32)
+    w["model.layers.1.self_attn.q_norm.weight"] = torch.zeros(32, dtype=torch.int64)
+    w["model.layers.2.mlp.down_proj.weight"] = torch.zeros(64, 192, dtype=torch.float64)
+    w["model.layers.3.self_attn.k_proj.weight"] = w["model.layers.3.self_attn.k_proj.weight"].half()   # fine
+    w["model.layers.3.self_attn.v_proj.weight"] = w["model.layers.3.self_attn.v_proj.weight"].float()  # fine
+    del w["model.norm.weight"]
+    for make in (lambda: DictWeightSource(w, needs),):
+        with pytest.raises(WeightError) as ei:
+            make()
+        e = ei.value
+        assert e.missing == ["model.norm.weight"] and not e.unexpected and not e.wrong_shape
+        assert sorted(e.wrong_dtype) == [("model.layers.0.mlp.up_proj.weight", "I32", "float"),
+                                         ("model.layers.1.self_attn.q_norm.weight", "I64", "float"),
+                                         ("model.layers.2.mlp.down_proj.weight", "F64", "float")]
+        assert "wrong element type (3)" in str(e) and "stored as I64, needs one of BF16/F16/F32" in str(e)
+    save_file({k: v.contiguous() for k, v in w.items()}, str(tmp_path / "model.safetensors"))
+    with pytest.raises(WeightError) as ei:
+        WeightSource(Checkpoint(str(tmp_path)), needs)
+    assert len(ei.value.wrong_dtype) == 3 and ei.value.missing == ["model.norm.weight"]
+    # an integer table is the other kind of need: floats in its place are refused, wide integers are
+    # narrowed only if they fit
+    table = TensorNeed("t", (3,), kind="int")
+    with pytest.raises(WeightError, match="stored as BF16, needs one of I64/I32/I16/I8/U8"):
+        DictWeightSource({"t": torch.zeros(3, dtype=torch.bfloat16)}, [table])
+    ok = DictWeightSource({"t": torch.tensor([1, 2, 2 ** 31 - 1])}, [table]).get("t")
+    assert ok.dtype == torch.int32 and ok.tolist() == [1, 2, 2 ** 31 - 1]
+    with pytest.raises(ValueError, match="do not fit"):
+        DictWeightSource({"t": torch.tensor([1, 2, 2 ** 31])}, [table]).get("t")
+    save_file({"t": torch.tensor([-5, 2 ** 40, 0])}, str(tmp_path / "wide.safetensors"))
+    os.remove(tmp_path / "model.safetensors")
+    with pytest.raises(ValueError, match="do not fit"):
+        Checkpoint(str(tmp_path)).read("t")
+
+
+def test_which_element_type_a_matrix_is_held_in():
+    """32-bit engines widen everything; a bfloat16 engine keeps bfloat16, casts half precision,
+    and keeps 32-bit storage unless told to cast it."""
+    from agave_amd.parts import BuildEnv
+    f32, bf16, f16 = torch.float32, torch.bfloat16, torch.float16
+    env = BuildEnv(bf16, None, None)
+    assert [env.weight_dtype(t) for t in (bf16, f16, f32)] == [bf16, bf16, f32]
+    env = BuildEnv(bf16, None, None, keep_stored_precision=False)
+    assert [env.weight_dtype(t) for t in (bf16, f16, f32)] == [bf16, bf16, bf16]
+    env = BuildEnv(f32, None, None)
+    assert [env.weight_dtype(t) for t in (bf16, f16, f32)] == [f32, f32, f32]
+    with pytest.raises(TypeError):
+        env.weight_dtype(torch.int32)
 
 
 def _raw_file(path, header: bytes, data: bytes = b"", hlen=None):
