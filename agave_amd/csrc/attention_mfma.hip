@@ -899,7 +899,10 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     // The ids of the pages this workgroup goes through, looked up once: a lookup inside the loop
     // is two dependent loads from memory a page, and waiting for them also waits for the next
     // page's loads, which were issued just before and should travel while this page is worked on.
+    // (the array holds a.width ids, a whole table row; the host refuses a step whose reach is wider than
+    // the table, and the bound below keeps the writes inside the array whatever the table says)
     int* pg_ids = reinterpret_cast<int*>(page_lds + (size_t)2 * buf_tiles * 64);
+    if (page_last - page_first >= a.width) page_last = page_first + a.width - 1;
     for (int i = threadIdx.x; i <= page_last - page_first; i += NWV * 64) pg_ids[i] = (int)page_of(a, b, page_first + i);
     __syncthreads();
 

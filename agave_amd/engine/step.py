@@ -22,7 +22,7 @@ from typing import List, Optional, Sequence, Tuple, Union
 import numpy as np
 import torch
 
-from ..cache import KVCache
+from ..cache import PAGE, KVCache, pages_in_reach
 
 Want = Union[str, Sequence[Sequence[int]]]
 
@@ -50,6 +50,7 @@ class Step:
     cu_dev: torch.Tensor            # int32 [B + 1]
     want_rows: torch.Tensor         # int32 [n_want]: rows of the step whose logits are wanted
     tables: List[Tuple[torch.Tensor, torch.Tensor]]   # per cache group: (pages [B, width], base [B])
+    bases_host: List[List[int]]     # per cache group: the host's copy of base
     cache: KVCache
     workspace: object = None
     fixed_span: Optional[int] = None    # a captured decode graph plans its splits for this many pages
@@ -62,18 +63,25 @@ class Step:
         if self.fixed_span is not None:
             span = self.fixed_span
             if window is not None:
-                span = min(span, (window + 62) // 64 + 1)
+                span = min(span, pages_in_reach(window, span * PAGE, 1))
             return max(1, span)
         span = 1
         for p0, n in zip(self.pos0, self.n_new):
             p = p0 + n - 1
             lo = max(0, p - window + 1) if window is not None else 0
-            span = max(span, p // 64 - lo // 64 + 1)
+            span = max(span, p // PAGE - lo // PAGE + 1)
         return span
 
     @property
     def is_decode(self) -> bool:
         return self.max_new == 1
+
+    def base_of(self, base: torch.Tensor) -> Optional[List[int]]:
+        """The host's copy of a group's ``base`` tensor (one of ``tables``), for checks before a launch."""
+        for (_, dev), host in zip(self.tables, self.bases_host):
+            if dev is base:
+                return host
+        return None
 
 
 def resolve_want(want: Want, n_new: Sequence[int]) -> List[List[int]]:
@@ -227,7 +235,8 @@ class StepPlanner:
             max_new=max(n_new), max_len=max(p + k for p, k in zip(pos0, n_new)),
             tokens=view(s_tok), tok_seq=view(s_seq), tok_pos=view(s_pos), slots_dev=view(s_slots),
             pos0_dev=view(s_pos0), cu_dev=view(s_cu), want_rows=view(s_want),
-            tables=[(view(t).view(b, w), view(sb)) for t, sb, w in s_tables], cache=self.cache,
+            tables=[(view(t).view(b, w), view(sb)) for t, sb, w in s_tables],
+            bases_host=[list(p.base) for p in plans], cache=self.cache,
             workspace=self.workspace, tables_start_at_reach=(max(n_new) == 1),
             carry_dev=view(s_carry) if s_carry is not None else None,
             floats_dev=view(s_floats).view(torch.float32) if s_floats is not None else None)

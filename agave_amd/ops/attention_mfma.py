@@ -31,6 +31,21 @@ def split_plan(page_span: int, units: int):
     return -(-page_span // per), per
 
 
+def check_table_reach(pos0, n_new, window: Optional[int], base, width: int) -> None:
+    """Raise unless every sequence's table row covers what its tokens of this step reach: the row's
+    first column (page index ``base[b]``) must not lie after the oldest page a query reaches, and
+    the newest page written must lie inside the row's ``width`` columns.  The prefill kernel keeps
+    a row's ids in an array of ``width`` entries and indexes it by page index minus the first
+    page it needs; a table that is narrower than the reach would send it outside."""
+    for b, (p0, n, b0) in enumerate(zip(pos0, n_new, base)):
+        first = (max(0, p0 - window + 1) if window else 0) // 64
+        last = (p0 + n - 1) // 64
+        if b0 > first:
+            raise ValueError(f"attention: sequence {b}'s table row starts at page {b0}, its queries reach back to page {first}")
+        if last - b0 + 1 > width:
+            raise ValueError(f"attention: sequence {b} reaches pages {b0}..{last}, the table has {width} columns")
+
+
 def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, table: torch.Tensor,
               base: torch.Tensor, step, n_heads: int, n_kv: int, head_dim: int, scale: float,
               window: Optional[int]) -> None:
@@ -43,6 +58,9 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
         raise ValueError("attention: q and out need contiguous rows")
     n_pages = kernels._check_pages(k_pages, v_pages, n_kv, head_dim, q.dtype, packed=True)
     width = kernels._check_table(table, base, step.tok_seq)
+    base_host = getattr(step, "base_of", lambda t: None)(base)
+    if base_host is not None:
+        check_table_reach(step.pos0, step.n_new, window, base_host, width)
     lib = kernels.lib("attention_mfma")
     w = int(window or 0)
     if step.is_decode:

@@ -221,3 +221,17 @@ def test_a_step_in_pieces_is_checked_as_a_whole():
     with pytest.raises(OutOfPages):
         c.check_pieces([b], split_pieces([1100], 128))
     assert [g.pool.n_free for g in c.groups] == free_before and c.length(b) == 0
+
+
+def test_a_table_narrower_than_a_step_s_reach_is_refused_on_the_host():
+    """The prefill kernel indexes a row of page ids by page index; the wrapper refuses a table whose
+    rows do not cover what the step's queries reach, before anything is launched."""
+    from agave_amd.ops.attention_mfma import check_table_reach
+    check_table_reach([0, 130], [200, 1], None, [0, 0], 4)               # pages 0..3 and 0..2
+    check_table_reach([1000], [70], 100, [14], 3)                        # reach 901..1069: pages 14..16
+    with pytest.raises(ValueError, match="columns"):
+        check_table_reach([0], [257], None, [0], 4)                      # page 4 is outside 4 columns
+    with pytest.raises(ValueError, match="reach back"):
+        check_table_reach([1000], [70], 100, [15], 3)                    # the row starts after page 14
+    with pytest.raises(ValueError, match="reach back"):
+        check_table_reach([1000], [1], None, [3], 64)                    # all keys: the row must start at page 0

@@ -501,3 +501,39 @@ def test_the_27b_sizes_at_the_whole_context_fit_the_gpu():
         eng.free_slot(s)
     del eng
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("which", ["A", "B", "4b layer"])
+def test_bfloat16_against_the_32_bit_path(tmp_path, which):
+    """The two paths of one engine on the same folder: how far the bfloat16 logits lie from the 32-bit
+    ones, relative to a row's largest logit, and how often both name the same most likely token.
+    With random weights many rows have two candidates within rounding of each other, so the rate
+    is not 1; where the 32-bit row's winner leads by more than twice the row's error, the
+    bfloat16 row must name it too."""
+    from agave_amd.engine import Engine
+    if which == "4b layer":
+        cfg = dict(P.tiny_config("A"), vocab_size=1536, num_hidden_layers=1, sliding_window_pattern=2, rope_theta=1e6,
+                   rope_local_base_freq=1e4, rms_norm_eps=1e-6, **BIG_LAYERS["4b"][0])
+        cfg.pop("layer_types", None)
+        n = 300
+    else:
+        cfg, n = P.tiny_config(which), 180
+    weights = P.random_weights(cfg, 31)
+    folder = U.write_model(str(tmp_path / "m"), cfg, weights)
+    toks = U.random_tokens(n, cfg["vocab_size"], 32)
+    rows = {}
+    for dtype in ("float32", "bfloat16"):
+        eng = Engine.from_folder(folder, dtype=dtype, max_slots=1, max_context=320)
+        rows[dtype] = U.run_tail(eng, toks, 32).double()
+        del eng
+    f32, bf = rows["float32"], rows["bfloat16"]
+    err = (bf - f32).abs().max(-1).values
+    rel = err / f32.abs().max(-1).values
+    top2 = f32.topk(2, -1).values
+    lead = top2[:, 0] - top2[:, 1]
+    same = bf.argmax(-1) == f32.argmax(-1)
+    rate = float(same.double().mean())
+    print(f"{which}: largest relative error {float(rel.max()):.4f}, mean {float(rel.mean()):.4f}, top-1 agreement {rate:.3f}")
+    assert float(rel.max()) < 0.04
+    assert bool(same[lead > 2 * err].all())
+    assert rate >= 0.9

@@ -550,7 +550,7 @@ class _FakeStep:
         return span
 
 
-def _mfma_attn_case(K, nh, nkv, hd, lens, window, scale, decode, seed=0, boost=None, last_row_only=False):
+def _mfma_attn_case(K, nh, nkv, hd, lens, window, scale, decode, seed=0, boost=None, last_row_only=False, fused=False):
     """Keys and values go into packed pages through the q/k kernel (no norm, no rotation); then
     either every position is a query (prefill) or only each sequence's last one (decode)."""
     from agave_amd.ops import attention_mfma
@@ -584,7 +584,11 @@ def _mfma_attn_case(K, nh, nkv, hd, lens, window, scale, decode, seed=0, boost=N
     step = _FakeStep(lens, (lambda L: L - 1) if decode else (lambda L: 0), window)
     q_sel = torch.cat([q[p0:] for q, p0 in zip(qs, step.pos0)]).reshape(-1, nh * hd).to(DEV)
     out = torch.full_like(q_sel, float("nan"))
-    attention_mfma.attention(q_sel, out, kp, vp, table, base, step, nh, nkv, hd, scale, window)
+    if fused:       # the decode kernel that also takes the new token's q and k: here it appends nothing
+        attention_mfma.decode_fused(q_sel, None, None, out, None, None, 0.0, 0.0, None, 1.0, kp, vp, table, base, step,
+                                    nh, nkv, hd, scale, window)
+    else:
+        attention_mfma.attention(q_sel, out, kp, vp, table, base, step, nh, nkv, hd, scale, window)
     if last_row_only and not decode:
         refs = []                                           # the caller checks rows of its choice
     elif last_row_only:
@@ -671,14 +675,26 @@ def test_attn_mfma_prefill_blocks_shared_among_workgroups(K, nh, nkv, hd, lens, 
     assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("decode", [True, False])
-def test_attn_mfma_far_key_and_window_edge(K, decode):
-    got, ref, vs = _mfma_attn_case(K, 2, 1, 32, [700], None, 0.5, decode, seed=1, boost=3)
+@pytest.mark.parametrize("hd", [32, 64, 128, 256])
+@pytest.mark.parametrize("how", ["decode", "fused decode", "prefill"])
+def test_attn_mfma_far_key_and_window_edge(K, how, hd):
+    """Key 3 of 700 is made to win every score of the last query; a window that ends just before
+    it must lose it and one that just includes it must keep it.  Head size 32 takes the general
+    kernels, 64 to 256 the fast ones (and the decode kernel that also handles the new token)."""
+    if how == "fused decode" and hd == 32:
+        pytest.skip("the fused decode kernel takes head sizes 64, 128 and 256")
+    kw = dict(decode=how != "prefill", fused=how == "fused decode", seed=1, boost=3)
+    scale = 0.5 * (32 / hd) ** 0.5
+    got, ref, vs = _mfma_attn_case(K, 2, 1, hd, [700], None, scale, **kw)
     assert torch.allclose(got[-1, 0], vs[0][3, 0].double(), atol=2e-2)
-    got_w, _, _ = _mfma_attn_case(K, 2, 1, 32, [700], 696, 0.5, decode, seed=1, boost=3)      # key 3 just outside
+    got_w, _, _ = _mfma_attn_case(K, 2, 1, hd, [700], 696, scale, **kw)      # key 3 just outside
     assert not torch.allclose(got_w[-1, 0], vs[0][3, 0].double(), atol=1e-1)
-    got_e, _, _ = _mfma_attn_case(K, 2, 1, 32, [700], 697, 0.5, decode, seed=1, boost=3)      # just inside
+    got_e, _, _ = _mfma_attn_case(K, 2, 1, hd, [700], 697, scale, **kw)      # just inside
     assert torch.allclose(got_e[-1, 0], vs[0][3, 0].double(), atol=2e-2)
+    # the same at a window's edge that falls on a page's edge and one row either side of it
+    for window, inside in ((700 - 64, False), (700 - 63, False), (700 - 3, True), (700 - 4, False)):
+        got_p, _, _ = _mfma_attn_case(K, 2, 1, hd, [700], window, scale, **kw)
+        assert torch.allclose(got_p[-1, 0], vs[0][3, 0].double(), atol=2e-2) == inside, window
 
 
 # the last three shapes take the 128 x 128, 128 x 256 and 256 x 256 tiles, the others the 64 x 128 one; the
