@@ -15,6 +15,7 @@ from __future__ import annotations
 from typing import Dict, List, Optional, Sequence
 
 import os
+import threading
 
 import torch
 
@@ -72,6 +73,7 @@ class Engine:
         matrices to bfloat16 at load.  Half precision is always cast to the engine's type."""
         self.device = require_gpu(device)
         self.dtype = parse_dtype(dtype)
+        self._cancel = threading.Event()
         self.spec = spec
         self.config = config
         torch.cuda.set_device(self.device)
@@ -248,6 +250,18 @@ class Engine:
             logits = self.model.forward(step)
         self.planner.commit(step)
         return logits, step
+
+    # ------------------------------------------------------------------ cancelling from another thread
+    def cancel(self) -> None:
+        """Ask the running :meth:`generate` call to stop after the step that is under way (the
+        reference's ``cancel``, ``src/models/model.zig:238-241``).  Safe to call from any thread."""
+        self._cancel.set()
+
+    def cancel_requested(self) -> bool:
+        return self._cancel.is_set()
+
+    def clear_cancel(self) -> None:
+        self._cancel.clear()
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.device)

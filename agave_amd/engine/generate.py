@@ -5,7 +5,11 @@ Reference (one sequence): ``generateAndPrintInner`` (``src/main.zig:2118-2461``)
 token comes from the prompt's last logits (``:2290-2294``), then up to ``max_tokens - 1``
 further steps (``:2342``); the repeat penalty covers every id generated so far (``:2350-2352``);
 an end-of-generation id stops the sequence and is not emitted (``:2366-2369``); a full cache
-ends it too (``KVCacheFull``, ``src/models/gemma3.zig:332``).  The reference's "halt after six
+ends it too (``KVCacheFull``, ``src/models/gemma3.zig:332``).  Another thread may cancel the
+call (the reference's ``cancelled`` flag, looked at between layers: ``src/models/gemma3.zig:141,
+342``; here between steps): a backend with ``cancel_requested()`` is asked before every step, and
+a cancelled call returns what it has, every unfinished request with the reason "cancelled".  The
+reference's "halt after six
 equal tokens" (``src/main.zig:2400-2407``) changes outputs and is not taken over.
 
 The loop's decisions need no GPU: it talks to a *backend* with ``max_context``, ``max_slots``,
@@ -95,6 +99,9 @@ def generate(backend, prompts: Sequence[Sequence[int]],
         return RowSampling(p.temperature, p.top_k, p.top_p, p.repeat_penalty, u, results[i].tokens)
 
     ahead = hasattr(backend, "launch_step") and all(p.repeat_penalty == 1.0 for p in plist)
+    cancel_requested = getattr(backend, "cancel_requested", lambda: False)
+    if hasattr(backend, "clear_cancel"):
+        backend.clear_cancel()              # a request to cancel belongs to the call it arrived in
 
     def settle(i: int, tok: int) -> None:
         """Book the token request i drew; sets its finish reason if it ends here."""
@@ -110,6 +117,8 @@ def generate(backend, prompts: Sequence[Sequence[int]],
                 r.finish_reason = "context"               # no room to feed this token
 
     while queue:
+        if cancel_requested():
+            break
         batch, queue = queue[:max_batch], queue[max_batch:]
         stats.batches += 1
         slots = {i: backend.alloc_slot() for i in batch}
@@ -118,7 +127,7 @@ def generate(backend, prompts: Sequence[Sequence[int]],
         first = True
         try:
             if not ahead:
-                while live:
+                while live and not cancel_requested():
                     t0 = time.perf_counter()
                     sampled = backend.step_sample([slots[i] for i in live], feed, [row(i) for i in live])
                     ms = (time.perf_counter() - t0) * 1e3
@@ -146,7 +155,7 @@ def generate(backend, prompts: Sequence[Sequence[int]],
             stats.prefill_tokens += sum(len(f) for f in feed)
             while True:
                 # who goes on unless the running step draws an end token: known beforehand
-                on = [i for i in live if not results[i].finish_reason
+                on = [i for i in live if not results[i].finish_reason and not cancel_requested()
                       and len(results[i].tokens) + 1 < plist[i].max_tokens
                       and results[i].prompt_tokens + len(results[i].tokens) + 1 <= backend.max_context]
                 following = None
@@ -176,4 +185,8 @@ def generate(backend, prompts: Sequence[Sequence[int]],
         finally:
             for s in slots.values():
                 backend.free_slot(s)
+    if cancel_requested():
+        for r in results:
+            if not r.finish_reason:
+                r.finish_reason = "cancelled"
     return results

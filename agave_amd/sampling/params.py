@@ -40,4 +40,5 @@ class GenerationResult:
     prompt_tokens: int
     tokens: List[int] = field(default_factory=list)
     finish_reason: str = ""          # "stop" (an end token was drawn; it is not emitted),
-                                     # "length" (max_tokens), "context" (the slot is full)
+                                     # "length" (max_tokens), "context" (the slot is full),
+                                     # "cancelled" (the call was cancelled before the request ended)

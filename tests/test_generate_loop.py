@@ -203,3 +203,40 @@ def test_command_line_options_follow_the_reference():
     assert parse_ids("2, 17  5") == [2, 17, 5]
     with pytest.raises(SystemExit):
         parse_ids("hello")
+
+
+@pytest.mark.parametrize("backend_cls", [FakeBackend, AheadBackend])
+def test_a_cancelled_call_returns_what_it_has_and_loses_no_slot(backend_cls):
+    """The reference's cancel flag (src/models/gemma3.zig:141, 342), looked at between steps: requests
+    that had ended keep their reason, the others and those still queued end as "cancelled"."""
+    class Cancellable(backend_cls):
+        def __init__(self, after, *a, **kw):
+            super().__init__(*a, **kw)
+            self.after, self.flag, self.cleared = after, False, 0
+
+        def cancel_requested(self):
+            return self.flag
+
+        def clear_cancel(self):
+            self.flag = False
+            self.cleared += 1
+
+        def step_sample(self, slots, tokens, rows):
+            out = super().step_sample(slots, tokens, rows)
+            if len(self.steps) == self.after:
+                self.flag = True                      # as if another thread had called cancel() during this step
+            return out
+
+    be = Cancellable(4, max_slots=2, max_context=64)
+    be.flag = True                                    # left over from an earlier call: does not count
+    res = generate(be, [[10], [20], [30]], [SamplingParams(max_tokens=2), SamplingParams(max_tokens=30),
+                                            SamplingParams(max_tokens=30)], eos_ids=[])
+    assert be.cleared == 1
+    assert res[0].finish_reason == "length" and res[0].tokens == [11, 12]
+    assert res[1].finish_reason == "cancelled" and res[1].tokens[:3] == [21, 22, 23] and len(res[1].tokens) in (4, 5)
+    assert res[2].finish_reason == "cancelled" and res[2].tokens == []         # never started
+    assert be.length == {} and sorted(be.free) == [0, 1] and len(be.steps) <= 5
+    # without a cancel the same call runs to its end
+    be = Cancellable(10 ** 9, max_slots=2, max_context=64)
+    res = generate(be, [[10], [20]], SamplingParams(max_tokens=6), eos_ids=[])
+    assert [r.finish_reason for r in res] == ["length", "length"]
