@@ -21,6 +21,7 @@
 #include "common_impl.h"
 #include "mfma.h"
 #include "qk_rope.h"
+#include "noalloc.h"
 #include <math.h>
 
 #define QT_MAX 4        // most q tiles (of 16 query slots) a wave takes
@@ -1038,6 +1039,13 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
 }
 
 // ------------------------------------------------------------------ host side
+// The partial results of the entry point that allocates nothing (noalloc.h).  In host code this
+// name is a stand-in, not a device address: host code only ever uses the address that
+// hipGetSymbolAddress gives for the current device, kept per device below.
+static __device__ __align__(256) float scratch[AGAVE_NOALLOC_SCRATCH_FLOATS];
+#define AGAVE_MAX_DEVICES 64
+static float* g_scratch_on_device[AGAVE_MAX_DEVICES] = {};
+
 static int check_common(const char* who, const AttnArgs& a, int N) {
     AGAVE_CHECK(N >= 0 && a.nh > 0 && a.nkv > 0 && a.hd > 0, "%s: bad sizes N=%d nh=%d nkv=%d hd=%d", who, N, a.nh, a.nkv, a.hd);
     AGAVE_CHECK(a.nh % a.nkv == 0, "%s: %d query heads are not a multiple of %d kv heads", who, a.nh, a.nkv);
@@ -1047,6 +1055,23 @@ static int check_common(const char* who, const AttnArgs& a, int N) {
     AGAVE_CHECK(a.q && a.out && a.k_pages && a.v_pages && a.table && a.base && a.tok_seq && a.tok_pos && a.width > 0 &&
                     a.n_pages > 0, "%s: null buffer or empty table", who);
     AGAVE_CHECK(a.window >= 0, "%s: negative window", who);
+    return 0;
+}
+
+// More than the default allowance of LDS for large groups of heads; set once.
+static int raise_decode_lds_allowance() {
+    static bool raised = false;
+    if (raised) return 0;
+    const void* fns[] = {(const void*)attn_decode_mfma_kernel<4>, (const void*)attn_decode_mfma_kernel<8>,
+                         (const void*)attn_decode_mfma_kernel<16>,
+                         (const void*)attn_decode_fast_kernel<4, false>, (const void*)attn_decode_fast_kernel<8, false>,
+                         (const void*)attn_decode_fast_kernel<16, false>,
+                         (const void*)attn_decode_fast_kernel<4, true>, (const void*)attn_decode_fast_kernel<8, true>,
+                         (const void*)attn_decode_fast_kernel<16, true>};
+    for (const void* fn : fns)
+        AGAVE_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) == hipSuccess,
+                    "attn_decode_mfma: cannot raise the LDS allowance");
+    raised = true;
     return 0;
 }
 
@@ -1064,19 +1089,7 @@ static int launch_decode(const AttnArgs& a, const QkFuse& f, int N, hipStream_t 
     size_t lds = ((size_t)4 * slots * hd + 4 * 16 * 2) * sizeof(float);
     if (FUSED) lds += (size_t)4 * hd * sizeof(float) + (size_t)16 * hd * sizeof(bf16);
     AGAVE_CHECK(lds <= 96 * 1024, "attn_decode_mfma: %zu bytes of LDS exceed what a workgroup may take", lds);
-    static bool raised = false;
-    if (!raised) {               // more than the default allowance of LDS for large groups of heads
-        const void* fns[] = {(const void*)attn_decode_mfma_kernel<4>, (const void*)attn_decode_mfma_kernel<8>,
-                             (const void*)attn_decode_mfma_kernel<16>,
-                             (const void*)attn_decode_fast_kernel<4, false>, (const void*)attn_decode_fast_kernel<8, false>,
-                             (const void*)attn_decode_fast_kernel<16, false>,
-                             (const void*)attn_decode_fast_kernel<4, true>, (const void*)attn_decode_fast_kernel<8, true>,
-                             (const void*)attn_decode_fast_kernel<16, true>};
-        for (const void* fn : fns)
-            AGAVE_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024) == hipSuccess,
-                        "attn_decode_mfma: cannot raise the LDS allowance");
-        raised = true;
-    }
+    if (raise_decode_lds_allowance()) return -1;
     if (FUSED) {
         AGAVE_CHECK(hd == 64 || hd == 128 || hd == 256, "attn_decode_fused: head_dim %d is not 64, 128 or 256", hd);
         if (hd == 64) attn_decode_fast_kernel<4, true><<<grid, 256, lds, stream>>>(a, f);
@@ -1106,6 +1119,59 @@ extern "C" int agave_attn_decode_mfma(const void* q, long ldq, void* out, long l
                table, width, base, n_pages, tok_seq, tok_pos, nullptr, 0, nh, nkv, hd, scale, window, splits,
                pages_per_split, seq_is_token, table_from_reach};
     if (check_common("attn_decode_mfma", a, N)) return -1;
+    return launch_decode<false>(a, QkFuse{}, N, stream);
+}
+
+// The address of `scratch` on the current device, looked up once per device (every GPU holds
+// its own copy of the array at its own address).
+static int scratch_of_current_device(float** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    AGAVE_CHECK(e == hipSuccess, "attn_noalloc: hipGetDevice failed: %s", hipGetErrorString(e));
+    AGAVE_CHECK(dev >= 0 && dev < AGAVE_MAX_DEVICES, "attn_noalloc: device %d is outside 0..%d", dev, AGAVE_MAX_DEVICES - 1);
+    if (!g_scratch_on_device[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        AGAVE_CHECK(e == hipSuccess && p != nullptr, "attn_noalloc: hipGetSymbolAddress failed on device %d: %s", dev,
+                    hipGetErrorString(e));
+        g_scratch_on_device[dev] = (float*)p;
+    }
+    *out = g_scratch_on_device[dev];
+    return 0;
+}
+
+extern "C" int agave_attn_noalloc_init(void) {
+    float* p = nullptr;
+    if (scratch_of_current_device(&p)) return -1;
+    return raise_decode_lds_allowance();
+}
+
+extern "C" int agave_attn_decode_mfma_noalloc(const void* q, long ldq, void* out, long ldo, const void* k_pages,
+                                              const void* v_pages, const int* table, int width, const int* base,
+                                              int n_pages, const int* tok_seq, const int* tok_pos, int N, int nh,
+                                              int nkv, int hd, float scale, int window, int splits,
+                                              int pages_per_split, int seq_is_token, int table_from_reach,
+                                              hipStream_t stream) {
+    AGAVE_CHECK(N >= 0 && nh > 0 && hd > 0 && splits >= 1, "attn_decode_mfma_noalloc: bad sizes N=%d nh=%d hd=%d splits=%d",
+                N, nh, hd, splits);
+    float* part_o = nullptr;
+    float* part_ml = nullptr;
+    if (splits > 1) {
+        const unsigned long long slots = (unsigned long long)N * nh * splits;
+        const unsigned long long need = slots * ((unsigned long long)hd + 2);
+        AGAVE_CHECK(need <= AGAVE_NOALLOC_SCRATCH_FLOATS,
+                    "attn_decode_mfma_noalloc: %d tokens x %d heads x %d splits x (%d + 2) = %llu floats exceed the "
+                    "library's %u; use agave_attn_decode_mfma with buffers of your own",
+                    N, nh, splits, hd, need, (unsigned)AGAVE_NOALLOC_SCRATCH_FLOATS);
+        float* mine = nullptr;
+        if (scratch_of_current_device(&mine)) return -1;
+        part_o = mine;                                  // [token][head][split][hd]
+        part_ml = mine + slots * hd;                    // [token][head][split][2]
+    }
+    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
+               table, width, base, n_pages, tok_seq, tok_pos, nullptr, 0, nh, nkv, hd, scale, window, splits,
+               pages_per_split, seq_is_token, table_from_reach};
+    if (check_common("attn_decode_mfma_noalloc", a, N)) return -1;
     return launch_decode<false>(a, QkFuse{}, N, stream);
 }
 

@@ -21,7 +21,7 @@ import time
 from typing import Dict, Iterable, List, Optional
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
-HEADERS = ("common.h", "common_impl.h", "mfma.h", "qk_rope.h")
+HEADERS = ("common.h", "common_impl.h", "mfma.h", "qk_rope.h", "noalloc.h")
 ARCH = "gfx950"
 # Packed 32-bit float instructions are switched off for all device code.
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
