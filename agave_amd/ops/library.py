@@ -27,7 +27,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-shared", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
 
-LIBRARIES = ("elementwise", "gemm", "gemm_mfma", "attention_plain", "attention_mfma", "sampling")
+LIBRARIES = ("elementwise", "gemm", "gemm_mfma", "attention_plain", "attention_mfma", "sampling", "peaks")
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

@@ -9,7 +9,16 @@ has the layer sizes of the published Gemma 3 4B text configuration, a batch of 8
 256 decoded tokens per sequence (W warm-up steps, then K timed ones).  One JSON line is
 printed: ``value`` is decoded tokens a second; ``prefill`` is one 2,048-token prompt;
 ``roofline`` prices the decode step by the bytes it has to read (every weight once, and the
-cache of the live requests) against 8 TB/s; ``points`` holds decode at batch 1 and 64.
+cache of the live requests) against 8 TB/s; ``points`` holds decode at batch 1 and 64;
+``peaks_measured`` is what this machine delivered to a streaming read and to a loop of
+matrix-core instructions on random data a moment before (the fractions stay against the
+published peaks).
+
+The other published shapes:
+
+    python bench.py --model 12b --ragged 16 --context 8192        # 16 prompts of unequal lengths 64..4096
+    python bench.py --model 27b --prompt-len 2048 --context 8192 --batch 1 --no-points
+    python bench.py --model 27b --prompt-len 2048 --context 8192 --batch 32 --no-points
 """
 from __future__ import annotations
 
@@ -68,6 +77,13 @@ def decode_step_bytes(m: dict, contexts) -> float:
     return float(weights + kv)
 
 
+def measured_peaks():
+    """What the machine delivers just now: a streaming read of 2 GiB and a loop of bfloat16
+    matrix-core instructions on normally distributed operands (the published peak holds for zeros)."""
+    from agave_amd.ops import peaks
+    return {"hbm_read_gbs": round(peaks.hbm_read_gbs(), 1), "mfma_bf16_tflops": round(peaks.mfma_bf16_tflops(), 1)}
+
+
 def prefill_flops(m: dict, t: int) -> float:
     """Multiply-adds of one prompt of t tokens, twice: the linear layers on every token, the
     output matrix on the one wanted row, and attention over the visible pairs."""
@@ -85,16 +101,45 @@ def random_prompts(n: int, length: int, vocab: int, seed: int):
     return [rng.integers(0, vocab, size=length).tolist() for _ in range(n)]
 
 
-def run_decode(engine, batch: int, steps: int, warmup: int, seed: int, prompt_len: int = PROMPT_LEN):
-    """Prefill ``batch`` prompts of ``prompt_len`` tokens, then time ``steps`` decode steps."""
+def ragged_lengths(n: int, lo: int, hi: int, seed: int):
+    """n prompt lengths drawn uniformly from lo..hi, the two ends among them."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(lo, hi + 1, size=n).tolist()
+    if n >= 2:
+        lens[0], lens[-1] = lo, hi
+    return lens
+
+
+def run_decode(engine, batch: int, steps: int, warmup: int, seed: int, prompt_len: int = PROMPT_LEN, lengths=None,
+               first_step=None):
+    """Prefill ``batch`` prompts of ``prompt_len`` tokens (or of the given unequal ``lengths``, then
+    as one ragged step whose time goes into ``first_step``), then time ``steps`` decode steps."""
+    import numpy as np
     import torch
     from agave_amd.engine.generate import RowSampling
-    prompts = random_prompts(batch, prompt_len, engine.vocab_size, seed)
+    if lengths is None:
+        prompts = random_prompts(batch, prompt_len, engine.vocab_size, seed)
+    else:
+        rng = np.random.default_rng(seed)
+        prompts = [rng.integers(0, engine.vocab_size, size=n).tolist() for n in lengths]
+    plens = [len(p) for p in prompts]
     slots = [engine.alloc_slot() for _ in range(batch)]
     rows = [RowSampling(0.0, 0, 1.0, 1.0, 0.0, []) for _ in range(batch)]
     try:
-        engine.prefill_chunk = 2048 if batch > 8 else 0
-        if batch > 8:                       # keep the untimed prefill's workspace small
+        engine.prefill_chunk = 2048 if (batch > 8 and lengths is None) else 0
+        if lengths is not None:             # the unequal prompts in one step, as a batch starts
+            engine.step_sample(slots, prompts, rows)            # once untimed: libraries, workspace
+            for s in slots:
+                engine.free_slot(s)
+            slots[:] = [engine.alloc_slot() for _ in range(batch)]
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            toks = engine.step_sample(slots, prompts, rows)
+            torch.cuda.synchronize()
+            if first_step is not None:
+                first_step.update(tokens=sum(plens), ms=round((time.perf_counter() - t0) * 1e3, 3))
+        elif batch > 8:                     # keep the untimed prefill's workspace small
             toks = None
             for i in range(0, batch, 8):
                 part = engine.step_sample(slots[i:i + 8], prompts[i:i + 8], rows[i:i + 8])
@@ -116,8 +161,8 @@ def run_decode(engine, batch: int, steps: int, warmup: int, seed: int, prompt_le
         toks = engine.finish_step(running)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        first_ctx = prompt_len + warmup + 1          # keys the first timed step attends to
-        contexts = [first_ctx + (steps - 1) / 2.0] * batch
+        # keys the first timed step attends to: the prompt, the warm-up steps' tokens and its own
+        contexts = [n + warmup + 1 + (steps - 1) / 2.0 for n in plens]
         return dt, contexts
     finally:
         for s in slots:
@@ -159,6 +204,9 @@ def main() -> int:
                     help="tokens of every prompt before the decode steps (the default run: 1024)")
     ap.add_argument("--context", type=int, default=CONTEXT, help="longest sequence a slot may hold")
     ap.add_argument("--prefill-len", type=int, default=PREFILL_LEN, help="tokens of the prefill prompt (the default run: 2048)")
+    ap.add_argument("--ragged", type=int, default=0, metavar="N",
+                    help="N prompts of unequal lengths 64..4096 (seeded) as one first step, then decode steps; "
+                         "replaces --batch and --prompt-len")
     ap.add_argument("--no-points", action="store_true", help="skip prefill and the batch 1 / 64 points")
     ap.add_argument("--prefill-only", action="store_true",
                     help="time only the 2048-token prefill and print its record (for profiles)")
@@ -168,6 +216,10 @@ def main() -> int:
         if int(os.environ.get("RANK", "0")) == 0:
             print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    lengths = None
+    if args.ragged:
+        lengths = ragged_lengths(args.ragged, 64, min(4096, args.context // 2), seed=7)
+        args.batch, args.prompt_len, args.no_points = args.ragged, max(lengths), True
     if args.steps + args.warmup > args.context - args.prompt_len:
         ap.error(f"--steps + --warmup must stay within {args.context - args.prompt_len} decoded tokens")
 
@@ -182,6 +234,7 @@ def main() -> int:
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     per_seq = -(-(args.prompt_len + max(DECODE_LEN, args.steps + args.warmup) + 64) // 64) * 64
     cache_tokens = max(max_batch * per_seq, -(-max(PREFILL_LEN, args.prefill_len) // 64) * 64 + 64)
+    peaks = measured_peaks() if args.dtype == "bfloat16" else None
     engine = Engine.from_random(cfg, seed=0, dtype=args.dtype, max_slots=max_batch, max_context=args.context,
                                 cache_tokens=cache_tokens, device="cuda:0")
     dkey = "bf16" if args.dtype == "bfloat16" else "fp32"
@@ -193,13 +246,17 @@ def main() -> int:
               flush=True)
         return 0
 
-    dt, contexts = run_decode(engine, args.batch, args.steps, args.warmup, seed=1, prompt_len=args.prompt_len)
+    first_step = {}
+    dt, contexts = run_decode(engine, args.batch, args.steps, args.warmup, seed=1, prompt_len=args.prompt_len,
+                              lengths=lengths, first_step=first_step)
     ms_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     need = decode_step_bytes(m, contexts)
     achieved = need / (ms_step * 1e-3) / 1e9
     out = {
-        "metric": f"decode tok/s, Gemma3-{args.model.upper()} {dkey}, batch {args.batch}, {args.prompt_len}-token prompts + 256 decoded",
+        "metric": f"decode tok/s, Gemma3-{args.model.upper()} {dkey}, batch {args.batch}, "
+                  + (f"prompts of unequal lengths {min(lengths)}..{max(lengths)}" if lengths else f"{args.prompt_len}-token prompts")
+                  + f" + {args.warmup + args.steps + 1} decoded ({args.steps} steps timed after {args.warmup} of warm-up)",
         "value": round(value, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dkey, "data": "synthetic: uniform-random token ids, random N(0,0.02) weights",
@@ -207,12 +264,20 @@ def main() -> int:
                    "hidden": m["e"], "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
                    "head_dim": cfg["head_dim"], "intermediate": m["ff"], "vocab": m["v"],
                    "sliding_window": m["window"], "sliding_pattern": cfg["sliding_window_pattern"],
-                   "global_batch": args.batch, "seq_len": args.prompt_len + DECODE_LEN, "prompt_len": args.prompt_len,
+                   "global_batch": args.batch, "seq_len": args.prompt_len + args.warmup + args.steps + 1,
+                   "prompt_len": args.prompt_len,
                    "context": args.context, "prefill_len": PREFILL_LEN, "parallelism": "single GPU",
                    "sampling": "greedy", "weights_gb": round(2 * (m["linear_params"] + m["table_params"]) / 1e9, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
     }
+    if peaks is not None:
+        out["peaks_measured"] = peaks
+    if lengths:
+        flops = sum(prefill_flops(m, n) for n in lengths)
+        out["ragged_prefill"] = {"value": round(first_step["tokens"] / (first_step["ms"] * 1e-3), 1),
+                                 "tokens": first_step["tokens"], "ms": first_step["ms"], "sequences": len(lengths),
+                                 "frac": round(flops / (first_step["ms"] * 1e-3) / PEAK_FLOPS[dkey], 4)}
     if not args.no_points:
         pdt = run_prefill(engine, seed=2)
         flops = prefill_flops(m, PREFILL_LEN)
