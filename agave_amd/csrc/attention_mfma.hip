@@ -1076,8 +1076,10 @@ static int raise_decode_lds_allowance() {
 }
 
 // FUSED: a.q is the raw q projection and f says how to normalise and rotate it (head sizes 64, 128, 256 only).
+// merge: run the pass that merges the splits' partial results into a.out (false: the caller's next
+// kernel reads the partial results themselves).
 template <bool FUSED>
-static int launch_decode(const AttnArgs& a, const QkFuse& f, int N, hipStream_t stream) {
+static int launch_decode(const AttnArgs& a, const QkFuse& f, int N, hipStream_t stream, bool merge = true) {
     const int nh = a.nh, nkv = a.nkv, hd = a.hd, splits = a.splits;
     AGAVE_CHECK(splits >= 1 && splits <= COMBINE_MAX_SPLITS && a.pages_per_split >= 1, "attn_decode_mfma: bad split plan %d x %d", splits, a.pages_per_split);
     AGAVE_CHECK(splits == 1 || (a.part_o && a.part_ml), "attn_decode_mfma: splits need the partial buffers");
@@ -1102,7 +1104,7 @@ static int launch_decode(const AttnArgs& a, const QkFuse& f, int N, hipStream_t 
     else if (hd <= 128) attn_decode_mfma_kernel<8><<<grid, 256, lds, stream>>>(a);
     else attn_decode_mfma_kernel<16><<<grid, 256, lds, stream>>>(a);
     AGAVE_LAUNCH_CHECK("attn_decode_mfma");
-    if (splits > 1) {
+    if (splits > 1 && merge) {
         attn_combine_kernel<<<N * nh, hd >= 256 ? 256 : (hd >= 128 ? 128 : 64), 0, stream>>>(a.part_o, a.part_ml, a.out, a.ldo, nh, hd, splits);
         AGAVE_LAUNCH_CHECK("attn_combine");
     }
@@ -1177,7 +1179,9 @@ extern "C" int agave_attn_decode_mfma_noalloc(const void* q, long ldq, void* out
 
 // Decode attention that first does the q/k head norm, the rotation and the cache write of each
 // sequence's new token (one token per sequence, positions tok_pos): q, k, v are the raw
-// projections; k and v null for a run that appends nothing.
+// projections; k and v null for a run that appends nothing.  leave_partials: with more than one
+// split, do not merge the splits' results into `out`; the caller's next kernel reads part_o and
+// part_ml itself (gemm_mfma.hip: the output projection that merges while it stages its input).
 extern "C" int agave_attn_decode_fused(const void* q, long ldq, const void* k, long ldk, const void* v, long ldv,
                                        const float* q_gain, const float* k_gain, float eps_q, float eps_k,
                                        const float* inv_freq, int rot_half, float pos_scale, void* out, long ldo,
@@ -1185,16 +1189,17 @@ extern "C" int agave_attn_decode_fused(const void* q, long ldq, const void* k, l
                                        int width, const int* base, int n_pages, const int* tok_seq,
                                        const int* tok_pos, int N, int nh, int nkv, int hd, float scale, int window,
                                        int splits, int pages_per_split, int seq_is_token, int table_from_reach,
-                                       hipStream_t stream) {
+                                       int leave_partials, hipStream_t stream) {
     AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
                table, width, base, n_pages, tok_seq, tok_pos, nullptr, 0, nh, nkv, hd, scale, window, splits,
                pages_per_split, seq_is_token, table_from_reach};
     if (check_common("attn_decode_fused", a, N)) return -1;
+    AGAVE_CHECK(!leave_partials || splits > 1, "attn_decode_fused: partial results exist only with more than one split");
     AGAVE_CHECK((k == nullptr) == (v == nullptr), "attn_decode_fused: k and v come together");
     AGAVE_CHECK(!k || (ldk >= (long)nkv * hd && ldv >= (long)nkv * hd), "attn_decode_fused: a k or v row stride is below nkv*hd");
     AGAVE_CHECK(rot_half >= 0 && 2 * rot_half <= hd && (rot_half == 0 || inv_freq), "attn_decode_fused: bad rotation (rotary_dim %d, head_dim %d)", 2 * rot_half, hd);
     QkFuse f{(const bf16*)k, ldk, (const bf16*)v, ldv, q_gain, k_gain, eps_q, eps_k, inv_freq, rot_half, pos_scale};
-    return launch_decode<true>(a, f, N, stream);
+    return launch_decode<true>(a, f, N, stream, !leave_partials);
 }
 
 // How many workgroups should share a block of positions' pages in a prefill of these sizes (1:

@@ -432,6 +432,193 @@ extern "C" int agave_gemm_skinny(const void* X, long ldx, const void* Wp, int dt
 }
 
 
+
+// ------------------------------------------------------------------ output projection from the decode attention's shares
+// A decode step over a long cache leaves, for every (token, head, share of the keys), an
+// unnormalised output row with its reference and its sum (attention_mfma.hip: part_o
+// [token][head][share][hd], part_ml [token][head][share][2] with the reference in natural
+// logarithms).  Merging them is a kernel of its own that moves next to nothing; here the
+// product that reads the merged rows merges them itself while it stages them:
+//   x[t][head] = sum_s part_o[s] * exp(m_s - m) / sum_s l_s * exp(m_s - m),  rounded to bfloat16
+// (the arithmetic of attn_combine_kernel; the sums may be taken in another order), then Y = x W^T.
+// A workgroup takes R row blocks of W and the columns of `hps` heads; the grid's y counts those
+// runs of heads, and Y is one 32-bit slice [M][N] per run: whoever reads Y adds the slices (the
+// residual kernel does).  Up to 16 tokens.
+#define OPC_MAX_COLS 1024          // columns (hps * hd) a workgroup stages
+#define OPC_MAX_SHARES 64
+// NKS: k-steps of 32 columns a wave takes (it takes every fourth one of the workgroup's);
+// RB: row blocks whose tiles a wave asks for at a time.  Everything the workgroup needs first (the
+// first RB row blocks' tiles, the shares' references and sums, the first eight shares' rows) is
+// asked for before anything is waited for: one round trip to memory.
+template <int NKS, int RB>
+__global__ __launch_bounds__(256) void gemm_oproj_combine_kernel(const float* __restrict__ part_o,
+                                                                  const float* __restrict__ part_ml,
+                                                                  const uint4* __restrict__ Wp, float* __restrict__ Y,
+                                                                  int M, int N, int nh, int hd, int shares, int hps, int R,
+                                                                  int NB, int KB) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char opc_smem[];
+    const int cols = hps * hd, row = cols + 8;                    // staged row in bf16, 16 bytes of padding
+    bf16* xs = reinterpret_cast<bf16*>(opc_smem);                  // [16][row]
+    float* red = reinterpret_cast<float*>(opc_smem);               // afterwards: [4 waves][R][256] partial sums
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
+    const int nb0 = blockIdx.x * R, run = blockIdx.y;
+    const int kb0 = run * (cols / 32), kbs = cols / 32;            // this run's k-steps
+    const int n_mine = (kbs - wave + 3) / 4;                       // k-steps wave, wave + 4, ...
+
+    // (two sets of registers, each named by a constant: an index known only at run time would send the array to memory)
+    frag16 wreg0[RB][NKS], wreg1[RB][NKS];
+    auto load_w = [&](frag16 (&wr)[RB][NKS], int r0) {
+#pragma unroll
+        for (int rr = 0; rr < RB; ++rr) {
+            const int nb = nb0 + r0 + rr < NB ? nb0 + r0 + rr : NB - 1;
+#pragma unroll
+            for (int i = 0; i < NKS; ++i) {
+                const int ks = wave + 4 * (i < n_mine ? i : 0);
+                wr[rr][i].u = Wp[w_tile(nb, kb0 + ks, NB, KB) * 64 + lane];
+            }
+        }
+    };
+    load_w(wreg0, 0);
+
+    // the merged rows, eight columns a thread at a time; rows past the last token are zero.  A thread
+    // works out the shares' weights of its (token, head) itself: a few exponentials cost less than
+    // a barrier between those who would compute them and those who use them.
+    const int groups = cols / 8;
+    for (int gi = threadIdx.x; gi < 16 * groups; gi += 256) {
+        const int m = gi / groups, c0 = (gi % groups) * 8;
+        uint4 packed = uint4{0, 0, 0, 0};
+        if (m < M) {
+            const int hh = c0 / hd, d0 = c0 % hd;
+            const size_t slot0 = ((size_t)m * nh + run * hps + hh) * shares;
+            const float* po = part_o + slot0 * hd + d0;
+            const float2* ml = reinterpret_cast<const float2*>(part_ml) + slot0;
+            float4 lo4[8], hi4[8];
+            float2 mls[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {                           // the first eight shares: asked for at once
+                const int sh = u < shares ? u : shares - 1;
+                lo4[u] = *reinterpret_cast<const float4*>(po + (size_t)sh * hd);
+                hi4[u] = *reinterpret_cast<const float4*>(po + (size_t)sh * hd + 4);
+                mls[u] = ml[sh];
+            }
+            float mx = -INFINITY;
+            for (int sh = 8; sh < shares; ++sh) mx = fmaxf(mx, ml[sh].x);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) mx = fmaxf(mx, mls[u].x);
+            float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            float l = 0.f;
+            for (int s0 = 0; s0 < shares; s0 += 8) {
+                if (s0 > 0) {
+#pragma unroll
+                    for (int u = 0; u < 8; ++u) {
+                        const int sh = s0 + u < shares ? s0 + u : shares - 1;
+                        lo4[u] = *reinterpret_cast<const float4*>(po + (size_t)sh * hd);
+                        hi4[u] = *reinterpret_cast<const float4*>(po + (size_t)sh * hd + 4);
+                        mls[u] = ml[sh];
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const float f = (s0 + u < shares && mls[u].x != -INFINITY) ? __expf(mls[u].x - mx) : 0.f;
+                    l += mls[u].y * f;
+                    acc[0] += lo4[u].x * f; acc[1] += lo4[u].y * f; acc[2] += lo4[u].z * f; acc[3] += lo4[u].w * f;
+                    acc[4] += hi4[u].x * f; acc[5] += hi4[u].y * f; acc[6] += hi4[u].z * f; acc[7] += hi4[u].w * f;
+                }
+            }
+            const float iv = l > 0.f ? 1.0f / l : 0.f;
+            packed.x = f32x2_to_bf16x2(acc[0] * iv, acc[1] * iv);
+            packed.y = f32x2_to_bf16x2(acc[2] * iv, acc[3] * iv);
+            packed.z = f32x2_to_bf16x2(acc[4] * iv, acc[5] * iv);
+            packed.w = f32x2_to_bf16x2(acc[6] * iv, acc[7] * iv);
+        }
+        *reinterpret_cast<uint4*>(xs + (size_t)m * row + c0) = packed;
+    }
+    __syncthreads();
+    // this wave's k-steps of the staged rows, as B operands
+    frag16 xb[NKS];
+#pragma unroll
+    for (int i = 0; i < NKS; ++i) {
+        const int ks = wave + 4 * (i < n_mine ? i : 0);
+        xb[i].u = *reinterpret_cast<const uint4*>(xs + (size_t)j * row + ks * 32 + g * 8);
+    }
+    __syncthreads();                                              // the staged rows give way to the partial sums
+    auto use_w = [&](const frag16 (&wr)[RB][NKS], int r0) {
+#pragma unroll
+        for (int rr = 0; rr < RB; ++rr) {
+            f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < NKS; ++i)
+                if (i < n_mine) acc = mfma_16x16x32(wr[rr][i], xb[i], acc);
+            if (r0 + rr < R) *reinterpret_cast<f32x4_t*>(red + ((size_t)wave * R + r0 + rr) * 256 + lane * 4) = acc;
+        }
+    };
+    for (int r0 = 0; r0 < R; r0 += 2 * RB) {
+        if (r0 + RB < R) load_w(wreg1, r0 + RB);
+        use_w(wreg0, r0);
+        if (r0 + 2 * RB < R) load_w(wreg0, r0 + 2 * RB);
+        if (r0 + RB < R) use_w(wreg1, r0 + RB);
+    }
+    __syncthreads();
+    float* y = Y + (size_t)run * M * N;
+    for (int r = wave; r < R; r += 4) {
+        if (nb0 + r >= NB || j >= M) continue;
+        f32x4_t sum = *reinterpret_cast<const f32x4_t*>(red + (size_t)r * 256 + lane * 4);
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const f32x4_t part = *reinterpret_cast<const f32x4_t*>(red + ((size_t)w * R + r) * 256 + lane * 4);
+            sum += part;
+        }
+        const int n = (nb0 + r) * 16 + g * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (n + e < N) y[(size_t)j * N + n + e] = sum[e];
+    }
+}
+
+// Heads a workgroup's run of columns holds, for a product over nh heads of hd columns: the fewest
+// that leave at most 8 runs (the reader adds that many slices); 0 if this kernel does not take
+// the sizes (the caller then merges the shares first and runs the ordinary product).
+extern "C" int agave_oproj_combine_heads_per_run(int M, int nh, int hd, int shares) {
+    if (M <= 0 || M > 16 || nh <= 0 || hd <= 0 || hd % 32 != 0 || shares < 2) return 0;
+    for (int hps = 1; hps <= nh; ++hps) {
+        if (nh % hps != 0 || nh / hps > 8) continue;
+        if (hps * hd > OPC_MAX_COLS || shares > OPC_MAX_SHARES) return 0;
+        return hps;
+    }
+    return 0;
+}
+
+// Y: [nh / hps][M][N] 32-bit slices.
+extern "C" int agave_gemm_oproj_combine(const float* part_o, const float* part_ml, const void* Wp, float* Y, int M,
+                                        int N, int nh, int hd, int shares, hipStream_t stream) {
+    const int hps = agave_oproj_combine_heads_per_run(M, nh, hd, shares);
+    AGAVE_CHECK(hps > 0, "gemm_oproj_combine: no kernel for %d tokens, %d heads of %d, %d shares", M, nh, hd, shares);
+    AGAVE_CHECK(part_o && part_ml && Wp && Y && N > 0, "gemm_oproj_combine: null tensor or no rows");
+    AGAVE_CHECK(((uintptr_t)part_o % 16) == 0 && ((uintptr_t)Y % 16) == 0, "gemm_oproj_combine: unaligned buffers");
+    const int runs = nh / hps, cols = hps * hd, K = nh * hd;
+    const int NB = (N + 15) / 16, KB = (K + 31) / 32;
+    int R = (int)(((long)NB * runs + 255) / 256);                 // some 256 workgroups
+    if (R < 1) R = 1;
+    if (R > 12) R = 12;
+    const size_t staged = (size_t)16 * (cols + 8) * 2;
+    const size_t sums = (size_t)4 * R * 256 * 4;
+    const size_t lds = staged > sums ? staged : sums;
+    AGAVE_CHECK(lds <= 64 * 1024, "gemm_oproj_combine: %zu bytes of LDS", lds);
+    const dim3 grid((NB + R - 1) / R, runs);
+    const int nks = (cols / 32 + 3) / 4;
+    // tiles a wave asks for at a time: RB * NKS, sixteen or so
+#define OPC_LAUNCH(NKS_, RB_)                                                                                   \
+    gemm_oproj_combine_kernel<NKS_, RB_><<<grid, 256, lds, stream>>>(part_o, part_ml, (const uint4*)Wp, Y, M, N, nh, \
+                                                                     hd, shares, hps, R, NB, KB)
+    if (nks <= 1) OPC_LAUNCH(1, 12);
+    else if (nks <= 2) OPC_LAUNCH(2, 6);
+    else if (nks <= 4) OPC_LAUNCH(4, 4);
+    else OPC_LAUNCH(8, 2);
+#undef OPC_LAUNCH
+    AGAVE_LAUNCH_CHECK("gemm_oproj_combine");
+    return 0;
+}
+
 // ------------------------------------------------------------------ tiled product (prefill)
 // A workgroup computes WT*64 weight rows x TT tokens in tiles of 32 x 32
 // (v_mfma_f32_32x32x16_bf16) with eight waves (2 x 4, a wave WT x TT/128 tiles): two per SIMD,

@@ -12,7 +12,7 @@ kernels.register_signatures("attention_mfma", {
     "agave_attn_decode_mfma": [_P, _L, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _I,
                                _I, _P],
     "agave_attn_decode_fused": [_P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I,
-                                _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _P],
+                                _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _P],
     "agave_attn_prefill_mfma": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
                                 _I, _P],
     "agave_attn_prefill_splits": [_I, _I, _I, _I, _I, _I],
@@ -101,9 +101,12 @@ def decode_fused(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.T
                  q_gain: Optional[torch.Tensor], k_gain: Optional[torch.Tensor], eps_q: float, eps_k: float,
                  inv_freq: Optional[torch.Tensor], pos_scale: float, k_pages: torch.Tensor, v_pages: torch.Tensor,
                  table: torch.Tensor, base: torch.Tensor, step, n_heads: int, n_kv: int, head_dim: int, scale: float,
-                 window: Optional[int]) -> None:
+                 window: Optional[int], partials_ok=None):
     """A decode step's attention from the raw projections: the kernel normalises and rotates q and
-    k, writes k and v into their pages (``k`` None: nothing is appended) and attends."""
+    k, writes k and v into their pages (``k`` None: nothing is appended) and attends.
+    ``partials_ok``: a function of the number of splits that says whether the caller's next kernel
+    can merge the splits' partial results itself; if it says so and the step is split, they are returned as ``(part_o [n, heads, splits, head_dim], part_ml [n, heads,
+    splits, 2])`` and ``out`` is left alone.  Otherwise None is returned and ``out`` is written."""
     n = step.n_tokens
     if not step.is_decode or head_dim not in FUSED_HEAD_DIMS:
         raise ValueError("decode_fused: needs a decode step and a head size of 64, 128 or 256")
@@ -132,6 +135,7 @@ def decode_fused(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.T
         ws = step.workspace
         part_o = ws.get("attn_part_o", n * n_heads * splits, head_dim, torch.float32)
         part_ml = ws.get("attn_part_ml", n * n_heads * splits, 2, torch.float32)
+    leave = bool(splits > 1 and partials_ok is not None and partials_ok(splits))
     library.call(kernels.lib("attention_mfma"), "agave_attn_decode_fused", q.data_ptr(), q.stride(0),
                  kernels.ptr(k), k.stride(0) if k is not None else 0, kernels.ptr(v),
                  v.stride(0) if v is not None else 0, kernels.ptr(q_gain), kernels.ptr(k_gain), eps_q, eps_k,
@@ -139,4 +143,7 @@ def decode_fused(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.T
                  kernels.ptr(part_ml), k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width,
                  base.data_ptr(), n_pages, step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), n, n_heads, n_kv,
                  head_dim, scale, int(window or 0), splits, per, 1 if step.n_seqs == n else 0,
-                 1 if getattr(step, "tables_start_at_reach", False) else 0, kernels.stream())
+                 1 if getattr(step, "tables_start_at_reach", False) else 0, 1 if leave else 0, kernels.stream())
+    if leave:
+        return part_o.view(n, n_heads, splits, head_dim), part_ml.view(n, n_heads, splits, 2)
+    return None

@@ -16,6 +16,8 @@ kernels.register_signatures("gemm_mfma", {
     "agave_gemm_tiled_slices": [_I, _I, _I],
     "agave_gemm_tiled_in_slices": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
     "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P, _L, _P],
+    "agave_oproj_combine_heads_per_run": [_I, _I, _I, _I],
+    "agave_gemm_oproj_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
 })
 
 SKINNY_MAX_M = 64
@@ -165,6 +167,42 @@ def try_linear(x: torch.Tensor, lin, out: torch.Tensor) -> bool:
         return False
     product(x, packed, out, lin.out_features, 0)
     return True
+
+
+def partials_runs(m: int, n_heads: int, head_dim: int, splits: int) -> int:
+    """How many 32-bit slices :func:`product_of_partials` leaves for these sizes (runs of heads that a
+    workgroup takes together); 0 if it does not take them."""
+    if splits < 2:
+        return 0
+    key = ("runs", m, n_heads, head_dim, splits)
+    got = _slices.get(key)
+    if got is None:
+        hps = int(kernels.lib("gemm_mfma").agave_oproj_combine_heads_per_run(m, n_heads, head_dim, splits))
+        got = _slices[key] = n_heads // hps if hps > 0 else 0
+    return got
+
+
+def product_of_partials(part_o: torch.Tensor, part_ml: torch.Tensor, packed: torch.Tensor, out: torch.Tensor,
+                        n_out: int) -> None:
+    """The product of the decode attention's merged output rows with W^T, from the splits' partial
+    results: out[r] (float32 [runs, M, n_out]) are slices that add up to it.  part_o is [M, heads,
+    splits, head_dim], part_ml [M, heads, splits, 2] (reference in natural logarithms, sum)."""
+    if not (part_o.is_cuda and part_ml.is_cuda and packed.is_cuda and out.is_cuda):
+        raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
+    if part_o.dim() != 4 or part_o.dtype != torch.float32 or not part_o.is_contiguous():
+        raise ValueError("product_of_partials: part_o must be a contiguous float32 [M, heads, splits, head_dim] tensor")
+    m, nh, splits, hd = part_o.shape
+    if part_ml.shape != (m, nh, splits, 2) or part_ml.dtype != torch.float32 or not part_ml.is_contiguous():
+        raise ValueError(f"product_of_partials: part_ml must be a contiguous float32 [{m}, {nh}, {splits}, 2] tensor")
+    runs = partials_runs(m, nh, hd, splits)
+    if runs == 0:
+        raise ValueError(f"product_of_partials: no kernel for {m} tokens, {nh} heads of {hd}, {splits} splits")
+    if out.dtype != torch.float32 or out.shape != (runs, m, n_out) or not out.is_contiguous():
+        raise ValueError(f"product_of_partials: out must be a contiguous float32 [{runs}, {m}, {n_out}] tensor")
+    if packed.dtype != torch.bfloat16 or packed.numel() != ((n_out + 15) // 16) * ((nh * hd + 31) // 32) * 512:
+        raise ValueError("product_of_partials: the packed weight does not fit these sizes")
+    library.call(kernels.lib("gemm_mfma"), "agave_gemm_oproj_combine", part_o.data_ptr(), part_ml.data_ptr(),
+                 packed.data_ptr(), out.data_ptr(), m, n_out, nh, hd, splits, kernels.stream())
 
 
 def embed_scale_packed(tokens: torch.Tensor, packed: torch.Tensor, scale: float, out: torch.Tensor, vocab: int) -> None:

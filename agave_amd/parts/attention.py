@@ -69,8 +69,14 @@ class Attention:
         ctx_out = ws.get("attn_ctx", n, self.qd, x.dtype)
         if fused is not None:
             inv_freq, pos_scale = fused()
-            attn_ops.qk_attention(q, k, v, q_out, ctx_out, qg, kg, qe, ke, inv_freq, pos_scale, k_pages, v_pages,
-                                  table, base, step, s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window, packed)
+            # a decode step whose keys are shared among workgroups leaves partial results, which the
+            # output product merges itself if it can (one kernel less a layer)
+            partials_ok = (lambda splits: self.o.takes_partials(n, s.n_heads, s.head_dim, splits)) if step.is_decode else None
+            parts = attn_ops.qk_attention(q, k, v, q_out, ctx_out, qg, kg, qe, ke, inv_freq, pos_scale, k_pages, v_pages,
+                                          table, base, step, s.n_heads, s.n_kv_heads, s.head_dim, s.scale, s.window,
+                                          packed, partials_ok=partials_ok)
+            if parts is not None:
+                return self.o.forward_partials(parts[0], parts[1], tag="attn_o")
             return self.o.forward(ctx_out, tag="attn_o", slices_ok=True)       # the block adds it to the residual stream
         else:
             # a position encoding the q/k kernel does not know: the norms, then the part's own

@@ -79,6 +79,27 @@ class Linear:
         library.profile.label = None
         return out
 
+    def takes_partials(self, n: int, n_heads: int, head_dim: int, splits: int) -> bool:
+        """Whether :meth:`forward_partials` can take the decode attention's partial results for
+        ``n`` tokens in ``splits`` splits (the kernel library has the last word on the sizes)."""
+        if self.packed is None or self.interleave_ff or self.in_features != n_heads * head_dim:
+            return False
+        from ..ops import gemm_mfma
+        return gemm_mfma.partials_runs(n, n_heads, head_dim, splits) > 0
+
+    def forward_partials(self, part_o: torch.Tensor, part_ml: torch.Tensor, tag: Optional[str] = None) -> torch.Tensor:
+        """The product of the attention rows that the splits' partial results stand for: they are
+        merged inside the product's kernel.  Returns float32 slices [runs, n, out] that add up."""
+        from ..ops import gemm_mfma, library
+        n, nh, splits, hd = part_o.shape
+        runs = gemm_mfma.partials_runs(n, nh, hd, splits)
+        out = self.env.workspace.get((tag or self.name) + "_runs", runs * n, self.out_features,
+                                     torch.float32).view(runs, n, self.out_features)
+        library.profile.label = self.name
+        gemm_mfma.product_of_partials(part_o, part_ml, self.packed, out, self.out_features)
+        library.profile.label = None
+        return out
+
     def forward_geglu(self, x: torch.Tensor, out: torch.Tensor) -> bool:
         """out = gelu_tanh(gate x) * (up x) in one kernel, if the weight was packed for it."""
         if not self.interleave_ff:

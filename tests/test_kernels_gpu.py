@@ -517,6 +517,60 @@ def test_gemm_skinny_refuses_what_it_cannot_do(G):
         G.skinny(torch.zeros(4, 60, dtype=torch.bfloat16, device=DEV), w, out[:4], 32)   # K no multiple of 8
 
 
+@pytest.mark.parametrize("m,nh,hd,splits,n", [(8, 8, 256, 6, 2560), (1, 8, 256, 64, 2560), (16, 32, 128, 4, 5376),
+                                              (3, 6, 64, 2, 100), (5, 16, 256, 3, 3840), (2, 4, 96, 9, 250),
+                                              (13, 20, 128, 5, 72)])
+def test_product_of_the_decode_attention_s_partial_results(G, m, nh, hd, splits, n):
+    """The output projection that merges the splits' partial results itself, against the merge
+    written out (with its rows rounded to bfloat16, as the separate merge kernel leaves them) and an
+    ordinary product.  Some splits are empty (reference -inf, sum 0), as behind a window's edge."""
+    g = torch.Generator().manual_seed(m * 1000 + nh + splits)
+    part_o = torch.randn(m, nh, splits, hd, generator=g)
+    ref_m = torch.randn(m, nh, splits, generator=g) * 3
+    sums = torch.rand(m, nh, splits, generator=g) * 30 + 0.5
+    empty = torch.rand(m, nh, splits, generator=g) < 0.2
+    empty[:, :, 0] = False                                   # every row keeps a split
+    if m > 1:
+        empty[1, 0, :] = True                                # but one: no key at all gives zeros
+    ref_m[empty], sums[empty] = float("-inf"), 0.0
+    part_o[empty] = 0.0
+    part_ml = torch.stack([ref_m, sums], dim=-1).contiguous()
+    runs = G.partials_runs(m, nh, hd, splits)
+    assert 1 <= runs <= 8 and nh % runs == 0
+    w = (torch.randn(n, nh * hd, generator=g) * 0.05).bfloat16()
+    packed = G.pack_weight(w.to(DEV))
+    out = torch.full((runs, m, n), float("nan"), device=DEV)
+    G.product_of_partials(part_o.to(DEV), part_ml.to(DEV), packed, out, n)
+    mx = ref_m.double().max(dim=-1, keepdim=True).values
+    f = torch.where(torch.isinf(ref_m), torch.zeros_like(ref_m, dtype=torch.float64), torch.exp(ref_m.double() - mx))
+    f = torch.nan_to_num(f, nan=0.0)
+    l = (sums.double() * f).sum(-1)
+    x = (part_o.double() * f[..., None]).sum(2) / torch.where(l > 0, l, torch.ones_like(l))[..., None]
+    x = torch.where((l > 0)[..., None], x, torch.zeros_like(x)).reshape(m, nh * hd).bfloat16().double()
+    ref = x @ w.double().T
+    got = out.cpu().double()
+    assert torch.isfinite(got).all()
+    scale = float(ref.abs().max())
+    # a merged value within rounding of a bfloat16 step's middle may round the other way: 2^-8 of one term
+    assert float((got.sum(0) - ref).abs().max()) <= 3e-3 * scale
+    # each slice is the product over its own run of heads
+    cols = nh * hd // runs
+    for r in range(runs):
+        part = x[:, r * cols:(r + 1) * cols] @ w.double()[:, r * cols:(r + 1) * cols].T
+        assert float((got[r] - part).abs().max()) <= 3e-3 * scale, r
+
+
+def test_product_of_partial_results_refuses_what_it_cannot_do(G):
+    assert G.partials_runs(17, 8, 256, 4) == 0          # more than one tile of tokens
+    assert G.partials_runs(4, 8, 48, 4) == 0            # heads that are no whole k-steps of 32 columns
+    assert G.partials_runs(4, 8, 256, 1) == 0           # nothing to merge
+    assert G.partials_runs(16, 32, 128, 65) == 0        # more splits than the kernel merges
+    with pytest.raises(ValueError, match="no kernel"):
+        G.product_of_partials(torch.zeros(17, 8, 4, 256, device=DEV), torch.zeros(17, 8, 4, 2, device=DEV),
+                              G.pack_weight(torch.zeros(32, 2048, dtype=torch.bfloat16, device=DEV)),
+                              torch.zeros(8, 17, 32, device=DEV), 32)
+
+
 # ---------------------------------------------------------------- matrix-core attention over packed pages
 class _FakeStep:
     """What the attention op reads of a step."""
