@@ -351,18 +351,24 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
             for (int k = 0; k < NV; ++k) vreg0[k] = vsrc0[lane + 64 * k];
         }
     }
-    // A wave takes half pages (units of 32 keys): wave w the half w % 2 of the pages
-    // page_lo + w / 2, + 2, + 4, ... of the workgroup's range, so that four waves share two pages
-    // at a time and a range of 2 pages is one unit, one round trip to memory, for every wave.
-    const int half = wave & 1, wpage = wave >> 1;
-    const int col0 = split * a.pages_per_split + wpage;
-    int pg0 = -1;                             // (kept as loaded: widening it here would wait for the load)
-    if (a.table_from_reach && col0 < a.width) pg0 = a.table[(size_t)b * a.width + col0];
+    // The keys this token sees lie in half pages (units of 32 keys) u_first .. u_last.  The launch's
+    // splits share them evenly, whatever the sequence's length (a run of whole pages per split would
+    // leave the last splits of a short sequence idle and the waves of a split unequal shares); a
+    // workgroup's four waves take its units in turn.  A unit is one round trip to memory, and with
+    // as many waves as units nearly every wave makes just one.
+    // The first columns of the table row are asked for before the position is known, a column per
+    // lane: which of them this wave needs depends on the position, but waiting for that first would
+    // put a second round trip before the first key.
+    int trow = -1;
+    if (a.table_from_reach) trow = a.table[(size_t)b * a.width + (lane < a.width ? lane : 0)];
     const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
     const int first = lo / AGAVE_PAGE, last = p / AGAVE_PAGE;
-    const int page_lo = first + split * a.pages_per_split;
-    int page_hi = page_lo + a.pages_per_split - 1;
-    if (page_hi > last) page_hi = last;
+    const int u_first = lo / 32, u_last = p / 32, n_u = u_last - u_first + 1;
+    const int ua = u_first + (int)((long)split * n_u / a.splits);
+    const int ub = u_first + (int)((long)(split + 1) * n_u / a.splits);
+    const int u0 = ua + wave;
+    const int half = u0 & 1;                                       // (a wave's units are four apart: one half)
+    const int n_my = u0 < ub ? (ub - u0 + 3) / 4 : 0;              // units this wave takes
     constexpr int hd = HDT * 16;
     const float scale2 = a.scale * 1.4426950408889634f;          // scores in units of log2
 
@@ -383,29 +389,27 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     float m_ref = -INFINITY, l = 0.f;
 
     constexpr size_t k_stride = (size_t)4 * KS * 64, v_stride = (size_t)HDT * 2 * 64;   // uint4 per (page, kv head)
-    // (the second half of the token's own page holds no key yet when the position lies in its first half)
-    const int my_hi = (half == 1 && page_hi == last && p % AGAVE_PAGE < 32) ? page_hi - 1 : page_hi;
-    const int n_my = (my_hi >= page_lo + wpage) ? (my_hi - page_lo - wpage) / 2 + 1 : 0;   // pages this wave takes
-    // the ids of this wave's first pages are fetched together, ahead of any use: a lookup in the
-    // loop would stand between every two pages
+    // a table wider than a wave: the ids of this wave's next pages are fetched together, ahead of
+    // any use (a lookup in the loop would stand between every two units)
     constexpr int PG_AHEAD = 10;
     int pg_pre[PG_AHEAD];
+    const bool wide = a.table_from_reach && a.width > 64;
 #pragma unroll
-    for (int i = 1; i < PG_AHEAD; ++i) {
-        const int col = page_lo + wpage + 2 * i - first;
-        pg_pre[i] = (a.table_from_reach && i < n_my && col < a.width) ? a.table[(size_t)b * a.width + col] : -1;
+    for (int i = 0; i < PG_AHEAD; ++i) {
+        const int col = ((u0 + 4 * i) >> 1) - first;
+        pg_pre[i] = (wide && i < n_my && col < a.width) ? a.table[(size_t)b * a.width + col] : -1;
     }
-    auto page_id = [&](int i) -> int {           // i-th page of this wave (page ids fit 31 bits)
-        const int pi = page_lo + wpage + 2 * i;
+    auto page_id = [&](int i) -> int {           // page of this wave's i-th unit (page ids fit 31 bits)
+        const int pi = (u0 + 4 * i) >> 1;
         int pg;
         if (a.table_from_reach) {
             const int col = pi - first;
-            if (i == 0) {
-                pg = pg0;
+            if (!wide) {
+                pg = col < a.width ? __shfl(trow, col, 64) : -1;
             } else if (i < PG_AHEAD) {
                 pg = -1;
 #pragma unroll
-                for (int k = 1; k < PG_AHEAD; ++k)
+                for (int k = 0; k < PG_AHEAD; ++k)
                     if (k == i) pg = pg_pre[k];
             } else {
                 pg = col < a.width ? a.table[(size_t)b * a.width + col] : -1;
@@ -440,8 +444,8 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     }
     // FUSED: the token's own key and value go into the page of position p, by the workgroup that
     // reads it; the wave whose first page that is waits with its loads until the row is there
-    const bool writer = FUSED && f.k_raw != nullptr && page_lo <= last && page_hi == last;
-    const bool early = !(writer && page_lo + wpage == last);
+    const bool writer = FUSED && f.k_raw != nullptr && split == a.splits - 1;       // (the last split ends with u_last)
+    const bool early = !(writer && u0 == u_last);
     if (have && early) {
         load_k();
         load_v();
@@ -510,8 +514,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
         load_v();
     }
     while (have) {
-        const int pi = page_lo + wpage + 2 * cur_page;
-        const int key0 = pi * AGAVE_PAGE + 32 * half;             // first key of this unit
+        const int key0 = (u0 + 4 * cur_page) * 32;                // first key of this unit
         // S^T for the unit's two key tiles
         f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0;
 #pragma unroll

@@ -21,14 +21,25 @@ kernels.register_signatures("attention_mfma", {
 TARGET_WORKGROUPS = 256      # workgroups (of 4 waves) a decode launch aims for: one per compute unit
 
 
-def split_plan(page_span: int, units: int):
+def split_plan(page_span: int, units: int, head_dim: int = 0):
     """(splits, pages per split) for sequences spanning at most ``page_span`` pages when the launch
-    has ``units`` (token, kv head) pairs.  A workgroup's four waves take half a page each at a time,
-    two pages together.  (An even run of pages per split, which leaves no wave a half page short,
-    was measured at batch 8: nine splits of two pages are 7 % of a step slower than six of three.)"""
-    want = max(1, min(page_span, -(-TARGET_WORKGROUPS // max(units, 1))))
+    has ``units`` (token, kv head) pairs.  The kernels for head sizes 64, 128 and 256 share a
+    sequence's half pages evenly among the splits, four waves a split and a half page a wave at a
+    time: as many splits as fill the compute units, but no more than leave a split six half pages
+    (at a batch of 8 and a reach of 17 pages, 6 splits of 5 or 6 half pages measured 3 % of the
+    kernel faster than 8 of 4 or 5: what more splits gain in balance they lose in partial results).
+    The general kernel gives each split a run of whole pages."""
+    want = max(1, -(-TARGET_WORKGROUPS // max(units, 1)))
+    if head_dim in FUSED_HEAD_DIMS:
+        splits = max(1, min(TARGET_WORKGROUPS // max(units, 1), -(-2 * page_span // 6), MAX_SPLITS))
+        return splits, -(-page_span // splits)
+    want = min(want, page_span)
     per = -(-page_span // want)
     return -(-page_span // per), per
+
+
+MAX_SPLITS = 64              # what the merge inside the output product takes
+FUSED_HEAD_DIMS = (64, 128, 256)
 
 
 def check_table_reach(pos0, n_new, window: Optional[int], base, width: int) -> None:
@@ -66,7 +77,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
     if step.is_decode:
         span = step.page_span(window)
         chunks = -(-(n_heads // n_kv) // 16)
-        splits, per = split_plan(span, n * n_kv * chunks)
+        splits, per = split_plan(span, n * n_kv * chunks, head_dim)
         part_o = part_ml = None
         if splits > 1:
             ws = step.workspace
@@ -92,9 +103,6 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
                      step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), step.cu_dev.data_ptr(), step.n_seqs,
                      step.max_new, n, n_heads, n_kv, head_dim, scale, w, kernels.ptr(part_o), kernels.ptr(part_ml),
                      splits, kernels.stream())
-
-
-FUSED_HEAD_DIMS = (64, 128, 256)
 
 
 def decode_fused(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], out: torch.Tensor,
@@ -129,7 +137,7 @@ def decode_fused(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.T
     width = kernels._check_table(table, base, step.tok_seq)
     span = step.page_span(window)
     chunks = -(-(n_heads // n_kv) // 16)
-    splits, per = split_plan(span, n * n_kv * chunks)
+    splits, per = split_plan(span, n * n_kv * chunks, head_dim)
     part_o = part_ml = None
     if splits > 1:
         ws = step.workspace
