@@ -684,57 +684,6 @@ __global__ void attn_combine_kernel(const float* __restrict__ part_o, const floa
     }
 }
 
-// The same merge for many rows and few splits (a prompt whose blocks of positions were shared
-// among workgroups): a wave per (token, head), four elements a lane at a time, every load asked
-// for before the first is used.
-#define COMBINE_ROWS_MAX_SPLITS 4
-__global__ __launch_bounds__(256) void attn_combine_rows_kernel(const float* __restrict__ part_o,
-                                                                const float* __restrict__ part_ml,
-                                                                bf16* __restrict__ out, long ldo, int nh, int hd,
-                                                                int splits, long rows) {
-    const int lane = threadIdx.x & 63;
-    const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (r >= rows) return;
-    const long t = r / nh;
-    const int head = (int)(r % nh);
-    const size_t slot0 = (size_t)r * splits;
-    float ms[COMBINE_ROWS_MAX_SPLITS], ls[COMBINE_ROWS_MAX_SPLITS];
-#pragma unroll
-    for (int sp = 0; sp < COMBINE_ROWS_MAX_SPLITS; ++sp) {
-        const int s2 = sp < splits ? sp : splits - 1;
-        ms[sp] = part_ml[(slot0 + s2) * 2];
-        ls[sp] = part_ml[(slot0 + s2) * 2 + 1];
-    }
-    for (int d0 = lane * 4; d0 < hd; d0 += 256) {
-        float4 v[COMBINE_ROWS_MAX_SPLITS];
-#pragma unroll
-        for (int sp = 0; sp < COMBINE_ROWS_MAX_SPLITS; ++sp) {
-            const int s2 = sp < splits ? sp : splits - 1;
-            v[sp] = *reinterpret_cast<const float4*>(part_o + (slot0 + s2) * hd + d0);
-        }
-        float m = -INFINITY;
-#pragma unroll
-        for (int sp = 0; sp < COMBINE_ROWS_MAX_SPLITS; ++sp)
-            if (sp < splits) m = fmaxf(m, ms[sp]);
-        float l = 0.f;
-        float4 acc = float4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int sp = 0; sp < COMBINE_ROWS_MAX_SPLITS; ++sp) {
-            const float f = (sp < splits && ms[sp] != -INFINITY) ? __expf(ms[sp] - m) : 0.f;
-            l += ls[sp] * f;
-            acc.x += v[sp].x * f;
-            acc.y += v[sp].y * f;
-            acc.z += v[sp].z * f;
-            acc.w += v[sp].w * f;
-        }
-        const float inv = l > 0.f ? 1.0f / l : 0.f;
-        uint2 u;
-        u.x = f32x2_to_bf16x2(acc.x * inv, acc.y * inv);
-        u.y = f32x2_to_bf16x2(acc.z * inv, acc.w * inv);
-        *reinterpret_cast<uint2*>(out + (size_t)t * ldo + (size_t)head * hd + d0) = u;
-    }
-}
-
 // ------------------------------------------------------------------ prefill: 64 positions x QT heads per workgroup
 // grid (block of positions, kv head * head chunks, sequence).  The four waves are hw heads
 // wide and 4/hw tiles of 16 positions deep; a wave takes QT heads of its tile (slot j of tile t
@@ -835,6 +784,78 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int 
     }
 }
 
+// ------------------------------------------------------------------ the items of a prefill step
+// The causal triangle gives a prompt's blocks of positions anything from one page of keys to the
+// whole reach, and a prompt of a few thousand tokens has fewer blocks than the chip has compute
+// units.  The host therefore cuts the step into *items* of about equal work and lists them with
+// the largest first: an item is a block of positions of one sequence and a run of the pages that
+// the block sees; a block whose reach is longer than an item may be is cut into several pieces,
+// which leave partial results for attn_merge_pieces_kernel.  Workgroups take the items in the
+// list's order as compute units free up (grid x = item * kv head chunks + kv head chunk), so the
+// last ones to start are the smallest.
+struct PrefillItem {
+    int seq;          // sequence of the step
+    int blk0;         // first of the block's tokens, counted within the sequence's tokens of this step
+    int page_first;   // first page (position / 64) of this piece
+    int n_pages;      // pages of this piece
+    int piece;        // which piece of the block this is
+    int n_pieces;     // pieces the block is cut into (1: the item writes the output itself)
+};
+
+// out[t][head] from the pieces' partial results, for the tokens of blocks that were cut into
+// pieces (tok_pieces[t] > 1; the others were written by their item itself): a wave per (token,
+// head), four elements a lane at a time, every load asked for before the first is used.
+#define MERGE_MAX_PIECES 4
+__global__ __launch_bounds__(256) void attn_merge_pieces_kernel(const float* __restrict__ part_o,
+                                                                const float* __restrict__ part_ml,
+                                                                const int* __restrict__ tok_pieces,
+                                                                bf16* __restrict__ out, long ldo, int nh, int hd,
+                                                                int max_pieces, long rows) {
+    const int lane = threadIdx.x & 63;
+    const long r = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= rows) return;
+    const long t = r / nh;
+    const int head = (int)(r % nh);
+    const int pieces = tok_pieces[t];
+    if (pieces <= 1) return;
+    const size_t slot0 = (size_t)r * max_pieces;
+    float ms[MERGE_MAX_PIECES], ls[MERGE_MAX_PIECES];
+#pragma unroll
+    for (int sp = 0; sp < MERGE_MAX_PIECES; ++sp) {
+        const int s2 = sp < pieces ? sp : pieces - 1;
+        ms[sp] = part_ml[(slot0 + s2) * 2];
+        ls[sp] = part_ml[(slot0 + s2) * 2 + 1];
+    }
+    for (int d0 = lane * 4; d0 < hd; d0 += 256) {
+        float4 v[MERGE_MAX_PIECES];
+#pragma unroll
+        for (int sp = 0; sp < MERGE_MAX_PIECES; ++sp) {
+            const int s2 = sp < pieces ? sp : pieces - 1;
+            v[sp] = *reinterpret_cast<const float4*>(part_o + (slot0 + s2) * hd + d0);
+        }
+        float m = -INFINITY;
+#pragma unroll
+        for (int sp = 0; sp < MERGE_MAX_PIECES; ++sp)
+            if (sp < pieces) m = fmaxf(m, ms[sp]);
+        float l = 0.f;
+        float4 acc = float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int sp = 0; sp < MERGE_MAX_PIECES; ++sp) {
+            const float f = (sp < pieces && ms[sp] != -INFINITY) ? __expf(ms[sp] - m) : 0.f;
+            l += ls[sp] * f;
+            acc.x += v[sp].x * f;
+            acc.y += v[sp].y * f;
+            acc.z += v[sp].z * f;
+            acc.w += v[sp].w * f;
+        }
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        uint2 u;
+        u.x = f32x2_to_bf16x2(acc.x * inv, acc.y * inv);
+        u.y = f32x2_to_bf16x2(acc.z * inv, acc.w * inv);
+        *reinterpret_cast<uint2*>(out + (size_t)t * ldo + (size_t)head * hd + d0) = u;
+    }
+}
+
 // ------------------------------------------------------------------ prefill, streamlined (head sizes 64, 128, 256)
 // The same frame as attn_prefill_mfma_kernel (a workgroup's waves share each page through LDS,
 // two pages in flight), with the decode kernel's inner loop: half pages as units, head size
@@ -845,23 +866,19 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(AttnArgs a, int 
 // 8: a page fetched into LDS then serves 64 positions instead of 32, which halves the traffic
 // from L2 that bounds this kernel, and two waves share a SIMD).
 template <int HDT, int NWV>
-__global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a, int hw) {
+__global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a, const PrefillItem* __restrict__ items, int nkc,
+                                                                   int hw, int max_pieces) {
     constexpr int KS = HDT / 2, hd = HDT * 16;
     constexpr int n_k = 4 * KS, n_v = HDT * 2, buf_tiles = n_k + n_v;         // tiles (of 64 uint4) per page
     extern __shared__ __attribute__((aligned(16))) uint4 page_lds[];          // [2][K tiles | V tiles][64]
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, j = lane & 15, g = lane >> 4;
+    const PrefillItem it = items[blockIdx.x / nkc];
     const int G = a.nh / a.nkv;
     const int chunks = (G + hw - 1) / hw;
-    const int kvh = blockIdx.y / chunks, chunk = blockIdx.y % chunks;
-    const int b = blockIdx.z;
+    const int kvhc = blockIdx.x % nkc, kvh = kvhc / chunks, chunk = kvhc % chunks;
+    const int b = it.seq;
     const int t0 = a.cu[b], n_new = a.cu[b + 1] - t0;
-    const int blk_len = (NWV / hw) * 16;                         // positions a workgroup covers
-    // a.splits workgroups share a block of positions: each takes a run of the block's pages and
-    // leaves partial results, which attn_combine_kernel merges (a prompt of a few thousand tokens
-    // has too few blocks to fill the compute units otherwise)
-    const int split = blockIdx.x % a.splits;
-    const int blk0 = (blockIdx.x / a.splits) * blk_len;
-    if (blk0 >= n_new) return;                                   // the whole workgroup leaves
+    const int blk0 = it.blk0;                                    // the block is (NWV / hw) * 16 positions long
     const int tile0 = blk0 + (wave / hw) * 16;                   // first step-token of this wave's tile
     const int gh = chunk * hw + wave % hw;                       // this wave's head within the group
     const bool wave_on = tile0 < n_new && gh < G;
@@ -889,16 +906,8 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     const int p_min = __shfl(p, 0, 64), p_max = __shfl(p, 15, 64);
     const int lo_min = __shfl(lo, 0, 64), lo_max = __shfl(lo, 15, 64);
     const int my_first = lo_min / AGAVE_PAGE, my_last = p_max / AGAVE_PAGE;
-    // the workgroup: positions are consecutive within the step
-    const int p_blk0 = a.tok_pos[t0 + blk0];
-    const int blk_n = (n_new - blk0 < blk_len) ? n_new - blk0 : blk_len;
-    const int lo_blk = a.window > 0 ? (p_blk0 - a.window + 1 > 0 ? p_blk0 - a.window + 1 : 0) : 0;
-    int page_first = lo_blk / AGAVE_PAGE, page_last = (p_blk0 + blk_n - 1) / AGAVE_PAGE;
-    if (a.splits > 1) {
-        const int per = (page_last - page_first + a.splits) / a.splits;
-        page_first += split * per;
-        if (page_last > page_first + per - 1) page_last = page_first + per - 1;     // (may leave no page at all)
-    }
+    const int page_first = it.page_first;
+    int page_last = it.page_first + it.n_pages - 1;
 
     // The ids of the pages this workgroup goes through, looked up once: a lookup inside the loop
     // is two dependent loads from memory a page, and waiting for them also waits for the next
@@ -1012,10 +1021,10 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     const int head = kvh * G + gh;
-    if (a.splits > 1) {
-        // sums as they stand, with the reference they are relative to (in natural logarithms, as the combine pass reads it)
+    if (it.n_pieces > 1) {
+        // sums as they stand, with the reference they are relative to (in natural logarithms, as the merge reads it)
         if (g == 0 && col_ok) {
-            const size_t ps = ((size_t)(t0 + tile0 + j) * a.nh + head) * a.splits + split;
+            const size_t ps = ((size_t)(t0 + tile0 + j) * a.nh + head) * max_pieces + it.piece;
             a.part_ml[ps * 2 + 0] = m_ref * 0.6931471805599453f;
             a.part_ml[ps * 2 + 1] = l;
         }
@@ -1023,7 +1032,7 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
         for (int e = 0; e < 4; ++e) {
             const int row = 4 * g + e;
             if (tile0 + row >= n_new) continue;
-            float* dst = a.part_o + (((size_t)(t0 + tile0 + row) * a.nh + head) * a.splits + split) * hd;
+            float* dst = a.part_o + (((size_t)(t0 + tile0 + row) * a.nh + head) * max_pieces + it.piece) * hd;
 #pragma unroll
             for (int d = 0; d < HDT; ++d) dst[16 * d + j] = o[d][e];
         }
@@ -1205,90 +1214,113 @@ extern "C" int agave_attn_decode_fused(const void* q, long ldq, const void* k, l
     return launch_decode<true>(a, f, N, stream, !leave_partials);
 }
 
-// How many workgroups should share a block of positions' pages in a prefill of these sizes (1:
-// none).  page_span: the most pages a block of positions reaches back over.  More than one only
-// for the streamlined kernel (head sizes 64, 128, 256) with eight waves, when its blocks leave
-// more than a third of the 256 compute units idle and every share still has four pages.
-extern "C" int agave_attn_prefill_splits(int n_seqs, int max_new, int nh, int nkv, int hd, int page_span) {
-    if (n_seqs <= 0 || max_new <= 32 || nkv <= 0 || nh % nkv != 0 || !(hd == 64 || hd == 128 || hd == 256)) return 1;
-    const int G = nh / nkv;
-    const int hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
-    const int blk_len = (8 / hw) * 16;
-    const long wgs = (long)((max_new + blk_len - 1) / blk_len) * nkv * ((G + hw - 1) / hw) * n_seqs;
-    int s = (int)(256 / (wgs > 0 ? wgs : 1));
-    if (wgs > 170) s = 1;
-    if (s > 4) s = 4;
-    while (s > 1 && page_span / s < 4) --s;
-    return s < 1 ? 1 : s;
-}
-
-// splits > 1 (only what agave_attn_prefill_splits gives): part_o [N][nh][splits][hd] and part_ml
-// [N][nh][splits][2], 32-bit, take the partial results.
+// A step that brings several tokens per sequence, any head size that is a multiple of 16 up to
+// 256 (the general kernel; head sizes 64, 128 and 256 go through agave_attn_prefill_items).
 extern "C" int agave_attn_prefill_mfma(const void* q, long ldq, void* out, long ldo, const void* k_pages,
                                        const void* v_pages, const int* table, int width, const int* base,
                                        int n_pages, const int* tok_seq, const int* tok_pos, const int* cu, int n_seqs,
                                        int max_new, int N, int nh, int nkv, int hd, float scale, int window,
-                                       float* part_o, float* part_ml, int splits, hipStream_t stream) {
-    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
-               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, splits, 0, 0, 0};
+                                       hipStream_t stream) {
+    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, nullptr, nullptr, (const uint4*)k_pages, (const uint4*)v_pages,
+               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, 1, 0, 0, 0};
     if (check_common("attn_prefill_mfma", a, N)) return -1;
-    AGAVE_CHECK(splits >= 1 && splits <= 4, "attn_prefill_mfma: %d splits", splits);
-    AGAVE_CHECK(splits == 1 || (part_o && part_ml && max_new > 32 && (hd == 64 || hd == 128 || hd == 256)),
-                "attn_prefill_mfma: splits need the partial buffers and the eight-wave kernel's sizes");
     AGAVE_CHECK(cu && n_seqs > 0 && max_new > 0, "attn_prefill_mfma: needs the sequences' token ranges");
     AGAVE_CHECK(n_seqs <= 65535, "attn_prefill_mfma: %d sequences exceed the grid limit", n_seqs);
     if (N == 0) return 0;
     const int G = nh / nkv;
-    const bool fast = hd == 64 || hd == 128 || hd == 256;
-    const int qt_cap = fast ? 1 : (hd > 128 ? 1 : (hd > 64 ? 2 : QT_MAX));   // heads per wave: what fits the register file
+    const int qt_cap = hd > 128 ? 1 : (hd > 64 ? 2 : QT_MAX);   // heads per wave: what fits the register file
     const int qt_heads = G < qt_cap ? G : qt_cap;
     // the other heads of the group go to other waves of the workgroup
     int hw = 1;
-    if (fast || hd > 128) hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
-    // the streamlined kernel takes eight waves once a sequence brings enough tokens for them
-    const int nwv = (fast && max_new > 32) ? 8 : 4;
-    const int wg_heads = qt_heads * hw, blk_len = (nwv / hw) * 16;
+    if (hd > 128) hw = G >= 4 ? 4 : (G >= 2 ? 2 : 1);
+    const int wg_heads = qt_heads * hw, blk_len = (4 / hw) * 16;
     const int chunks = (G + wg_heads - 1) / wg_heads;
     AGAVE_CHECK(nkv * chunks <= 65535, "attn_prefill_mfma: too many head chunks");
-    dim3 grid((max_new + blk_len - 1) / blk_len * splits, nkv * chunks, n_seqs);
+    dim3 grid((max_new + blk_len - 1) / blk_len, nkv * chunks, n_seqs);
     // two pages (K and V tiles) in LDS
     const size_t lds = (size_t)2 * (4 * ((hd + 31) / 32) + (hd / 16) * 2) * 64 * sizeof(uint4);
     static bool raised = false;
     if (!raised) {
-        const int cap = 144 * 1024;
         const void* fns[] = {(const void*)attn_prefill_mfma_kernel<4, QT_MAX>, (const void*)attn_prefill_mfma_kernel<8, 2>,
-                             (const void*)attn_prefill_mfma_kernel<16, 1>,
-                             (const void*)attn_prefill_fast_kernel<4, 4>, (const void*)attn_prefill_fast_kernel<8, 4>,
-                             (const void*)attn_prefill_fast_kernel<16, 4>, (const void*)attn_prefill_fast_kernel<4, 8>,
-                             (const void*)attn_prefill_fast_kernel<8, 8>, (const void*)attn_prefill_fast_kernel<16, 8>};
+                             (const void*)attn_prefill_mfma_kernel<16, 1>};
         for (const void* fn : fns)
-            AGAVE_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, cap) == hipSuccess,
+            AGAVE_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024) == hipSuccess,
                         "attn_prefill_mfma: cannot raise the LDS allowance");
         raised = true;
     }
-    // the streamlined kernel also keeps the ids of a workgroup's pages in LDS (at most the table's width)
-    const size_t lds_fast = lds + (size_t)width * sizeof(int);
-    AGAVE_CHECK(!fast || lds_fast <= 144 * 1024, "attn_prefill_mfma: a page table of %d columns does not fit the LDS", width);
-    if (fast && nwv == 8) {
-        if (hd == 64) attn_prefill_fast_kernel<4, 8><<<grid, 512, lds_fast, stream>>>(a, hw);
-        else if (hd == 128) attn_prefill_fast_kernel<8, 8><<<grid, 512, lds_fast, stream>>>(a, hw);
-        else attn_prefill_fast_kernel<16, 8><<<grid, 512, lds_fast, stream>>>(a, hw);
-    } else if (fast) {
-        if (hd == 64) attn_prefill_fast_kernel<4, 4><<<grid, 256, lds_fast, stream>>>(a, hw);
-        else if (hd == 128) attn_prefill_fast_kernel<8, 4><<<grid, 256, lds_fast, stream>>>(a, hw);
-        else attn_prefill_fast_kernel<16, 4><<<grid, 256, lds_fast, stream>>>(a, hw);
-    } else if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
+    if (hd <= 64) attn_prefill_mfma_kernel<4, QT_MAX><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else if (hd <= 128) attn_prefill_mfma_kernel<8, 2><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     else attn_prefill_mfma_kernel<16, 1><<<grid, 256, lds, stream>>>(a, qt_heads, hw);
     AGAVE_LAUNCH_CHECK("attn_prefill_mfma");
-    if (splits > 1) {
-        AGAVE_CHECK((long)N * nh < (1L << 31), "attn_prefill_mfma: too many (token, head) pairs for the combine pass");
+    return 0;
+}
+
+// A step that brings several tokens per sequence, head sizes 64, 128 and 256, cut into items by
+// the host (see PrefillItem).  items: n_items records of six ints in the order in which workgroups
+// are to take them; `waves` (4 or 8) waves a workgroup, hw = agave_attn_prefill_items_hw(nh, nkv)
+// heads side by side, so a block is (waves / hw) * 16 positions long; max_item_pages: the most
+// pages any item has; tok_pieces[t]: pieces the block of token t is cut into (part_o
+// [N][nh][max_pieces][hd] and part_ml [N][nh][max_pieces][2] take their partial results when
+// max_pieces > 1).
+extern "C" int agave_attn_prefill_items_hw(int nh, int nkv) {
+    if (nkv <= 0 || nh % nkv != 0) return 0;
+    const int G = nh / nkv;
+    return G >= 4 ? 4 : (G >= 2 ? 2 : 1);
+}
+
+extern "C" int agave_attn_prefill_items(const void* q, long ldq, void* out, long ldo, const void* k_pages,
+                                        const void* v_pages, const int* table, int width, const int* base,
+                                        int n_pages, const int* tok_seq, const int* tok_pos, const int* cu, int n_seqs,
+                                        int N, int nh, int nkv, int hd, float scale, int window, const int* items,
+                                        int n_items, int waves, int max_item_pages, const int* tok_pieces,
+                                        float* part_o, float* part_ml, int max_pieces, hipStream_t stream) {
+    AttnArgs a{(const bf16*)q, ldq, (bf16*)out, ldo, part_o, part_ml, (const uint4*)k_pages, (const uint4*)v_pages,
+               table, width, base, n_pages, tok_seq, tok_pos, cu, n_seqs, nh, nkv, hd, scale, window, 1, 0, 0, 0};
+    if (check_common("attn_prefill_items", a, N)) return -1;
+    AGAVE_CHECK(hd == 64 || hd == 128 || hd == 256, "attn_prefill_items: head_dim %d is not 64, 128 or 256", hd);
+    AGAVE_CHECK(waves == 4 || waves == 8, "attn_prefill_items: %d waves a workgroup", waves);
+    AGAVE_CHECK(cu && n_seqs > 0 && items && n_items >= 0 && max_item_pages >= 1, "attn_prefill_items: needs sequences and items");
+    AGAVE_CHECK(max_pieces >= 1 && max_pieces <= MERGE_MAX_PIECES, "attn_prefill_items: %d pieces", max_pieces);
+    AGAVE_CHECK(max_pieces == 1 || (part_o && part_ml && tok_pieces), "attn_prefill_items: pieces need the partial buffers");
+    if (N == 0 || n_items == 0) return 0;
+    const int hw = agave_attn_prefill_items_hw(nh, nkv);
+    const int G = nh / nkv, chunks = (G + hw - 1) / hw, nkc = nkv * chunks;
+    AGAVE_CHECK((long)n_items * nkc < (1L << 31), "attn_prefill_items: too many workgroups");
+    // two pages (K and V tiles) in LDS, and the ids of the item's pages
+    const size_t lds = (size_t)2 * (4 * (hd / 32) + (hd / 16) * 2) * 64 * sizeof(uint4) + (size_t)max_item_pages * sizeof(int);
+    AGAVE_CHECK(lds <= 144 * 1024, "attn_prefill_items: items of %d pages do not fit the LDS", max_item_pages);
+    static bool raised = false;
+    if (!raised) {
+        const void* fns[] = {(const void*)attn_prefill_fast_kernel<4, 4>, (const void*)attn_prefill_fast_kernel<8, 4>,
+                             (const void*)attn_prefill_fast_kernel<16, 4>, (const void*)attn_prefill_fast_kernel<4, 8>,
+                             (const void*)attn_prefill_fast_kernel<8, 8>, (const void*)attn_prefill_fast_kernel<16, 8>};
+        for (const void* fn : fns)
+            AGAVE_CHECK(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024) == hipSuccess,
+                        "attn_prefill_items: cannot raise the LDS allowance");
+        raised = true;
+    }
+    const unsigned grid = (unsigned)((long)n_items * nkc);
+    const PrefillItem* its = reinterpret_cast<const PrefillItem*>(items);
+#define PF_LAUNCH(HDT_, NWV_) \
+    attn_prefill_fast_kernel<HDT_, NWV_><<<grid, NWV_ * 64, lds, stream>>>(a, its, nkc, hw, max_pieces)
+    if (waves == 8) {
+        if (hd == 64) PF_LAUNCH(4, 8);
+        else if (hd == 128) PF_LAUNCH(8, 8);
+        else PF_LAUNCH(16, 8);
+    } else {
+        if (hd == 64) PF_LAUNCH(4, 4);
+        else if (hd == 128) PF_LAUNCH(8, 4);
+        else PF_LAUNCH(16, 4);
+    }
+#undef PF_LAUNCH
+    AGAVE_LAUNCH_CHECK("attn_prefill_items");
+    if (max_pieces > 1) {
+        AGAVE_CHECK((long)N * nh < (1L << 31) && ldo % 4 == 0 && ((uintptr_t)out % 8) == 0,
+                    "attn_prefill_items: the merge needs 8-byte aligned output rows");
         const long rows = (long)N * nh;
-        if (ldo % 4 == 0 && ((uintptr_t)out % 8) == 0 && splits <= COMBINE_ROWS_MAX_SPLITS)
-            attn_combine_rows_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, stream>>>(part_o, part_ml, a.out, a.ldo, nh, hd, splits, rows);
-        else
-            attn_combine_kernel<<<N * nh, hd >= 256 ? 256 : (hd >= 128 ? 128 : 64), 0, stream>>>(part_o, part_ml, a.out, a.ldo, nh, hd, splits);
-        AGAVE_LAUNCH_CHECK("attn_combine");
+        attn_merge_pieces_kernel<<<(unsigned)((rows + 3) / 4), 256, 0, stream>>>(part_o, part_ml, tok_pieces, a.out, a.ldo,
+                                                                                 nh, hd, max_pieces, rows);
+        AGAVE_LAUNCH_CHECK("attn_merge_pieces");
     }
     return 0;
 }

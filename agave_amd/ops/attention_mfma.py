@@ -13,9 +13,10 @@ kernels.register_signatures("attention_mfma", {
                                _I, _P],
     "agave_attn_decode_fused": [_P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F, _P, _L, _P, _P, _P, _P, _P, _I, _P, _I,
                                 _P, _P, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _P],
-    "agave_attn_prefill_mfma": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P,
-                                _I, _P],
-    "agave_attn_prefill_splits": [_I, _I, _I, _I, _I, _I],
+    "agave_attn_prefill_mfma": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "agave_attn_prefill_items_hw": [_I, _I],
+    "agave_attn_prefill_items": [_P, _L, _P, _L, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I,
+                                 _I, _P, _P, _P, _I, _P],
 })
 
 TARGET_WORKGROUPS = 256      # workgroups (of 4 waves) a decode launch aims for: one per compute unit
@@ -40,6 +41,82 @@ def split_plan(page_span: int, units: int, head_dim: int = 0):
 
 MAX_SPLITS = 64              # what the merge inside the output product takes
 FUSED_HEAD_DIMS = (64, 128, 256)
+
+
+ITEM_PLACES = 256            # workgroups of the item kernel that run at a time: one a compute unit
+ITEM_MIN_PAGES = 4           # pages an item holds at least (what an item costs besides its pages is about a page)
+ITEM_MAX_PIECES = 4
+ITEM_MAX_PARTIAL_BYTES = 1 << 30
+
+
+def plan_prefill_items(pos0, n_new, window: Optional[int], blk_len: int, heads_of_block: int, n_heads: int,
+                       head_dim: int):
+    """Cut a step of several tokens per sequence into items of about equal work for the item
+    kernel.  A block is ``blk_len`` consecutive tokens of a sequence; it sees the pages from the
+    window's edge of its first token to its last token.  With ``heads_of_block`` workgroups per
+    item (kv heads times head chunks) and ITEM_PLACES workgroups running at a time, an item should
+    hold about total / places pages; a block that sees more is cut into up to four pieces (whose
+    partial results a second kernel merges), unless the partial results of the whole step would
+    not fit a gigabyte.  Returns (items [n, 6] int32 sorted by falling size, pieces per token [N]
+    int32, most pieces, most pages of an item)."""
+    import numpy as np
+    blocks = []                                   # (sequence, first token within the sequence, first page, pages)
+    for b, (p0, n) in enumerate(zip(pos0, n_new)):
+        for blk0 in range(0, n, blk_len):
+            first, last = p0 + blk0, p0 + min(n, blk0 + blk_len) - 1
+            lo = max(0, first - window + 1) if window else 0
+            blocks.append((b, blk0, lo // 64, last // 64 - lo // 64 + 1))
+    total = sum(blk[3] for blk in blocks) * heads_of_block
+    per_item = max(ITEM_MIN_PAGES, -(-total // ITEM_PLACES))
+    n_tokens = sum(n_new)
+    may_cut = n_tokens * n_heads * ITEM_MAX_PIECES * (head_dim + 2) * 4 <= ITEM_MAX_PARTIAL_BYTES
+    items = []
+    tok_pieces = np.ones(n_tokens, dtype=np.int32)
+    starts = np.concatenate([[0], np.cumsum(n_new)])
+    max_pieces = 1
+    for b, blk0, pg0, npg in blocks:
+        pieces = min(ITEM_MAX_PIECES, -(-npg // per_item)) if may_cut else 1
+        max_pieces = max(max_pieces, pieces)
+        if pieces > 1:
+            tok_pieces[starts[b] + blk0:starts[b] + min(n_new[b], blk0 + blk_len)] = pieces
+        for k in range(pieces):
+            lo, hi = k * npg // pieces, (k + 1) * npg // pieces
+            items.append((b, blk0, pg0 + lo, hi - lo, k, pieces))
+    items.sort(key=lambda it: -it[3])
+    arr = np.asarray(items, dtype=np.int32).reshape(-1, 6)
+    return arr, tok_pieces, max_pieces, int(arr[:, 3].max()) if len(items) else 1
+
+
+def prefill_by_items(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                     table: torch.Tensor, base: torch.Tensor, step, n_heads: int, n_kv: int, head_dim: int,
+                     scale: float, window: Optional[int], width: int, n_pages: int) -> None:
+    """Attention of a step that brings several tokens per sequence, head sizes 64, 128 and 256."""
+    import numpy as np
+    lib = kernels.lib("attention_mfma")
+    hw = int(lib.agave_attn_prefill_items_hw(n_heads, n_kv))
+    waves = 8 if step.max_new > 32 else 4          # eight waves once a sequence brings enough tokens for them
+    blk_len = (waves // hw) * 16
+    chunks = -(-(n_heads // n_kv) // hw)
+    cache = step.__dict__.setdefault("_prefill_items", {})
+    key = (window, blk_len, n_kv * chunks, n_heads, head_dim)
+    plan = cache.get(key)
+    if plan is None:
+        items, tok_pieces, max_pieces, max_item_pages = plan_prefill_items(step.pos0, step.n_new, window, blk_len,
+                                                                           n_kv * chunks, n_heads, head_dim)
+        both = torch.from_numpy(np.concatenate([items.reshape(-1), tok_pieces])).to(q.device)
+        plan = cache[key] = (both[:items.size].view(-1, 6), both[items.size:], max_pieces, max_item_pages)
+    items_dev, pieces_dev, max_pieces, max_item_pages = plan
+    n = step.n_tokens
+    part_o = part_ml = None
+    if max_pieces > 1:
+        ws = step.workspace
+        part_o = ws.get("attn_part_o", n * n_heads * max_pieces, head_dim, torch.float32)
+        part_ml = ws.get("attn_part_ml", n * n_heads * max_pieces, 2, torch.float32)
+    library.call(lib, "agave_attn_prefill_items", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+                 k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width, base.data_ptr(), n_pages,
+                 step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), step.cu_dev.data_ptr(), step.n_seqs, n, n_heads, n_kv,
+                 head_dim, scale, int(window or 0), items_dev.data_ptr(), items_dev.shape[0], waves, max_item_pages,
+                 pieces_dev.data_ptr(), kernels.ptr(part_o), kernels.ptr(part_ml), max_pieces, kernels.stream())
 
 
 def check_table_reach(pos0, n_new, window: Optional[int], base, width: int) -> None:
@@ -89,20 +166,13 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
                      step.tok_pos.data_ptr(), n, n_heads, n_kv, head_dim, scale, w, splits, per,
                      1 if step.n_seqs == n else 0, 1 if getattr(step, "tables_start_at_reach", False) else 0,
                      kernels.stream())
+    elif head_dim in FUSED_HEAD_DIMS:
+        prefill_by_items(q, out, k_pages, v_pages, table, base, step, n_heads, n_kv, head_dim, scale, window, width, n_pages)
     else:
-        # a prompt with few blocks of positions: several workgroups share a block's pages
-        splits = int(lib.agave_attn_prefill_splits(step.n_seqs, step.max_new, n_heads, n_kv, head_dim,
-                                                   step.page_span(window)))
-        part_o = part_ml = None
-        if splits > 1:
-            ws = step.workspace
-            part_o = ws.get("attn_part_o", n * n_heads * splits, head_dim, torch.float32)
-            part_ml = ws.get("attn_part_ml", n * n_heads * splits, 2, torch.float32)
         library.call(lib, "agave_attn_prefill_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
                      k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width, base.data_ptr(), n_pages,
                      step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), step.cu_dev.data_ptr(), step.n_seqs,
-                     step.max_new, n, n_heads, n_kv, head_dim, scale, w, kernels.ptr(part_o), kernels.ptr(part_ml),
-                     splits, kernels.stream())
+                     step.max_new, n, n_heads, n_kv, head_dim, scale, w, kernels.stream())
 
 
 def decode_fused(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], out: torch.Tensor,

@@ -235,3 +235,34 @@ def test_a_table_narrower_than_a_step_s_reach_is_refused_on_the_host():
         check_table_reach([1000], [70], 100, [15], 3)                    # the row starts after page 14
     with pytest.raises(ValueError, match="reach back"):
         check_table_reach([1000], [1], None, [3], 64)                    # all keys: the row must start at page 0
+
+
+@pytest.mark.parametrize("pos0,n_new,window,blk_len", [([0], [2048], 1024, 64), ([0], [2048], None, 64),
+                                                       ([5, 0, 100], [1, 70, 300], 70, 32), ([4000], [200], 1500, 64),
+                                                       ([0, 0, 0], [33, 4096, 640], 1024, 64)])
+def test_the_items_of_a_prefill_step_cover_every_block_and_page_once(pos0, n_new, window, blk_len):
+    """The host cuts a step of several tokens per sequence into items (a block of positions and a
+    run of the pages it sees): together they cover each block's reach exactly once, the pieces of a
+    block are runs that follow each other, the list starts with the largest, and every token knows
+    how many pieces its block has."""
+    import numpy as np
+    from agave_amd.ops.attention_mfma import ITEM_MAX_PIECES, plan_prefill_items
+    items, tok_pieces, max_pieces, max_pages = plan_prefill_items(pos0, n_new, window, blk_len, 4, 8, 256)
+    assert items.dtype == np.int32 and items.shape[1] == 6 and 1 <= max_pieces <= ITEM_MAX_PIECES
+    assert list(items[:, 3]) == sorted(items[:, 3], reverse=True) and max_pages == items[:, 3].max()
+    starts = np.concatenate([[0], np.cumsum(n_new)])
+    seen = {}
+    for b, blk0, pg0, npg, piece, pieces in items.tolist():
+        assert npg >= 1 and 0 <= piece < pieces <= max_pieces
+        seen.setdefault((b, blk0), []).append((piece, pg0, npg, pieces))
+    for b, (p0, n) in enumerate(zip(pos0, n_new)):
+        for blk0 in range(0, n, blk_len):
+            first, last = p0 + blk0, p0 + min(n, blk0 + blk_len) - 1
+            lo = max(0, first - window + 1) if window else 0
+            got = sorted(seen.pop((b, blk0)))
+            assert [g[0] for g in got] == list(range(got[0][3])) and all(g[3] == got[0][3] for g in got)
+            assert got[0][1] == lo // 64 and got[-1][1] + got[-1][2] - 1 == last // 64
+            for x, y in zip(got, got[1:]):
+                assert x[1] + x[2] == y[1]                        # runs that follow each other
+            assert (tok_pieces[starts[b] + blk0:starts[b] + min(n, blk0 + blk_len)] == got[0][3]).all()
+    assert not seen and len(tok_pieces) == sum(n_new)

@@ -718,12 +718,12 @@ def test_attn_mfma_prefill_of_tens_of_thousands_of_tokens(K, nh, nkv, hd, L, win
 @pytest.mark.parametrize("nh,nkv,hd,lens,window", [(4, 2, 128, [1500], None), (4, 2, 128, [1500], 1024),
                                                    (8, 4, 256, [700, 300], None), (2, 2, 64, [1100, 64, 1], 600)])
 def test_attn_mfma_prefill_blocks_shared_among_workgroups(K, nh, nkv, hd, lens, window):
-    """A prompt with few blocks of positions: several workgroups share a block's pages and a
-    second pass merges what they leave."""
-    from agave_amd.ops import attention_mfma, kernels
-    step = _FakeStep(lens, lambda L: 0, window)
-    lib = kernels.lib("attention_mfma")
-    assert lib.agave_attn_prefill_splits(len(lens), max(lens), nh, nkv, hd, step.page_span(window)) > 1
+    """A prompt with few blocks of positions: the blocks with a long reach are cut into pieces
+    that go to workgroups of their own, and a second pass merges what they leave."""
+    from agave_amd.ops import attention_mfma
+    hw = 2 if nh // nkv >= 2 else 1
+    plan = attention_mfma.plan_prefill_items([0] * len(lens), lens, window, (8 // hw) * 16, nkv, nh, hd)
+    assert plan[2] > 1 and (plan[1] > 1).any() and (plan[1] == 1).any()      # some blocks in pieces, some whole
     got, ref, _ = _mfma_attn_case(K, nh, nkv, hd, lens, window, 0.3 * (16 / hd) ** 0.5, False, seed=7)
     assert torch.isfinite(got).all()
     assert torch.allclose(got, ref, atol=2e-2, rtol=2e-2)
