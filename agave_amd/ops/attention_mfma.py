@@ -43,9 +43,10 @@ MAX_SPLITS = 64              # what the merge inside the output product takes
 FUSED_HEAD_DIMS = (64, 128, 256)
 
 
-ITEM_PLACES = 256            # workgroups of the item kernel that run at a time: one a compute unit
+ITEM_PLACES = 192            # items are sized as if three quarters of the compute units' places were there: measured,
+                             # fewer and larger pieces beat an even share (a piece more costs its partial results)
 ITEM_MIN_PAGES = 4           # pages an item holds at least (what an item costs besides its pages is about a page)
-ITEM_MAX_PIECES = 4
+ITEM_MAX_PIECES = 3
 ITEM_MAX_PARTIAL_BYTES = 1 << 30
 
 
@@ -55,7 +56,7 @@ def plan_prefill_items(pos0, n_new, window: Optional[int], blk_len: int, heads_o
     kernel.  A block is ``blk_len`` consecutive tokens of a sequence; it sees the pages from the
     window's edge of its first token to its last token.  With ``heads_of_block`` workgroups per
     item (kv heads times head chunks) and ITEM_PLACES workgroups running at a time, an item should
-    hold about total / places pages; a block that sees more is cut into up to four pieces (whose
+    hold about total / places pages; a block that sees more is cut into up to three pieces (whose
     partial results a second kernel merges), unless the partial results of the whole step would
     not fit a gigabyte.  Returns (items [n, 6] int32 sorted by falling size, pieces per token [N]
     int32, most pieces, most pages of an item)."""
