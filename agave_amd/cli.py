@@ -10,7 +10,7 @@ quantised caches, vision, speculative decoding, its single-dispatch kernel and g
 counterpart here.  There is no tokenizer in this library: a prompt is a list
 of token ids ("2 17 5" or "2,17,5"), and the output is token ids.
 
-Added: ``--prompt-file`` (one request per line), ``--dtype``, ``--max-batch``, ``--ignore-eos``, ``--cast-weights``,
+Added: ``--prompt-file`` (one request per line), ``--dtype``, ``--max-batch``, ``--ignore-eos``, ``--logprobs``, ``--cast-weights``,
 ``--random-weights CONFIG.json`` (write a random model folder at <model> first).
 """
 from __future__ import annotations
@@ -60,6 +60,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--dtype", choices=["bfloat16", "float32", "bf16", "fp32"], default="bfloat16")
     ap.add_argument("--max-batch", type=int, default=8, help="sequences per batch [default: 8]")
     ap.add_argument("--ignore-eos", action="store_true", help="do not stop at end-of-sequence ids")
+    ap.add_argument("--logprobs", action="store_true", help="with --json: the log-probability of every generated token")
     ap.add_argument("--no-bos", action="store_true", help="do not prepend the begin-of-sequence id")
     ap.add_argument("--cast-weights", action="store_true",
                     help="cast matrices that the checkpoint stores in 32-bit to the engine's dtype (default: they stay 32-bit)")
@@ -142,7 +143,7 @@ def main(argv: Optional[List[str]] = None) -> int:
             print(f"[debug] request {i}: {len(p)} prompt token ids: {' '.join(map(str, p))}", file=sys.stderr)
     params = SamplingParams(max_tokens=args.max_tokens, temperature=args.temperature, top_k=args.top_k,
                             top_p=args.top_p, repeat_penalty=args.repeat_penalty, seed=args.seed,
-                            ignore_eos=args.ignore_eos)
+                            ignore_eos=args.ignore_eos, logprobs=args.logprobs)
     stats = GenerationStats()
     engine.prefill_chunk = max(0, args.prefill_batch_size)
     if args.profile:
@@ -158,7 +159,8 @@ def main(argv: Optional[List[str]] = None) -> int:
         extra = {"profile": [{"op": n, "calls": c, "ms": round(ms, 3)} for n, c, ms in table]} if table else {}
         print(json.dumps({**extra,
             "outputs": [{"request": r.request, "tokens": r.tokens, "finish_reason": r.finish_reason,
-                         "prompt_tokens": r.prompt_tokens} for r in results],
+                         "prompt_tokens": r.prompt_tokens,
+                         **({"logprobs": [round(x, 6) for x in r.logprobs]} if args.logprobs else {})} for r in results],
             "tokens": stats.tokens, "tok_per_sec": round(stats.tok_per_sec, 2),
             "prefill_tokens": stats.prefill_tokens, "prefill_ms": round(stats.prefill_ms, 3),
             "prefill_tok_per_sec": round(stats.prefill_tok_per_sec, 2), "gen_ms": round(stats.gen_ms, 3),

@@ -893,6 +893,60 @@ extern "C" int agave_repeat_penalty(float* logits, long ld, const int* ids, cons
 }
 
 
+// ------------------------------------------------------------------ log-probability of the drawn token
+// out[b] = logits[b][tok[b]] - log sum_v exp(logits[b][v]): the natural logarithm of the model's
+// probability of the token that was drawn, from the row as the sampler saw it (temperature and
+// filters are the sampler's own business and leave this number alone).  One workgroup a row; every
+// thread keeps a running maximum and a sum relative to it, merged pairwise at the end.
+__global__ __launch_bounds__(1024) void token_logprob_kernel(const float* __restrict__ logits, long ld,
+                                                             const int* __restrict__ tok, float* __restrict__ out, int V) {
+    __shared__ float sm[16], ss[16];
+    const float* x = logits + (size_t)blockIdx.x * ld;
+    float m = -INFINITY, s = 0.f;
+    for (int i = threadIdx.x; i < V; i += blockDim.x) {
+        const float v = x[i];
+        if (v > m) {
+            s = s * expf(m - v) + 1.0f;          // (m = -inf: s is 0 and stays so)
+            m = v;
+        } else if (v > -INFINITY) {
+            s += expf(v - m);
+        }
+    }
+    // the wave, then the workgroup: (m, s) pairs merge as s1 e^(m1 - m) + s2 e^(m2 - m)
+    for (int off = 32; off > 0; off >>= 1) {
+        const float m2 = __shfl_xor(m, off, 64), s2 = __shfl_xor(s, off, 64);
+        const float mm = fmaxf(m, m2);
+        s = (m > -INFINITY ? s * expf(m - mm) : 0.f) + (m2 > -INFINITY ? s2 * expf(m2 - mm) : 0.f);
+        m = mm;
+    }
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    if ((threadIdx.x & 63) == 0) {
+        sm[wave] = m;
+        ss[wave] = s;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float mm = -INFINITY;
+        for (int w = 0; w < nw; ++w) mm = fmaxf(mm, sm[w]);
+        float tot = 0.f;
+        for (int w = 0; w < nw; ++w)
+            if (sm[w] > -INFINITY) tot += ss[w] * expf(sm[w] - mm);
+        const int t = tok[blockIdx.x];
+        out[blockIdx.x] = (t >= 0 && t < V && tot > 0.f) ? x[t] - mm - logf(tot) : -INFINITY;
+    }
+}
+
+extern "C" int agave_token_logprob(const float* logits, long ld, const int* tok, float* out, int B, int V,
+                                   hipStream_t stream) {
+    AGAVE_CHECK(B >= 0 && V > 0 && ld >= V, "token_logprob: bad sizes B=%d V=%d ld=%ld", B, V, ld);
+    AGAVE_CHECK(B == 0 || (logits && tok && out), "token_logprob: null buffer");
+    if (B == 0) return 0;
+    token_logprob_kernel<<<B, V >= 1024 ? 1024 : 256, 0, stream>>>(logits, ld, tok, out, V);
+    AGAVE_LAUNCH_CHECK("token_logprob");
+    return 0;
+}
+
+
 // ------------------------------------------------------------------ sampled tokens feed the next step
 // dst[i] = src[map[i]]: the tokens a step sampled become the next step's input on the device, so
 // that the host can launch that step before it has read them.

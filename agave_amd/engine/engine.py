@@ -315,21 +315,31 @@ class Engine:
         scratch = self.workspace.get("sample_scratch", b, sample_ops.scratch_words(), torch.float32).view(-1)
         sample_ops.sample(logits, work, step.floats_dev.view(b, 4), out, scratch,
                           kinds=sample_ops.kinds_of(rows, self.spec.vocab_size))
+        # the host gets the tokens, and behind them the drawn tokens' log-probabilities (as bits) if any row wants them
+        want_lp = any(getattr(r, "logprob", False) for r in rows)
+        lp_dev = None
+        if want_lp:
+            lp_dev = self.workspace.get("sampled_logprob", self.max_slots, 1, torch.float32).view(-1)[:b]
+            sample_ops.token_logprob(logits, out, lp_dev)
         self._result_turn = 1 - getattr(self, "_result_turn", 0)
         hosts = getattr(self, "_result_hosts", None)
         if hosts is None:
-            hosts = self._result_hosts = [torch.empty(self.max_slots, dtype=torch.int32, pin_memory=True)
+            hosts = self._result_hosts = [torch.empty(2 * self.max_slots, dtype=torch.int32, pin_memory=True)
                                           for _ in range(2)]
         host = hosts[self._result_turn]
         host[:b].copy_(out, non_blocking=True)
+        if want_lp:
+            host[self.max_slots:self.max_slots + b].copy_(lp_dev.view(torch.int32), non_blocking=True)
         done = torch.cuda.Event()
         done.record()
-        return host, done, b
+        return host, done, b, want_lp
 
     def finish_step(self, handle) -> List[int]:
         """The tokens of a step that :meth:`launch_step` enqueued (waits for it)."""
-        host, done, b = handle
+        host, done, b, want_lp = handle
         done.synchronize()
+        # (what generation reads after every step: the step's log-probabilities, or None)
+        self.last_logprobs = host[self.max_slots:self.max_slots + b].view(torch.float32).tolist() if want_lp else None
         return host[:b].tolist()
 
     def generate(self, prompts, params=None, max_batch: Optional[int] = None, stats=None):

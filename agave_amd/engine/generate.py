@@ -43,6 +43,7 @@ class RowSampling:
     repeat_penalty: float
     u: float                     # uniform draw in [0, 1) of this request's own stream
     generated: List[int]         # ids generated so far (for the repeat penalty)
+    logprob: bool = False        # the drawn token's log-probability is wanted
 
 
 @dataclass
@@ -96,20 +97,22 @@ def generate(backend, prompts: Sequence[Sequence[int]],
     def row(i: int) -> RowSampling:
         p = plist[i]
         u = float(rngs[i].random(dtype=np.float32)) if p.temperature > 0 else 0.0
-        return RowSampling(p.temperature, p.top_k, p.top_p, p.repeat_penalty, u, results[i].tokens)
+        return RowSampling(p.temperature, p.top_k, p.top_p, p.repeat_penalty, u, results[i].tokens, p.logprobs)
 
     ahead = hasattr(backend, "launch_step") and all(p.repeat_penalty == 1.0 for p in plist)
     cancel_requested = getattr(backend, "cancel_requested", lambda: False)
     if hasattr(backend, "clear_cancel"):
         backend.clear_cancel()              # a request to cancel belongs to the call it arrived in
 
-    def settle(i: int, tok: int) -> None:
+    def settle(i: int, tok: int, logprob: Optional[float] = None) -> None:
         """Book the token request i drew; sets its finish reason if it ends here."""
         r = results[i]
         if tok in stops[i]:
             r.finish_reason = "stop"                      # the end token is not emitted
         else:
             r.tokens.append(tok)
+            if plist[i].logprobs and logprob is not None:
+                r.logprobs.append(logprob)
             stats.tokens += 1
             if len(r.tokens) >= plist[i].max_tokens:
                 r.finish_reason = "length"
@@ -139,8 +142,9 @@ def generate(backend, prompts: Sequence[Sequence[int]],
                         stats.decode_tokens += len(live)
                     first = False
                     nxt = []
-                    for i, tok in zip(live, sampled):
-                        settle(i, int(tok))
+                    lps = getattr(backend, "last_logprobs", None) or [None] * len(live)
+                    for i, tok, lp in zip(live, sampled, lps):
+                        settle(i, int(tok), lp)
                         if results[i].finish_reason:
                             backend.free_slot(slots.pop(i))               # given back at once
                         else:
@@ -169,11 +173,12 @@ def generate(backend, prompts: Sequence[Sequence[int]],
                     stats.prefill_ms += ms
                 else:
                     stats.gen_ms += ms
-                for i, tok in zip(live, sampled):
+                lps = getattr(backend, "last_logprobs", None) or [None] * len(live)
+                for i, tok, lp in zip(live, sampled, lps):
                     if results[i].finish_reason:
                         backend.free_slot(slots.pop(i))       # ended a step ago; no step uses its slot now
                         continue
-                    settle(i, int(tok))
+                    settle(i, int(tok), lp)
                     if not first:
                         stats.decode_tokens += 1
                     if results[i].finish_reason and i not in on:

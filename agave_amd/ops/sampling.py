@@ -12,6 +12,7 @@ kernels.register_signatures("sampling", {
     "agave_sample": [_P, _L, _P, _L, _P, _P, _I, _I, _P, _I, _P],
     "agave_repeat_penalty": [_P, _L, _P, _P, _P, _I, _I, _P],
     "agave_gather_tokens": [_P, _P, _P, _I, _I, _P],
+    "agave_token_logprob": [_P, _L, _P, _P, _I, _I, _P],
 })
 
 
@@ -96,3 +97,15 @@ def gather_tokens(src: torch.Tensor, index: torch.Tensor, dst: torch.Tensor) -> 
         raise ValueError("gather_tokens: one index per destination")
     library.call(kernels.lib("sampling"), "agave_gather_tokens", src.data_ptr(), index.data_ptr(), dst.data_ptr(),
                  dst.numel(), src.numel(), kernels.stream())
+
+
+def token_logprob(logits: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
+    """out[b] = log softmax(logits[b])[tokens[b]] (natural logarithm, float32)."""
+    ld = _logits(logits)
+    b, v = logits.shape
+    if tokens.dtype != torch.int32 or tokens.numel() != b or not tokens.is_contiguous() or not tokens.is_cuda:
+        raise TypeError(f"token_logprob: tokens must be {b} contiguous int32 on the GPU")
+    if out.dtype != torch.float32 or out.numel() != b or not out.is_contiguous() or not out.is_cuda:
+        raise TypeError(f"token_logprob: out must be {b} contiguous float32 on the GPU")
+    library.call(kernels.lib("sampling"), "agave_token_logprob", logits.data_ptr(), ld, tokens.data_ptr(),
+                 out.data_ptr(), b, v, kernels.stream())

@@ -20,6 +20,7 @@ class SamplingParams:
     seed: Optional[int] = None       # None: taken from the clock, once per call
     stop_ids: Tuple[int, ...] = ()   # on top of the model's end-of-sequence ids
     ignore_eos: bool = False         # benchmarks: run to max_tokens
+    logprobs: bool = False           # also return log p(token) of every emitted token (the reference has none)
 
     def __post_init__(self):
         if self.max_tokens < 1:
@@ -39,6 +40,8 @@ class GenerationResult:
     request: int                     # index of the prompt in the call
     prompt_tokens: int
     tokens: List[int] = field(default_factory=list)
+    logprobs: List[float] = field(default_factory=list)      # one per token, if asked for: natural logarithm of the
+                                                             # model's probability, from the logits the sampler saw
     finish_reason: str = ""          # "stop" (an end token was drawn; it is not emitted),
                                      # "length" (max_tokens), "context" (the slot is full),
                                      # "cancelled" (the call was cancelled before the request ended)

@@ -290,3 +290,38 @@ def test_more_kinds_of_decode_steps_than_graphs_are_kept(model_b, dtype):
     assert len(kept) <= 4 and a.graphs.evicted >= 14
     assert sorted(k[0] for k in kept) == [1, 2, 3, 4], kept          # the batch sizes that ran last
     assert not b.graphs._graphs
+
+
+def test_log_probabilities_of_the_generated_tokens(model_b):
+    """Requests that ask for them get, with every emitted token, the natural logarithm of the model's
+    probability of that token (from the logits as the sampler saw them), whatever way it was drawn
+    and whether steps run ahead or not; a stop token is not emitted and neither is its number."""
+    import math
+    from agave_amd import Engine, SamplingParams
+    cfg, w, folder = model_b
+    eng = Engine.from_folder(folder, dtype="float32", max_slots=3, max_context=96)
+    prompts = [U.random_tokens(n, cfg["vocab_size"], 600 + i) for i, n in enumerate((4, 21, 9))]
+    sps = [SamplingParams(max_tokens=7, logprobs=True, ignore_eos=True),
+           SamplingParams(max_tokens=5, temperature=0.9, seed=3, ignore_eos=True),                      # does not ask
+           SamplingParams(max_tokens=6, temperature=1.3, top_k=20, seed=4, logprobs=True, ignore_eos=True)]
+    res = eng.generate(prompts, sps)
+    assert res[1].logprobs == [] and len(res[0].logprobs) == 7 and len(res[2].logprobs) == 6
+    for i in (0, 2):
+        toks = list(prompts[i])
+        for tok, lp in zip(res[i].tokens, res[i].logprobs):
+            row = P.forward(cfg, w, toks)[-1].double()
+            want = float(row[tok] - torch.logsumexp(row, 0))
+            assert math.isclose(lp, want, rel_tol=0, abs_tol=2e-4), (i, len(toks), lp, want)
+            toks.append(tok)
+    # with a repeat penalty (steps do not run ahead then) and a stop token
+    stop = res[0].tokens[3]
+    one = eng.generate([prompts[0]], SamplingParams(max_tokens=7, logprobs=True, repeat_penalty=1.0, stop_ids=(stop,)))[0]
+    assert one.finish_reason == "stop" and one.tokens == res[0].tokens[:3] and len(one.logprobs) == 3
+    assert all(math.isclose(a, b, abs_tol=1e-5) for a, b in zip(one.logprobs, res[0].logprobs))
+    pen = eng.generate([prompts[0]], SamplingParams(max_tokens=4, logprobs=True, repeat_penalty=1.4, ignore_eos=True))[0]
+    toks, out = list(prompts[0]), []
+    for tok, lp in zip(pen.tokens, pen.logprobs):
+        row = P.apply_repeat_penalty(P.forward(cfg, w, toks)[-1], out, 1.4).double()
+        assert tok == P.argmax_first(row) and math.isclose(lp, float(row[tok] - torch.logsumexp(row, 0)), abs_tol=2e-4)
+        toks.append(tok)
+        out.append(tok)

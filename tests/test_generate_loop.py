@@ -240,3 +240,16 @@ def test_a_cancelled_call_returns_what_it_has_and_loses_no_slot(backend_cls):
     be = Cancellable(10 ** 9, max_slots=2, max_context=64)
     res = generate(be, [[10], [20]], SamplingParams(max_tokens=6), eos_ids=[])
     assert [r.finish_reason for r in res] == ["length", "length"]
+
+
+def test_log_probabilities_go_to_the_requests_that_ask():
+    class WithLogprobs(FakeBackend):
+        def step_sample(self, slots, tokens, rows):
+            out = super().step_sample(slots, tokens, rows)
+            self.last_logprobs = [-(t + 1) / 10 for t in out] if any(r.logprob for r in rows) else None
+            return out
+
+    be = WithLogprobs()
+    res = generate(be, [[10], [20]], [SamplingParams(max_tokens=3, logprobs=True), SamplingParams(max_tokens=3)], eos_ids=[13])
+    assert res[0].tokens == [11, 12] and res[0].finish_reason == "stop"            # 13 stops it and is not emitted
+    assert res[0].logprobs == [-1.2, -1.3] and res[1].logprobs == [] and res[1].tokens == [21, 22, 23]

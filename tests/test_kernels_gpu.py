@@ -430,6 +430,23 @@ def test_cpu_tensors_are_refused(K):
 
 
 # ---------------------------------------------------------------- matrix-core products
+@pytest.mark.parametrize("b,v", [(1, 7), (5, 1000), (8, 262208), (3, 4099)])
+def test_token_logprob(S, b, v):
+    """log softmax at one entry of each row, rows with -inf entries and a row strides apart among them."""
+    g = torch.Generator().manual_seed(b + v)
+    wide = (torch.randn(b, v + 5, generator=g) * 4).to(DEV)
+    logits = wide[:, :v]
+    logits[0, : v // 2] = float("-inf")
+    toks = torch.randint(v // 2, v, (b,), generator=g).to(torch.int32).to(DEV)
+    out = torch.full((b,), float("nan"), device=DEV)
+    S.token_logprob(logits, toks, out)
+    ref = torch.log_softmax(logits.double(), -1)[torch.arange(b), toks.long()]
+    assert torch.allclose(out.double(), ref, atol=2e-5, rtol=0)
+    if v > 2:                                               # an entry that is -inf has probability 0
+        S.token_logprob(logits, torch.zeros(b, dtype=torch.int32, device=DEV), out)
+        assert float(out[0]) == float("-inf")
+
+
 @pytest.fixture(scope="module")
 def G():
     from agave_amd.ops import gemm_mfma
