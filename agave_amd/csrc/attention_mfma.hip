@@ -329,7 +329,12 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     // the token's sequence and position are asked for first: the page ids wait for them
     const int b = a.seq_is_token ? t : a.tok_seq[t];
     const int p = a.tok_pos[t];
-    // FUSED: the first rows of the q/k work are requested before anything else (wave w takes query
+    // The first columns of the table row are asked for before the position is known, a column per
+    // lane, and before every other vector load: loads come back in the order they left, so behind
+    // the rows of q and k the page ids would wait for those, and the first keys for the page ids.
+    int trow = -1;
+    if (a.table_from_reach) trow = a.table[(size_t)b * a.width + (lane < a.width ? lane : 0)];
+    // FUSED: the first rows of the q/k work are requested next (wave w takes query
     // head w of the chunk; the wave after the last head takes the key and value rows, in case
     // this workgroup turns out to be the one that writes them)
     constexpr int NV = HDT / 4;               // groups of 64 elements in a head
@@ -356,16 +361,14 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
     // leave the last splits of a short sequence idle and the waves of a split unequal shares); a
     // workgroup's four waves take its units in turn.  A unit is one round trip to memory, and with
     // as many waves as units nearly every wave makes just one.
-    // The first columns of the table row are asked for before the position is known, a column per
-    // lane: which of them this wave needs depends on the position, but waiting for that first would
-    // put a second round trip before the first key.
-    int trow = -1;
-    if (a.table_from_reach) trow = a.table[(size_t)b * a.width + (lane < a.width ? lane : 0)];
+    // Which columns of the table row (asked for at the start) this wave needs depends on the
+    // position; asking only then would put a second round trip before the first key.
     const int lo = a.window > 0 ? (p - a.window + 1 > 0 ? p - a.window + 1 : 0) : 0;
     const int first = lo / AGAVE_PAGE, last = p / AGAVE_PAGE;
     const int u_first = lo / 32, u_last = p / 32, n_u = u_last - u_first + 1;
-    const int ua = u_first + (int)((long)split * n_u / a.splits);
-    const int ub = u_first + (int)((long)(split + 1) * n_u / a.splits);
+    // (32-bit: at most 64 splits times the half pages of a context; a 64-bit division is some hundred instructions)
+    const int ua = u_first + (int)((unsigned)(split * n_u) / (unsigned)a.splits);
+    const int ub = u_first + (int)((unsigned)((split + 1) * n_u) / (unsigned)a.splits);
     const int u0 = ua + wave;
     const int half = u0 & 1;                                       // (a wave's units are four apart: one half)
     const int n_my = u0 < ub ? (ub - u0 + 3) / 4 : 0;              // units this wave takes
@@ -405,7 +408,7 @@ __global__ __launch_bounds__(256) void attn_decode_fast_kernel(AttnArgs a, QkFus
         if (a.table_from_reach) {
             const int col = pi - first;
             if (!wide) {
-                pg = col < a.width ? __shfl(trow, col, 64) : -1;
+                pg = col < a.width ? __builtin_amdgcn_readlane(trow, col) : -1;
             } else if (i < PG_AHEAD) {
                 pg = -1;
 #pragma unroll
@@ -1096,6 +1099,7 @@ static int launch_decode(const AttnArgs& a, const QkFuse& f, int N, hipStream_t 
     AGAVE_CHECK(splits >= 1 && splits <= COMBINE_MAX_SPLITS && a.pages_per_split >= 1, "attn_decode_mfma: bad split plan %d x %d", splits, a.pages_per_split);
     AGAVE_CHECK(splits == 1 || (a.part_o && a.part_ml), "attn_decode_mfma: splits need the partial buffers");
     AGAVE_CHECK(N <= 65535, "attn_decode_mfma: %d tokens exceed the grid limit", N);
+    AGAVE_CHECK((2l * a.n_pages + 2) * (splits + 1) < (1l << 31), "attn_decode_mfma: %d pages in %d splits exceed 32-bit unit counts", a.n_pages, splits);
     if (N == 0) return 0;
     const int G = nh / nkv;
     dim3 grid(splits, nkv * ((G + 15) / 16), N);

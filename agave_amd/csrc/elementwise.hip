@@ -119,7 +119,7 @@ template <> __device__ __forceinline__ void store4<bf16>(bf16* p, float4 v) {
 // loaded is touched before everything has been asked for, so the loads travel together.
 __device__ __forceinline__ float sumsq(bool in, float4 v) { return in ? v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w : 0.f; }
 
-template <typename T, int VPT>
+template <typename T, int VPT, int PB>          // PB: slices asked for at a time
 __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
                                           long part_stride, const float* __restrict__ post_gain, float post_eps,
                                           T* __restrict__ out, long ldo, const float* __restrict__ pre_gain,
@@ -129,7 +129,6 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
     const int r = rows ? rows[i] : i;
     float* hr = h + (size_t)r * e;
     const float4 z = float4{0.f, 0.f, 0.f, 0.f};
-    constexpr int PB = 4;                       // slices asked for at a time
     float4 hv[VPT], bv[VPT], g1[VPT], g2[VPT], pv[PB][VPT];
     int col[VPT];
     bool in[VPT];
@@ -236,8 +235,14 @@ static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, in
         threads = 64 * ((e / 4 + per * 64 - 1) / (per * 64));
     }
     const int vpt = (e / 4 + threads - 1) / threads;
+    // more than four slices (the output product's runs of heads): eight at a time when a thread holds one float4 of each
 #define RN_FAST(V)                                                                                                    \
-    residual_norm_fast_kernel<T, V><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts, part_stride,  \
+    if (n_parts > 4 && V == 1)                                                                                        \
+        residual_norm_fast_kernel<T, V, 8><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts,        \
+                                                                           part_stride, post_gain, post_eps, (T*)out, \
+                                                                           ldo, pre_gain, pre_eps, rows, e);          \
+    else                                                                                                              \
+    residual_norm_fast_kernel<T, V, 4><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts, part_stride,  \
                                                                     post_gain, post_eps,                             \
                                                                     (T*)out, ldo, pre_gain, pre_eps, rows, e)
     if (vpt <= 1) RN_FAST(1);

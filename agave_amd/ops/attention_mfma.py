@@ -19,27 +19,36 @@ kernels.register_signatures("attention_mfma", {
                                  _I, _P, _P, _P, _I, _P],
 })
 
-TARGET_WORKGROUPS = 256      # workgroups (of 4 waves) a decode launch aims for: one per compute unit
+TARGET_WORKGROUPS = 256      # workgroups (of 4 waves) the general decode kernel aims for: one per compute unit
+FAST_TARGET = 192            # and the kernels that share half pages: see split_plan
 
 
 def split_plan(page_span: int, units: int, head_dim: int = 0):
     """(splits, pages per split) for sequences spanning at most ``page_span`` pages when the launch
     has ``units`` (token, kv head) pairs.  The kernels for head sizes 64, 128 and 256 share a
     sequence's half pages evenly among the splits, four waves a split and a half page a wave at a
-    time: as many splits as fill the compute units, but no more than leave a split six half pages
-    (at a batch of 8 and a reach of 17 pages, 6 splits of 5 or 6 half pages measured 3 % of the
-    kernel faster than 8 of 4 or 5: what more splits gain in balance they lose in partial results).
+    time.  Measured over whole decode steps of three model sizes at batches of 1, 8 and 32 with 17
+    pages in reach: up to 192 workgroups every further split pays, down to a page a split; a launch
+    of 256 workgroups is slower than one of 192 or of 128 (6 splits beat 8 at 32 units, 3 beat 4 at
+    64, 1 beats 2 at 128), and beyond that each further split costs its partial results and gains
+    nothing.  With 64 pages or more in reach the keys outweigh that: 2 splits beat 1 at 128 units
+    (by 1 % at 121 pages, by 4 % at 500), so there a launch that would leave half the compute units
+    idle is split further (6 splits still beat 8 at 32 units and 500 pages).
     The general kernel gives each split a run of whole pages."""
-    want = max(1, -(-TARGET_WORKGROUPS // max(units, 1)))
     if head_dim in FUSED_HEAD_DIMS:
-        splits = max(1, min(TARGET_WORKGROUPS // max(units, 1), -(-2 * page_span // 6), MAX_SPLITS))
+        splits = FAST_TARGET // max(units, 1)
+        if page_span >= 64 and splits * units <= TARGET_WORKGROUPS // 2:
+            splits = TARGET_WORKGROUPS // max(units, 1)
+        splits = max(1, min(splits, page_span, SPLITS_AT_ONCE if page_span < 64 else MAX_SPLITS))
         return splits, -(-page_span // splits)
-    want = min(want, page_span)
+    want = max(1, min(page_span, -(-TARGET_WORKGROUPS // max(units, 1))))
     per = -(-page_span // want)
     return -(-page_span // per), per
 
 
 MAX_SPLITS = 64              # what the merge inside the output product takes
+SPLITS_AT_ONCE = 12          # and what it merges with one round trip to memory (at a batch of 1, 12 splits
+                             # measured as fast as 16; with 500 pages in reach 32 beat 16 by 1 %)
 FUSED_HEAD_DIMS = (64, 128, 256)
 
 

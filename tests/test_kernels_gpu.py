@@ -536,7 +536,7 @@ def test_gemm_skinny_refuses_what_it_cannot_do(G):
 
 @pytest.mark.parametrize("m,nh,hd,splits,n", [(8, 8, 256, 6, 2560), (1, 8, 256, 64, 2560), (16, 32, 128, 4, 5376),
                                               (3, 6, 64, 2, 100), (5, 16, 256, 3, 3840), (2, 4, 96, 9, 250),
-                                              (13, 20, 128, 5, 72)])
+                                              (13, 20, 128, 5, 72), (16, 8, 256, 11, 512), (1, 16, 256, 17, 3840)])
 def test_product_of_the_decode_attention_s_partial_results(G, m, nh, hd, splits, n):
     """The output projection that merges the splits' partial results itself, against the merge
     written out (with its rows rounded to bfloat16, as the separate merge kernel leaves them) and an
