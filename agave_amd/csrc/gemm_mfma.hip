@@ -480,7 +480,8 @@ __global__ __launch_bounds__(512) void gemm_oproj_combine_kernel(const float* __
             const int ks = wave + 4 * (i < n_mine ? i : 0);
 #pragma unroll
             for (int rr = 0; rr < RB; ++rr) {
-                const int nb = nb0 + r0 + rr < NB ? nb0 + r0 + rr : NB - 1;
+                // (a row block past the workgroup's or the matrix's last: its first one again, from the cache)
+                const int nb = (r0 + rr < R && nb0 + r0 + rr < NB) ? nb0 + r0 + rr : nb0;
                 wr[rr][i].u = Wp[w_tile(nb, kb0 + ks, NB, KB) * 64 + lane];
             }
         }
