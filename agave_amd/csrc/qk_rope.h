@@ -54,10 +54,18 @@ __device__ __forceinline__ QkRow<T, NV> qk_row_load(const T* src, const float* _
     return r;
 }
 
+// Between a wave's writes to its own part of LDS and its reads of what other lanes wrote there.
+// The LDS serves a wave's accesses in order, so no instruction is needed; the compiler must keep
+// the order too.
+__device__ __forceinline__ void wave_lds_order() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // y[0..hd) (LDS, 32-bit) <- rotate(row * rsqrt(mean(row^2) + eps) * gain) for the row that qk_row_load
 // fetched.  has_gain false: no norm; rot_half 0: no rotation.  pf: position times the position
-// scale.  Every wave of the workgroup calls this together (it holds two workgroup barriers); a
-// wave without work passes active = false.
+// scale.  y is the calling wave's own; a wave without work passes active = false.
 template <typename T, int NV>
 __device__ __forceinline__ void qk_row_finish(const QkRow<T, NV>& r, float* y, bool has_gain, float eps, int rot_half,
                                               float pf, int hd, int lane, bool active) {
@@ -78,7 +86,7 @@ __device__ __forceinline__ void qk_row_finish(const QkRow<T, NV>& r, float* y, b
         const int d = lane + 64 * k;
         if (active && d < hd) y[d] = has_gain ? xv[k] * inv * r.gv[k] : xv[k];
     }
-    __syncthreads();
+    wave_lds_order();
     // rotation, in place in LDS: y[i], y[i + rot_half] <- rotated pair
 #pragma unroll
     for (int k = 0; k < (NV + 1) / 2; ++k) {
@@ -91,7 +99,7 @@ __device__ __forceinline__ void qk_row_finish(const QkRow<T, NV>& r, float* y, b
             y[i + rot_half] = a * s + b2 * c;
         }
     }
-    __syncthreads();
+    wave_lds_order();
 }
 
 // One wave writes a key row y[0..hd) (LDS) and a value row (in registers: vreg[k] is element
