@@ -20,26 +20,45 @@ kernels.register_signatures("attention_mfma", {
 })
 
 TARGET_WORKGROUPS = 256      # workgroups (of 4 waves) the general decode kernel aims for: one per compute unit
-FAST_TARGET = 192            # and the kernels that share half pages: see split_plan
+FAST_TARGET = 192            # the kernels that share half pages, 64 pages or more in reach: see split_plan
+FAST_CAP = 240               # and with fewer pages in reach
 
 
 def split_plan(page_span: int, units: int, head_dim: int = 0):
     """(splits, pages per split) for sequences spanning at most ``page_span`` pages when the launch
     has ``units`` (token, kv head) pairs.  The kernels for head sizes 64, 128 and 256 share a
     sequence's half pages evenly among the splits, four waves a split and a half page a wave at a
-    time.  Measured over whole decode steps of three model sizes at batches of 1, 8 and 32 with 17
-    pages in reach: up to 192 workgroups every further split pays, down to a page a split; a launch
-    of 256 workgroups is slower than one of 192 or of 128 (6 splits beat 8 at 32 units, 3 beat 4 at
-    64, 1 beats 2 at 128), and beyond that each further split costs its partial results and gains
-    nothing.  With 64 pages or more in reach the keys outweigh that: 2 splits beat 1 at 128 units
-    (by 1 % at 121 pages, by 4 % at 500), so there a launch that would leave half the compute units
-    idle is split further (6 splits still beat 8 at 32 units and 500 pages).
+    time, so a split of n half pages takes ceil(n / 4) rounds.  The rules are fitted to whole
+    decode steps of three model sizes at batches of 1 to 32.
+
+    Fewer than 64 pages in reach (measured with 17): no more than 240 workgroups (256 are slower
+    than 192 or 128; a second round of workgroups is far slower) and no more than 12 splits (what
+    the output product merges with one round trip to memory).  Within that, the fewest rounds;
+    among equals the fewest splits (each costs its partial results: 6 or 5 splits beat 7 and 8 at
+    32 units, 3 beat 4 at 56 and 64), except that once every wave has at most one half page more
+    splits still gain a little (12 beat 9 at a batch of 1 and of 4).
+
+    64 pages or more: the keys outweigh the rest; as many splits as make 192 workgroups (6 beat 8
+    at 32 units and 500 pages), but a launch that would leave half the compute units idle is split
+    further (2 splits beat 1 at 128 units: by 1 % at 121 pages, by 4 % at 500).
+
     The general kernel gives each split a run of whole pages."""
     if head_dim in FUSED_HEAD_DIMS:
-        splits = FAST_TARGET // max(units, 1)
-        if page_span >= 64 and splits * units <= TARGET_WORKGROUPS // 2:
-            splits = TARGET_WORKGROUPS // max(units, 1)
-        splits = max(1, min(splits, page_span, SPLITS_AT_ONCE if page_span < 64 else MAX_SPLITS))
+        u = max(units, 1)
+        if page_span >= 64:
+            splits = FAST_TARGET // u
+            if splits * u <= TARGET_WORKGROUPS // 2:
+                splits = TARGET_WORKGROUPS // u
+            splits = max(1, min(splits, page_span, MAX_SPLITS))
+        else:
+            half_pages = 2 * page_span
+            cap = max(1, min(FAST_CAP // u, page_span, SPLITS_AT_ONCE))
+
+            def rounds(s):
+                return -(-(-(-half_pages // s)) // 4)
+            splits = min(range(1, cap + 1), key=lambda s: (rounds(s), s))
+            if rounds(splits) == 1:
+                splits = cap
         return splits, -(-page_span // splits)
     want = max(1, min(page_span, -(-TARGET_WORKGROUPS // max(units, 1))))
     per = -(-page_span // want)
@@ -48,7 +67,7 @@ def split_plan(page_span: int, units: int, head_dim: int = 0):
 
 MAX_SPLITS = 64              # what the merge inside the output product takes
 SPLITS_AT_ONCE = 12          # and what it merges with one round trip to memory (at a batch of 1, 12 splits
-                             # measured as fast as 16; with 500 pages in reach 32 beat 16 by 1 %)
+                             # measured as fast as 16)
 FUSED_HEAD_DIMS = (64, 128, 256)
 
 
