@@ -1082,6 +1082,11 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
             const int n_main = EPI == 0 ? nb_main * 16 : nb_main * 8;
             int rc = launch_tiled<4, 1, 4, EPI, TC, 8, 256, true>(X, ldx, Wp, Y, ldy, M, n_main, K, KB, nb_main, stream, 1, 0, NB);
             if (rc != 0) return rc;
+            // (a quarter of a round or less: tiles of a quarter of the size, which again fill the compute units)
+            if (rest <= 64 && (rows16 - rows_main) * 2 * ((M + 127) / 128) <= 256)
+                return launch_tiled<2, 2, 3, EPI, TC, 8, 128, false>(X, ldx, (const uint4*)Wp + w_tile(nb_main, 0, NB, KB) * 64,
+                                                                     (TC*)Y + n_main, ldy, M, N - n_main, K, KB, NB - nb_main,
+                                                                     stream, 1, 0, NB);
             return launch_tiled<2, 2, 3, EPI, TC, 8, 256, false>(X, ldx, (const uint4*)Wp + w_tile(nb_main, 0, NB, KB) * 64,
                                                                  (TC*)Y + n_main, ldy, M, N - n_main, K, KB, NB - nb_main, stream,
                                                                  1, 0, NB);
@@ -1104,20 +1109,26 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
 // 10,240 columns (measured: down at 2,048 tokens takes 114 us in three slices instead of 136, and
 // the kernel that adds them 8 us more), in proportion to the tiles and inversely to the columns.
 // Products that run in 256 x 256 tiles are left alone: sliced, they were slower (measured at
-// 4,096 and 8,192 tokens, by 4 %).
+// 4,096 and 8,192 tokens, by 4 %).  Shorter prompts gain as much: down at 1,024 tokens takes 59 us
+// in three slices of 80 tiles instead of 81 us in 160 tiles of 128 x 128 (a prefill of 384 to
+// 1,024 tokens 2 to 5 % less).
 static int cut_tiled_slices(int M, int N, int K) {
     const long NB = (N + 15) / 16;
     const long rows16 = (NB + 15) / 16, rows8 = (NB + 7) / 8;
     const long t256 = (M + 255) / 256;
-    if (rows16 * t256 >= 160 || rows8 * t256 < 160) return 1;      // 256 x 256 tiles, or smaller ones than 128 x 256
+    if (rows16 * t256 >= 160 || rows8 * t256 < 20) return 1;      // 256 x 256 tiles, or next to no tiles at all
     const long t = rows8 * t256;
+    // fewer than 160 tiles of 128 x 256 (shorter prompts, which would run in smaller tiles on 160
+    // or 240 compute units): only with long runs of columns a slice (down, not o, whose 2,048
+    // columns in two slices were no faster)
+    const int min_stages = t >= 160 ? 16 : 32;
     auto rounds = [](long g) { return (double)((g + 255) / 256); };
     const double slice_cost = 0.07 * (10240.0 / K) * ((double)t / 160.0);
     const int n_stage = (K + 63) / 64;
     double best = rounds(t);
     int z_best = 1;
     for (int z = 2; z <= 4; ++z) {
-        if (n_stage / z < 16) break;
+        if (n_stage / z < min_stages) break;
         const double cost = rounds(t * z) / z + (z - 1) * slice_cost;
         if (cost < 0.93 * best) {
             best = cost;

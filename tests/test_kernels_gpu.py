@@ -774,7 +774,9 @@ def test_attn_mfma_far_key_and_window_edge(K, how, hd):
                                    # many stages (the loads run several stages ahead of the multiplications): each tile
                                    (300, 2000, 1000), (600, 5000, 1000), (1024, 5120, 1000), (1024, 10240, 1000),
                                    # 640 tiles: two rounds of 256 x 256 tiles and the last rows in tiles of half the height
-                                   (2048, 20470, 64)])
+                                   (2048, 20470, 64),
+                                   # 320 tiles: one round and the last rows in tiles of a quarter of the size
+                                   (1024, 20470, 64)])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_gemm_tiled(G, m, n, k, out_dtype):
     g = torch.Generator().manual_seed(m + n + k)
@@ -795,7 +797,10 @@ def test_gemm_tiled(G, m, n, k, out_dtype):
     (2000, 2552, 10248, 3),     # ragged edges
     (8192, 640, 10240, 3),      # 160 tiles of 128 x 256 whose slices in 256 x 256 would be 288: they stay 480 of 128 x 256
     (2048, 2560, 2048, 1),      # few columns: one product
-    (300, 200, 4096, 1)])       # small tiles: one product
+    (1024, 2560, 10240, 3),     # a shorter prompt: 80 tiles of 128 x 256 in three slices
+    (768, 2560, 10240, 4),      # 60 tiles in four
+    (1024, 2560, 2048, 1),      # 80 tiles, but too few columns for a slice
+    (300, 200, 4096, 1)])       # next to no tiles: one product
 def test_gemm_tiled_in_slices(G, m, n, k, slices):
     """A product of many tokens whose tiles fill the compute units badly comes as 32-bit slices
     that add up to it, for a reader that adds them."""
@@ -815,7 +820,8 @@ def test_gemm_tiled_in_slices(G, m, n, k, slices):
     assert float(out[0].abs().max()) > 0 and float(out[z - 1].abs().max()) > 0
 
 
-@pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40), (1024, 5120, 1000), (2048, 10236, 64)])
+@pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40), (1024, 5120, 1000), (2048, 10236, 64),
+                                    (1024, 10236, 64)])
 def test_gemm_tiled_geglu(G, m, ff, k):
     g = torch.Generator().manual_seed(ff + m)
     x = torch.randn(m, k, generator=g).bfloat16()
