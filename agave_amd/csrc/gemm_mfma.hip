@@ -1109,7 +1109,8 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
 // 10,240 columns (measured: down at 2,048 tokens takes 114 us in three slices instead of 136, and
 // the kernel that adds them 8 us more), in proportion to the tiles and inversely to the columns.
 // Products that run in 256 x 256 tiles are left alone: sliced, they were slower (measured at
-// 4,096 and 8,192 tokens, by 4 %).  Shorter prompts gain as much: down at 1,024 tokens takes 59 us
+// 4,096 and 8,192 tokens, by 4 %; slices of 256 x 256 tiles by 1 to 2 %, except for 168 tiles, a
+// round two thirds full, where they gained 2 %).  Shorter prompts gain as much: down at 1,024 tokens takes 59 us
 // in three slices of 80 tiles instead of 81 us in 160 tiles of 128 x 128 (a prefill of 384 to
 // 1,024 tokens 2 to 5 % less).
 static int cut_tiled_slices(int M, int N, int K) {
