@@ -1071,12 +1071,15 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
         // 256 compute units take 256 tiles at a time.  When the last round would be at most half
         // full, the rows of that round are computed in tiles of half the height instead, in a
         // second launch: all compute units then work for half a round, not half of them for a whole one.
-        const long tiles = wgs[0], rest = tiles % 256;
+        const long tiles = wgs[0];
         long rows_main = 0;                                // 256-row tiles of the first launch
-        if (tiles > 256 && rest > 0 && rest <= 128) {
-            rows_main = (tiles - rest) / t256;             // whole rounds, if they are whole rows of tiles
-            if (rows_main * t256 != tiles - rest || (rows16 - rows_main) * 2 * t256 > 256) rows_main = 0;
+        if (tiles > 256 && tiles % 256 > 0) {
+            // as many whole rows of tiles as fit the whole rounds; the others, if their tiles of half
+            // the height fit one round
+            rows_main = (tiles / 256) * 256 / t256;
+            if (rows_main <= 0 || (rows16 - rows_main) * 2 * t256 > 256) rows_main = 0;
         }
+        const long rest = tiles - rows_main * t256;        // 256 x 256 tiles' worth of the second launch
         if (rows_main > 0) {
             const int nb_main = (int)rows_main * 16;
             const int n_main = EPI == 0 ? nb_main * 16 : nb_main * 8;
