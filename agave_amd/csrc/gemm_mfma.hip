@@ -1045,6 +1045,9 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
         for (int i = 1; i < 4; ++i)
             if (wgs[i] > wgs[pick]) pick = i;
     }
+    // up to 128 tokens would leave half of a 256-token tile empty: tiles of 128 tokens (a step of 65
+    // to 128 tokens 3 to 5 % faster)
+    if (pick <= 1 && M <= 128) pick = 2;
     // Still few workgroups and many columns: several workgroups share a tile's columns and leave
     // partial sums (32-bit, in a buffer the caller lends), which a second kernel adds up.
     int splits = 1;
