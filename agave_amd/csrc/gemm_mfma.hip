@@ -344,7 +344,7 @@ static SkinnyCut cut_skinny(int M, int NB, int KB, int max_z, int only_z = 0) {
             }
         return cut;
     }
-    static const int cand2[] = {1, 2, 4, 5, 0}, cand3[] = {1, 4, 5, 0};
+    static const int cand2[] = {1, 2, 4, 5, 0}, cand3[] = {1, 2, 4, 5, 0};
     const int* cand = mt <= 2 ? cand2 : cand3;
     const int n_chunks = (KB + (mt <= 2 ? 4 : 2) - 1) / (mt <= 2 ? 4 : 2);
     double best = 1e30;
@@ -385,9 +385,11 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
         case 2 * 8 + 4: SK_CASE(4, 2);
         case 2 * 8 + 5: SK_CASE(5, 2);
         case 3 * 8 + 1: SK_CASE(1, 3);
+        case 3 * 8 + 2: SK_CASE(2, 3);
         case 3 * 8 + 4: SK_CASE(4, 3);
         case 3 * 8 + 5: SK_CASE(5, 3);
         case 4 * 8 + 1: SK_CASE(1, 4);
+        case 4 * 8 + 2: SK_CASE(2, 4);
         case 4 * 8 + 4: SK_CASE(4, 4);
         case 4 * 8 + 5: SK_CASE(5, 4);
         default: AGAVE_CHECK(false, "gemm_skinny: no kernel for %d tokens with %d row blocks a workgroup", M, r);
