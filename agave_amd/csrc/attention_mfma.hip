@@ -960,11 +960,23 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
                 lds_settle();
 #pragma unroll
                 for (int i = 0; i < 2 * KS; ++i) lds_use(fr[i]);
-                f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0;
+                // Head sizes up to 128: four chains of multiplications instead of two (measured at 128:
+                // 55 us instead of 70 for 2,048 tokens and 32 heads; at 256, with chains of 8 and 4, no gain).
+                constexpr bool FOUR_CHAINS = KS > 1 && KS <= 4;
+                f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0, st0b = st0, st1b = st0;
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
-                    st0 = mfma_16x16x32(fr[2 * ks], qf[ks], st0);
-                    st1 = mfma_16x16x32(fr[2 * ks + 1], qf[ks], st1);
+                    if (FOUR_CHAINS && (ks & 1)) {
+                        st0b = mfma_16x16x32(fr[2 * ks], qf[ks], st0b);
+                        st1b = mfma_16x16x32(fr[2 * ks + 1], qf[ks], st1b);
+                    } else {
+                        st0 = mfma_16x16x32(fr[2 * ks], qf[ks], st0);
+                        st1 = mfma_16x16x32(fr[2 * ks + 1], qf[ks], st1);
+                    }
+                }
+                if (FOUR_CHAINS) {
+                    st0 += st0b;
+                    st1 += st1b;
                 }
                 __builtin_amdgcn_sched_barrier(0);
                 static_for<0, HDT>([&](auto d) { lds_read16<(n_k + d.value * 2 + half) * 1024>(fr[d.value], kaddr); });
