@@ -392,6 +392,26 @@ def test_layers_of_the_published_sizes(tmp_path, dtype, size):
         close(dtype)(o, U.plain_logits(cfg, weights, r), f"{size} layers, request {i + 1} of a batch", **kw)
 
 
+@pytest.mark.parametrize("n_seqs", [12, 70])
+def test_wide_batches_at_a_published_size(tmp_path, n_seqs):
+    """Decode steps of 12 and of 70 sequences with the 4B model's layer sizes: the products of 9 to
+    16 tokens are cut into workgroups like the larger batches', those of 65 and more run in tiles,
+    and the attention's splits follow the number of sequences.  Requests of unequal lengths, so the
+    batch shrinks as it goes."""
+    from agave_amd.engine import Engine
+    sizes, _, _ = BIG_LAYERS["4b"]
+    cfg = dict(P.tiny_config("A"), vocab_size=1536, num_hidden_layers=2, sliding_window_pattern=2, rope_theta=1e6,
+               rope_local_base_freq=1e4, rms_norm_eps=1e-6, max_position_embeddings=4096, **dict(sizes, sliding_window=24))
+    cfg.pop("layer_types", None)
+    weights = P.random_weights(cfg, 21)
+    folder = U.write_model(str(tmp_path / "m"), cfg, weights)
+    eng = Engine.from_folder(folder, dtype="bfloat16", max_slots=n_seqs, max_context=128)
+    reqs = [U.random_tokens(30 + i % 7, cfg["vocab_size"], 40 + i) for i in range(n_seqs)]
+    outs = U.run_batched(eng, reqs, [14 + i % 5 for i in range(n_seqs)])
+    for i in (0, 1, n_seqs // 2, n_seqs - 2, n_seqs - 1):
+        close("bfloat16")(outs[i], U.plain_logits(cfg, weights, reqs[i]), f"request {i} of {n_seqs}")
+
+
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
 def test_sizes_that_fit_no_fast_kernel(tmp_path, dtype):
     """Width 100 and inner size 52 (no multiples of 8), heads of 20 (no multiple of 16), an odd
