@@ -946,88 +946,230 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
             // this lane's 16 bytes of the page's first tile; tiles follow each other by 1 KB
             const unsigned kaddr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) uint4*)page_lds +
                                    (unsigned)(buf * buf_tiles * 64 + lane) * 16u;
-            static_for<0, 2>([&](auto halfc) {
-                constexpr int half = decltype(halfc)::value;
-                const int key0 = pi * AGAVE_PAGE + 32 * half;
-                if (key0 > p_max || key0 + 31 < lo_min) return;                // no column sees this unit
-                // all of the unit's key tiles are asked for at once, then multiplied; the value tiles
-                // are asked for before the exponentials and arrive while those are computed
-                frag16 fr[2 * KS > HDT ? 2 * KS : HDT];
-                static_for<0, KS>([&](auto ks) {
-                    lds_read16<((2 * half) * KS + ks.value) * 1024>(fr[2 * ks.value], kaddr);
-                    lds_read16<((2 * half + 1) * KS + ks.value) * 1024>(fr[2 * ks.value + 1], kaddr);
-                });
-                lds_settle();
-#pragma unroll
-                for (int i = 0; i < 2 * KS; ++i) lds_use(fr[i]);
-                // Head sizes up to 128: four chains of multiplications instead of two (measured at 128:
-                // 55 us instead of 70 for 2,048 tokens and 32 heads; at 256, with chains of 8 and 4, no gain).
-                constexpr bool FOUR_CHAINS = KS > 1 && KS <= 4;
-                f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0, st0b = st0, st1b = st0;
-#pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
-                    if (FOUR_CHAINS && (ks & 1)) {
-                        st0b = mfma_16x16x32(fr[2 * ks], qf[ks], st0b);
-                        st1b = mfma_16x16x32(fr[2 * ks + 1], qf[ks], st1b);
-                    } else {
-                        st0 = mfma_16x16x32(fr[2 * ks], qf[ks], st0);
-                        st1 = mfma_16x16x32(fr[2 * ks + 1], qf[ks], st1);
+            if constexpr (HDT == 16) {
+                // Which of the page's two units (half pages) some column of the tile sees.
+                const bool see0 = !(pi * AGAVE_PAGE > p_max || pi * AGAVE_PAGE + 31 < lo_min);
+                const bool see1 = !(pi * AGAVE_PAGE + 32 > p_max || pi * AGAVE_PAGE + 63 < lo_min);
+                // A unit's key tiles and its value tiles come from LDS in two batches each, into two sets
+                // of registers that take turns: while the multiplications of one batch run, the next
+                // batch is on its way, so that the LDS and the matrix cores work at the same time
+                // (read whole and then multiplied, the eight waves all read, then all multiply).  The
+                // keys of the page's second unit are asked for during the first unit's last
+                // multiplications.  The LDS returns a wave's reads in order: a wait for "at most n
+                // outstanding" leaves the younger batch in flight.
+                constexpr int KH = KS / 2;                            // k-steps per batch of key tiles
+                frag16 fa[KS], fb[KS];
+                auto read_keys_a = [&](auto halfc) {
+                    constexpr int half = decltype(halfc)::value;
+                    static_for<0, KH>([&](auto ks) {
+                        lds_read16<((2 * half) * KS + ks.value) * 1024>(fa[2 * ks.value], kaddr);
+                        lds_read16<((2 * half + 1) * KS + ks.value) * 1024>(fa[2 * ks.value + 1], kaddr);
+                    });
+                };
+                auto read_keys_b = [&](auto halfc) {
+                    constexpr int half = decltype(halfc)::value;
+                    static_for<0, KH>([&](auto ks) {
+                        lds_read16<((2 * half) * KS + KH + ks.value) * 1024>(fb[2 * ks.value], kaddr);
+                        lds_read16<((2 * half + 1) * KS + KH + ks.value) * 1024>(fb[2 * ks.value + 1], kaddr);
+                    });
+                };
+                auto unit = [&](auto halfc, bool keys_asked, bool ask_next) {
+                    constexpr int half = decltype(halfc)::value;
+                    const int key0 = pi * AGAVE_PAGE + 32 * half;
+                    if (!keys_asked) {
+                        read_keys_a(halfc);
+                        read_keys_b(halfc);
                     }
-                }
-                if (FOUR_CHAINS) {
-                    st0 += st0b;
-                    st1 += st1b;
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                static_for<0, HDT>([&](auto d) { lds_read16<(n_k + d.value * 2 + half) * 1024>(fr[d.value], kaddr); });
-                __builtin_amdgcn_sched_barrier(0);
-                float s[8];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    s[e] = st0[e] * scale2;
-                    s[4 + e] = st1[e] * scale2;
-                }
-                if (key0 + 31 > p_min || key0 < lo_max) {                      // the diagonal or the window's edge
-#pragma unroll
+                    lds_settle_to<KS>();                              // the first batch of keys is here
+    #pragma unroll
+                    for (int i = 0; i < KS; ++i) lds_use(fa[i]);
+                    // Head sizes up to 128: four chains of multiplications instead of two (measured at 128:
+                    // 55 us instead of 70 for 2,048 tokens and 32 heads; at 256, with chains of 8 and 4, no gain).
+                    constexpr bool FOUR_CHAINS = KS > 1 && KS <= 4;
+                    f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0, st0b = st0, st1b = st0;
+    #pragma unroll
+                    for (int ks = 0; ks < KH; ++ks) {
+                        if (FOUR_CHAINS && (ks & 1)) {
+                            st0b = mfma_16x16x32(fa[2 * ks], qf[ks], st0b);
+                            st1b = mfma_16x16x32(fa[2 * ks + 1], qf[ks], st1b);
+                        } else {
+                            st0 = mfma_16x16x32(fa[2 * ks], qf[ks], st0);
+                            st1 = mfma_16x16x32(fa[2 * ks + 1], qf[ks], st1);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    lds_settle_to<0>();                               // the second batch
+    #pragma unroll
+                    for (int i = 0; i < KS; ++i) lds_use(fb[i]);
+                    static_for<0, KS>([&](auto d) { lds_read16<(n_k + d.value * 2 + half) * 1024>(fa[d.value], kaddr); });
+                    __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                    for (int ks = 0; ks < KH; ++ks) {
+                        if (FOUR_CHAINS && ((KH + ks) & 1)) {
+                            st0b = mfma_16x16x32(fb[2 * ks], qf[KH + ks], st0b);
+                            st1b = mfma_16x16x32(fb[2 * ks + 1], qf[KH + ks], st1b);
+                        } else {
+                            st0 = mfma_16x16x32(fb[2 * ks], qf[KH + ks], st0);
+                            st1 = mfma_16x16x32(fb[2 * ks + 1], qf[KH + ks], st1);
+                        }
+                    }
+                    if (FOUR_CHAINS) {
+                        st0 += st0b;
+                        st1 += st1b;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    static_for<0, KS>([&](auto d) { lds_read16<(n_k + (KS + d.value) * 2 + half) * 1024>(fb[d.value], kaddr); });
+                    __builtin_amdgcn_sched_barrier(0);
+                    float s[8];
+    #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const int k0 = key0 + 4 * g + e, k1 = k0 + 16;
-                        if (k0 > p || k0 < lo) s[e] = -INFINITY;
-                        if (k1 > p || k1 < lo) s[4 + e] = -INFINITY;
+                        s[e] = st0[e] * scale2;
+                        s[4 + e] = st1[e] * scale2;
                     }
-                }
-                float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                if (__any(mx > m_ref + LAZY_LOG2)) {
-                    const float m_new = fmaxf(m_ref, mx);
-                    const float f = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
-                    l *= f;
-                    float f4[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) f4[e] = __shfl(f, 4 * g + e, 64);
-#pragma unroll
-                    for (int d = 0; d < HDT; ++d)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) o[d][e] *= f4[e];
-                    m_ref = m_new;
-                }
-                const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
-                frag16 pf;
-                float sum = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const float pe = __builtin_amdgcn_exp2f(s[e] - m_use);
-                    sum += pe;
-                    pf.v[e] = (__bf16)pe;
-                }
-                l += sum;
-                lds_settle();
-#pragma unroll
-                for (int d = 0; d < HDT; ++d) {
-                    lds_use(fr[d]);
-                    o[d] = mfma_16x16x32(pf, fr[d], o[d]);
-                }
-            });
+                    if (key0 + 31 > p_min || key0 < lo_max) {                      // the diagonal or the window's edge
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int k0 = key0 + 4 * g + e, k1 = k0 + 16;
+                            if (k0 > p || k0 < lo) s[e] = -INFINITY;
+                            if (k1 > p || k1 < lo) s[4 + e] = -INFINITY;
+                        }
+                    }
+                    float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+                    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                    if (__any(mx > m_ref + LAZY_LOG2)) {
+                        const float m_new = fmaxf(m_ref, mx);
+                        const float f = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+                        l *= f;
+                        float f4[4];
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e) f4[e] = __shfl(f, 4 * g + e, 64);
+    #pragma unroll
+                        for (int d = 0; d < HDT; ++d)
+    #pragma unroll
+                            for (int e = 0; e < 4; ++e) o[d][e] *= f4[e];
+                        m_ref = m_new;
+                    }
+                    const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
+                    frag16 pf;
+                    float sum = 0.f;
+    #pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float pe = __builtin_amdgcn_exp2f(s[e] - m_use);
+                        sum += pe;
+                        pf.v[e] = (__bf16)pe;
+                    }
+                    l += sum;
+                    lds_settle_to<KS>();                              // the first batch of values
+    #pragma unroll
+                    for (int d = 0; d < KS; ++d) {
+                        lds_use(fa[d]);
+                        o[d] = mfma_16x16x32(pf, fa[d], o[d]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (ask_next) {
+                        if constexpr (half == 0) read_keys_a(std::integral_constant<int, 1>{});
+                        lds_settle_to<KS>();                          // the second batch of values (the next keys stay in flight)
+                    } else {
+                        lds_settle_to<0>();
+                    }
+    #pragma unroll
+                    for (int d = 0; d < KS; ++d) {
+                        lds_use(fb[d]);
+                        o[KS + d] = mfma_16x16x32(pf, fb[d], o[KS + d]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (ask_next) {
+                        if constexpr (half == 0) read_keys_b(std::integral_constant<int, 1>{});
+                    }
+                };
+                if (see0) unit(std::integral_constant<int, 0>{}, false, see1);
+                if (see1) unit(std::integral_constant<int, 1>{}, see0, false);
+            } else {
+                // (smaller heads: a unit is too short for batches; measured at 128, two batches were a fifth slower)
+                static_for<0, 2>([&](auto halfc) {
+                    constexpr int half = decltype(halfc)::value;
+                    const int key0 = pi * AGAVE_PAGE + 32 * half;
+                    if (key0 > p_max || key0 + 31 < lo_min) return;                // no column sees this unit
+                    // all of the unit's key tiles are asked for at once, then multiplied; the value tiles
+                    // are asked for before the exponentials and arrive while those are computed
+                    frag16 fr[2 * KS > HDT ? 2 * KS : HDT];
+                    static_for<0, KS>([&](auto ks) {
+                        lds_read16<((2 * half) * KS + ks.value) * 1024>(fr[2 * ks.value], kaddr);
+                        lds_read16<((2 * half + 1) * KS + ks.value) * 1024>(fr[2 * ks.value + 1], kaddr);
+                    });
+                    lds_settle();
+    #pragma unroll
+                    for (int i = 0; i < 2 * KS; ++i) lds_use(fr[i]);
+                    // Head sizes up to 128: four chains of multiplications instead of two (measured at 128:
+                    // 55 us instead of 70 for 2,048 tokens and 32 heads; at 256, with chains of 8 and 4, no gain).
+                    constexpr bool FOUR_CHAINS = KS > 1 && KS <= 4;
+                    f32x4_t st0 = f32x4_t{0.f, 0.f, 0.f, 0.f}, st1 = st0, st0b = st0, st1b = st0;
+    #pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+                        if (FOUR_CHAINS && (ks & 1)) {
+                            st0b = mfma_16x16x32(fr[2 * ks], qf[ks], st0b);
+                            st1b = mfma_16x16x32(fr[2 * ks + 1], qf[ks], st1b);
+                        } else {
+                            st0 = mfma_16x16x32(fr[2 * ks], qf[ks], st0);
+                            st1 = mfma_16x16x32(fr[2 * ks + 1], qf[ks], st1);
+                        }
+                    }
+                    if (FOUR_CHAINS) {
+                        st0 += st0b;
+                        st1 += st1b;
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    static_for<0, HDT>([&](auto d) { lds_read16<(n_k + d.value * 2 + half) * 1024>(fr[d.value], kaddr); });
+                    __builtin_amdgcn_sched_barrier(0);
+                    float s[8];
+    #pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        s[e] = st0[e] * scale2;
+                        s[4 + e] = st1[e] * scale2;
+                    }
+                    if (key0 + 31 > p_min || key0 < lo_max) {                      // the diagonal or the window's edge
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const int k0 = key0 + 4 * g + e, k1 = k0 + 16;
+                            if (k0 > p || k0 < lo) s[e] = -INFINITY;
+                            if (k1 > p || k1 < lo) s[4 + e] = -INFINITY;
+                        }
+                    }
+                    float mx = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])), fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+                    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                    if (__any(mx > m_ref + LAZY_LOG2)) {
+                        const float m_new = fmaxf(m_ref, mx);
+                        const float f = (m_ref == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+                        l *= f;
+                        float f4[4];
+    #pragma unroll
+                        for (int e = 0; e < 4; ++e) f4[e] = __shfl(f, 4 * g + e, 64);
+    #pragma unroll
+                        for (int d = 0; d < HDT; ++d)
+    #pragma unroll
+                            for (int e = 0; e < 4; ++e) o[d][e] *= f4[e];
+                        m_ref = m_new;
+                    }
+                    const float m_use = (m_ref == -INFINITY) ? 0.f : m_ref;
+                    frag16 pf;
+                    float sum = 0.f;
+    #pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float pe = __builtin_amdgcn_exp2f(s[e] - m_use);
+                        sum += pe;
+                        pf.v[e] = (__bf16)pe;
+                    }
+                    l += sum;
+                    lds_settle();
+    #pragma unroll
+                    for (int d = 0; d < HDT; ++d) {
+                        lds_use(fr[d]);
+                        o[d] = mfma_16x16x32(pf, fr[d], o[d]);
+                    }
+                });
+            }
         }
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();

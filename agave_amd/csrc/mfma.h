@@ -63,4 +63,10 @@ template <int OFFSET> __device__ __forceinline__ void lds_read16(frag16& dst, un
     asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst.r) : "v"(addr), "n"(OFFSET));
 }
 __device__ __forceinline__ void lds_settle() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// Until at most N of the wave's LDS reads are outstanding (they come back in the order they were
+// asked for, so the N youngest stay in flight; N up to 15).
+template <int N> __device__ __forceinline__ void lds_settle_to() {
+    static_assert(N >= 0 && N <= 15, "the counter holds four bits");
+    asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N) : "memory");
+}
 __device__ __forceinline__ void lds_use(frag16& v) { asm volatile("" : "+v"(v.r)); }
