@@ -19,6 +19,10 @@ kernels.register_signatures("attention_mfma", {
                                  _I, _P, _P, _P, _I, _P],
 })
 
+FUSED_HEAD_DIMS = (64, 128, 256)
+MAX_SPLITS = 64              # what the merge inside the output product takes
+SPLITS_AT_ONCE = 12          # and what it merges with one round trip to memory (at a batch of 1, 12 splits
+                             # measured as fast as 16)
 TARGET_WORKGROUPS = 256      # workgroups (of 4 waves) the general decode kernel aims for: one per compute unit
 FAST_TARGET = 192            # the kernels that share half pages, 64 pages or more in reach: see split_plan
 FAST_CAP = 240               # and with fewer pages in reach
@@ -63,12 +67,6 @@ def split_plan(page_span: int, units: int, head_dim: int = 0):
     want = max(1, min(page_span, -(-TARGET_WORKGROUPS // max(units, 1))))
     per = -(-page_span // want)
     return -(-page_span // per), per
-
-
-MAX_SPLITS = 64              # what the merge inside the output product takes
-SPLITS_AT_ONCE = 12          # and what it merges with one round trip to memory (at a batch of 1, 12 splits
-                             # measured as fast as 16)
-FUSED_HEAD_DIMS = (64, 128, 256)
 
 
 ITEM_PLACES = 192            # items are sized as if three quarters of the compute units' places were there: measured,

@@ -266,3 +266,19 @@ def test_the_items_of_a_prefill_step_cover_every_block_and_page_once(pos0, n_new
                 assert x[1] + x[2] == y[1]                        # runs that follow each other
             assert (tok_pieces[starts[b] + blk0:starts[b] + min(n, blk0 + blk_len)] == got[0][3]).all()
     assert not seen and len(tok_pieces) == sum(n_new)
+
+
+def test_the_decode_attention_s_split_plan():
+    """The number of splits stays within what the kernels and the merge take, whatever the sizes,
+    and follows the measured rules at the sizes they were measured at."""
+    from agave_amd.ops.attention_mfma import split_plan, MAX_SPLITS
+    for hd in (0, 64, 128, 256):
+        for span in (1, 2, 5, 17, 40, 63, 64, 121, 512, 2048):
+            for units in (1, 4, 8, 32, 33, 64, 100, 128, 256, 1000):
+                splits, per = split_plan(span, units, hd)
+                limit = MAX_SPLITS if hd else 256        # (the general kernel's merge takes 256 shares)
+                assert 1 <= splits <= min(span, limit) and per * splits >= span, (hd, span, units)
+    # 17 pages in reach, head size 256: a batch of 1, 8, 16, 17, 24 and 32 sequences of the 4B sizes (4 kv heads)
+    assert [split_plan(17, b * 4, 256)[0] for b in (1, 8, 16, 17, 24, 32)] == [12, 5, 3, 3, 2, 1]
+    # 500 pages: six splits at 32 units, and a launch that would leave half the chip idle is split further
+    assert split_plan(500, 32, 256)[0] == 6 and split_plan(500, 128, 256)[0] == 2
