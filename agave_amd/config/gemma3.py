@@ -260,4 +260,7 @@ class Gemma3Config:
             layers=layers, order=[RunEntry(i, i, True) for i in range(len(layers))],
             final_norm=norm(p + "norm.weight", e), head_weight=head,
             max_context=self.max_position_embeddings, bos_token_id=self.bos_token_id,
-            eos_token_ids=self.eos_token_ids)
+            eos_token_ids=self.eos_token_ids,
+            # what the reference's lookup can reach: names under the chosen prefix and the
+            # top-level output matrix (safetensors.zig:333-349, 535-540)
+            tensor_scope=(p, "lm_head."))

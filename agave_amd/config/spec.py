@@ -112,6 +112,10 @@ class ModelSpec:
     max_context: int
     bos_token_id: Optional[int] = None
     eos_token_ids: Tuple[int, ...] = ()
+    # Name prefixes of the tensors that are this model's own.  A checkpoint's tensor that no
+    # part asked for is an error under one of them and is passed over elsewhere (a vision
+    # tower beside a text decoder).  None: every name in the checkpoint is the model's.
+    tensor_scope: Optional[Tuple[str, ...]] = None
     extra: Dict[str, object] = field(default_factory=dict)
 
     def default_order(self) -> List[RunEntry]:

@@ -870,7 +870,7 @@ __global__ __launch_bounds__(256) void attn_merge_pieces_kernel(const float* __r
 // from L2 that bounds this kernel, and two waves share a SIMD).
 template <int HDT, int NWV>
 __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a, const PrefillItem* __restrict__ items, int nkc,
-                                                                   int hw, int max_pieces) {
+                                                                   int hw, int max_pieces, int max_item_pages) {
     constexpr int KS = HDT / 2, hd = HDT * 16;
     constexpr int n_k = 4 * KS, n_v = HDT * 2, buf_tiles = n_k + n_v;         // tiles (of 64 uint4) per page
     extern __shared__ __attribute__((aligned(16))) uint4 page_lds[];          // [2][K tiles | V tiles][64]
@@ -915,10 +915,10 @@ __global__ __launch_bounds__(NWV * 64) void attn_prefill_fast_kernel(AttnArgs a,
     // The ids of the pages this workgroup goes through, looked up once: a lookup inside the loop
     // is two dependent loads from memory a page, and waiting for them also waits for the next
     // page's loads, which were issued just before and should travel while this page is worked on.
-    // (the array holds a.width ids, a whole table row; the host refuses a step whose reach is wider than
-    // the table, and the bound below keeps the writes inside the array whatever the table says)
+    // (the array holds max_item_pages ids, the most pages that the host says any item has; the bound
+    // below keeps the writes inside the array whatever the items in device memory say)
     int* pg_ids = reinterpret_cast<int*>(page_lds + (size_t)2 * buf_tiles * 64);
-    if (page_last - page_first >= a.width) page_last = page_first + a.width - 1;
+    if (page_last - page_first >= max_item_pages) page_last = page_first + max_item_pages - 1;
     for (int i = threadIdx.x; i <= page_last - page_first; i += NWV * 64) pg_ids[i] = (int)page_of(a, b, page_first + i);
     __syncthreads();
 
@@ -1460,7 +1460,7 @@ extern "C" int agave_attn_prefill_items(const void* q, long ldq, void* out, long
     const unsigned grid = (unsigned)((long)n_items * nkc);
     const PrefillItem* its = reinterpret_cast<const PrefillItem*>(items);
 #define PF_LAUNCH(HDT_, NWV_) \
-    attn_prefill_fast_kernel<HDT_, NWV_><<<grid, NWV_ * 64, lds, stream>>>(a, its, nkc, hw, max_pieces)
+    attn_prefill_fast_kernel<HDT_, NWV_><<<grid, NWV_ * 64, lds, stream>>>(a, its, nkc, hw, max_pieces, max_item_pages)
     if (waves == 8) {
         if (hd == 64) PF_LAUNCH(4, 8);
         else if (hd == 128) PF_LAUNCH(8, 8);

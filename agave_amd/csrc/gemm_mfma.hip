@@ -483,7 +483,9 @@ __global__ __launch_bounds__(512) void gemm_oproj_combine_kernel(const float* __
     auto load_w = [&](frag16 (&wr)[RB][NKS], int r0) {
 #pragma unroll
         for (int i = 0; i < NKS; ++i) {           // (a k-step's row blocks lie side by side: asked for one after another)
-            const int ks = wave + 4 * (i < n_mine ? i : 0);
+            // (a k-step this wave does not have: its first one again; a wave without any, which a
+            // run of fewer than four k-steps leaves, the run's first, which always exists)
+            const int ks = i < n_mine ? wave + 4 * i : (n_mine > 0 ? wave : 0);
 #pragma unroll
             for (int rr = 0; rr < RB; ++rr) {
                 // (a row block past the workgroup's or the matrix's last: its first one again, from the cache)
@@ -602,7 +604,7 @@ __global__ __launch_bounds__(512) void gemm_oproj_combine_kernel(const float* __
     if (!merger) {
 #pragma unroll
         for (int i = 0; i < NKS; ++i) {
-            const int ks = wave + 4 * (i < n_mine ? i : 0);
+            const int ks = i < n_mine ? wave + 4 * i : (n_mine > 0 ? wave : 0);     // (as in load_w: never past the run)
             xb[i].u = *reinterpret_cast<const uint4*>(xs + (size_t)j * row + ks * 32 + g * 8);
         }
     }

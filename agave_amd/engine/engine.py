@@ -125,7 +125,7 @@ class Engine:
         cfg = arch.parse(raw)
         ckpt = Checkpoint(model_dir)
         spec = arch.spec(cfg, ckpt.names())
-        weights = WeightSource(ckpt, tensor_needs(spec))
+        weights = WeightSource(ckpt, tensor_needs(spec), spec.tensor_scope)
         return cls(spec, weights, config=cfg, **kw)
 
     @classmethod
@@ -133,7 +133,7 @@ class Engine:
         arch = find_architecture(raw_config)
         cfg = arch.parse(raw_config)
         spec = arch.spec(cfg, tensors.keys())
-        return cls(spec, DictWeightSource(tensors, tensor_needs(spec)), config=cfg, **kw)
+        return cls(spec, DictWeightSource(tensors, tensor_needs(spec), scope=spec.tensor_scope), config=cfg, **kw)
 
     @classmethod
     def from_random(cls, raw_config: dict, seed: int = 0, **kw) -> "Engine":

@@ -101,8 +101,6 @@ def generate(backend, prompts: Sequence[Sequence[int]],
 
     ahead = hasattr(backend, "launch_step") and all(p.repeat_penalty == 1.0 for p in plist)
     cancel_requested = getattr(backend, "cancel_requested", lambda: False)
-    if hasattr(backend, "clear_cancel"):
-        backend.clear_cancel()              # a request to cancel belongs to the call it arrived in
 
     def settle(i: int, tok: int, logprob: Optional[float] = None) -> None:
         """Book the token request i drew; sets its finish reason if it ends here."""
@@ -194,4 +192,9 @@ def generate(backend, prompts: Sequence[Sequence[int]],
         for r in results:
             if not r.finish_reason:
                 r.finish_reason = "cancelled"
+        # The call that a request to cancel ends also uses it up (the reference's owner resets the
+        # flag between requests, src/models/model.zig:315-317).  It is not cleared on entry: a
+        # request that arrives just before the call starts ends that call before its first step.
+        if hasattr(backend, "clear_cancel"):
+            backend.clear_cancel()
     return results

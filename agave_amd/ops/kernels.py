@@ -58,7 +58,14 @@ def lib(name: str):
     return handle
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream() -> int:
+    """The current HIP stream's handle.  Every launch asks for it, so it is read through torch's own
+    raw accessor where there is one (a fraction of a microsecond; the stream object costs several)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 

@@ -61,11 +61,17 @@ class Workspace:
 
     def __init__(self, device: torch.device):
         self.device = device
-        self._buffers: Dict[str, torch.Tensor] = {}
+        self._buffers: Dict[tuple, torch.Tensor] = {}
+        self._views: Dict[tuple, torch.Tensor] = {}        # (name, cols, dtype, rows) -> the first rows of the buffer
         self.generation = 0
 
     def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
-        key = f"{name}:{cols}:{dtype}"
+        # (a step asks for a few hundred buffers: the views are kept, one dictionary lookup each)
+        vkey = (name, cols, dtype, rows)
+        view = self._views.get(vkey)
+        if view is not None:
+            return view
+        key = (name, cols, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.shape[0] < rows:
             cap = max(rows, 1)
@@ -74,7 +80,12 @@ class Workspace:
             buf = torch.empty((cap, cols), dtype=dtype, device=self.device)
             self._buffers[key] = buf
             self.generation += 1
-        return buf[:rows]
+            for k in [k for k in self._views if k[:3] == key]:
+                del self._views[k]                           # views of the buffer that gave way
+        if len(self._views) > 4096:
+            self._views.clear()
+        view = self._views[vkey] = buf[:rows]
+        return view
 
     def reserve(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> None:
         self.get(name, rows, cols, dtype)
@@ -82,7 +93,7 @@ class Workspace:
     def zeros(self, name: str, n: int, dtype: torch.dtype = torch.int32) -> torch.Tensor:
         """A zero-filled buffer that is zeroed only when it is made: for counters that every
         kernel using them leaves at zero again."""
-        key = f"zeros:{name}:{dtype}"
+        key = ("zeros:" + name, 0, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < n:
             buf = torch.zeros(max(n, 1024 if buf is None else 2 * buf.numel()), dtype=dtype, device=self.device)

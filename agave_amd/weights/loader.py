@@ -7,10 +7,16 @@ F16 and BF16 are the floating-point types it takes).  Here every part of the mod
 tensors it needs (name, shape, and whether it holds floats or integers); all of them are
 checked before anything is read, and a single :class:`WeightError` lists the missing names, the
 names the checkpoint holds that no part asked for, the shapes that do not fit and the tensors
-stored in an element type that their use does not take.
+stored in an element type that their use does not take.  The reference's lookup by name never
+sees the tensors it does not ask for (``src/format/safetensors.zig:333-349``: the name, then the
+name under each prefix of ``hf_prefixes``, ``:517-521``), so a folder that also holds a vision
+tower loads there; here an architecture states which names are its own
+(``ModelSpec.tensor_scope``): a name nobody asked for is an error inside that scope and is passed
+over, and counted, outside it.
 """
 from __future__ import annotations
 
+import sys
 from dataclasses import dataclass
 from typing import Dict, Iterable, List, Optional, Sequence, Tuple
 
@@ -60,14 +66,23 @@ class WeightError(ValueError):
 
 
 def check_tensors(have: Dict[str, Tuple[int, ...]], needs: Iterable[TensorNeed], where: str = "",
-                  stored: Optional[Dict[str, str]] = None) -> None:
+                  stored: Optional[Dict[str, str]] = None,
+                  scope: Optional[Sequence[str]] = None) -> List[str]:
     """Raise one :class:`WeightError` if ``have`` (name -> shape) and ``needs`` differ, or if
     ``stored`` (name -> the container's name of the element type) holds a type that a tensor's
-    use does not take."""
+    use does not take.  ``scope`` lists the name prefixes that belong to the model: a name that
+    no part asked for is an error if it starts with one of them (or if ``scope`` is None) and
+    is returned, as one of the names passed over, if it does not."""
     needs = list(needs)
     wanted = {n.name for n in needs}
     missing = [n.name for n in needs if n.name not in have]
-    unexpected = sorted(n for n in have if n not in wanted)
+    unasked = sorted(n for n in have if n not in wanted)
+    if scope is None:
+        unexpected, passed_over = unasked, []
+    else:
+        own = tuple(scope)
+        unexpected = [n for n in unasked if n.startswith(own)]
+        passed_over = [n for n in unasked if not n.startswith(own)]
     wrong = [(n.name, tuple(have[n.name]), tuple(n.shape)) for n in needs
              if n.name in have and tuple(have[n.name]) != tuple(n.shape)]
     bad_type = []
@@ -76,14 +91,26 @@ def check_tensors(have: Dict[str, Tuple[int, ...]], needs: Iterable[TensorNeed],
                     if n.name in stored and not n.accepts(stored[n.name])]
     if missing or unexpected or wrong or bad_type:
         raise WeightError(missing, unexpected, wrong, where, bad_type)
+    return passed_over
+
+
+def _report_passed_over(names: Sequence[str], where: str) -> None:
+    if names:
+        heads = sorted({".".join(n.split(".")[:2]) for n in names})
+        shown = ", ".join(heads[:4]) + (", ..." if len(heads) > 4 else "")
+        print(f"[agave_amd] {where}: {len(names)} tensors that are not the model's were passed over ({shown})",
+              file=sys.stderr, flush=True)
 
 
 class WeightSource:
     """What the model builder reads tensors from: a checked checkpoint."""
 
-    def __init__(self, checkpoint: Checkpoint, needs: Iterable[TensorNeed]):
-        check_tensors({n: checkpoint.shape(n) for n in checkpoint.names()}, needs, checkpoint.model_dir,
-                      stored={n: checkpoint.stored_dtype(n) for n in checkpoint.names()})
+    def __init__(self, checkpoint: Checkpoint, needs: Iterable[TensorNeed],
+                 scope: Optional[Sequence[str]] = None):
+        self.passed_over = check_tensors(
+            {n: checkpoint.shape(n) for n in checkpoint.names()}, needs, checkpoint.model_dir,
+            stored={n: checkpoint.stored_dtype(n) for n in checkpoint.names()}, scope=scope)
+        _report_passed_over(self.passed_over, checkpoint.model_dir)
         self._ckpt = checkpoint
 
     def get(self, name: str) -> torch.Tensor:
@@ -94,9 +121,12 @@ class WeightSource:
 class DictWeightSource:
     """The same over tensors already in memory (tests, random weights without a folder)."""
 
-    def __init__(self, tensors: Dict[str, torch.Tensor], needs: Iterable[TensorNeed], where: str = "dict"):
-        check_tensors({n: tuple(t.shape) for n, t in tensors.items()}, needs, where,
-                      stored={n: _STORAGE_OF.get(t.dtype, str(t.dtype)) for n, t in tensors.items()})
+    def __init__(self, tensors: Dict[str, torch.Tensor], needs: Iterable[TensorNeed], where: str = "dict",
+                 scope: Optional[Sequence[str]] = None):
+        self.passed_over = check_tensors(
+            {n: tuple(t.shape) for n, t in tensors.items()}, needs, where,
+            stored={n: _STORAGE_OF.get(t.dtype, str(t.dtype)) for n, t in tensors.items()}, scope=scope)
+        _report_passed_over(self.passed_over, where)
         self._tensors = tensors
 
     def get(self, name: str) -> torch.Tensor:

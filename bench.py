@@ -9,7 +9,8 @@ has the layer sizes of the published Gemma 3 4B text configuration, a batch of 8
 256 decoded tokens per sequence (W warm-up steps, then K timed ones).  One JSON line is
 printed: ``value`` is decoded tokens a second; ``prefill`` is one 2,048-token prompt;
 ``roofline`` prices the decode step by the bytes it has to read (every weight once, and the
-cache of the live requests) against 8 TB/s; ``points`` holds decode at batch 1 and 64;
+cache of the live requests) against 8 TB/s; ``points`` holds decode at batch 1 and 64 and
+prompts of 256 and 512 tokens (tokens a second each);
 ``peaks_measured`` is what this machine delivered to a streaming read and to a loop of
 matrix-core instructions on random data a moment before (the fractions stay against the
 published peaks).
@@ -266,7 +267,7 @@ def main() -> int:
                    "sliding_window": m["window"], "sliding_pattern": cfg["sliding_window_pattern"],
                    "global_batch": args.batch, "seq_len": args.prompt_len + args.warmup + args.steps + 1,
                    "prompt_len": args.prompt_len,
-                   "context": args.context, "prefill_len": PREFILL_LEN, "parallelism": "single GPU",
+                   "context": args.context, "prefill_len": args.prefill_len, "parallelism": "single GPU",
                    "sampling": "greedy", "weights_gb": round(2 * (m["linear_params"] + m["table_params"]) / 1e9, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
@@ -279,14 +280,16 @@ def main() -> int:
                                  "tokens": first_step["tokens"], "ms": first_step["ms"], "sequences": len(lengths),
                                  "frac": round(flops / (first_step["ms"] * 1e-3) / PEAK_FLOPS[dkey], 4)}
     if not args.no_points:
-        pdt = run_prefill(engine, seed=2)
-        flops = prefill_flops(m, PREFILL_LEN)
-        out["prefill"] = {"value": round(PREFILL_LEN / pdt, 1), "tokens": PREFILL_LEN, "ms": round(pdt * 1e3, 3),
+        pdt = run_prefill(engine, seed=2, length=args.prefill_len)
+        flops = prefill_flops(m, args.prefill_len)
+        out["prefill"] = {"value": round(args.prefill_len / pdt, 1), "tokens": args.prefill_len, "ms": round(pdt * 1e3, 3),
                           "frac": round(flops / pdt / PEAK_FLOPS[dkey], 4)}
         points = {}
         for b, k in ((1, 64), (64, 32)):
             d, _ = run_decode(engine, b, k, 8, seed=3 + b)
             points[f"decode_b{b}"] = round(b * k / d, 2)
+        for n in (256, 512):                      # short prompts: tokens a second of one prompt of n tokens
+            points[f"prefill_{n}"] = round(n / run_prefill(engine, seed=5, length=n), 1)
         out["points"] = points
     print(json.dumps(out), flush=True)
     return 0

@@ -300,6 +300,30 @@ def test_a_half_precision_folder_is_cast_to_the_engine_s_type(tmp_path, dtype):
     close(dtype)(U.run_tail(eng, toks, 20), ref, "half-precision storage, tail")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("prefix", ["language_model.model.", "model.language_model."])
+def test_a_folder_that_holds_more_than_the_decoder(tmp_path, dtype, prefix):
+    """A folder in the layout of the published checkpoints: the text keys inside ``text_config``,
+    the decoder's tensors under a prefix, a vision tower and a projector beside them
+    (src/format/safetensors.zig:333-349, 517-521; src/arch.zig:22-23).  The logits are the plain
+    implementation's of the decoder alone."""
+    from agave_amd.engine import Engine
+    inner = P.tiny_config("A")
+    weights = P.random_weights(inner, 4)
+    raw = {"architectures": ["Gemma3ForConditionalGeneration"], "model_type": "gemma3",
+           "text_config": {k: v for k, v in inner.items() if k != "architectures"},
+           "vision_config": {"hidden_size": 8}}
+    stored = {prefix + k[len("model."):]: v.bfloat16() for k, v in weights.items()}
+    stored["vision_tower.vision_model.embeddings.patch_embedding.weight"] = torch.randn(4, 3, 2, 2).bfloat16()
+    stored["multi_modal_projector.mm_input_projection_weight"] = torch.randn(8, 8).bfloat16()
+    eng = Engine.from_folder(_save_folder(str(tmp_path / "wrapped"), raw, stored), dtype=dtype, max_slots=2,
+                             max_context=128)
+    toks = U.random_tokens(60, inner["vocab_size"], 12)
+    ref = U.plain_logits(inner, weights, toks)
+    close(dtype)(U.run_whole(eng, toks), ref, "wrapped folder, whole")
+    close(dtype)(U.run_tail(eng, toks, 20), ref, "wrapped folder, tail")
+
+
 @pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "float32"), ("B", "bfloat16")])
 def test_random_schedules_of_ragged_steps(tmp_path, which, dtype):
     """Forty steps whose make-up is drawn at random: some sequences bring many tokens and others one
@@ -408,7 +432,7 @@ def test_wide_batches_at_a_published_size(tmp_path, n_seqs):
     eng = Engine.from_folder(folder, dtype="bfloat16", max_slots=n_seqs, max_context=128)
     reqs = [U.random_tokens(30 + i % 7, cfg["vocab_size"], 40 + i) for i in range(n_seqs)]
     outs = U.run_batched(eng, reqs, [14 + i % 5 for i in range(n_seqs)])
-    for i in (0, 1, n_seqs // 2, n_seqs - 2, n_seqs - 1):
+    for i in range(n_seqs):
         close("bfloat16")(outs[i], U.plain_logits(cfg, weights, reqs[i]), f"request {i} of {n_seqs}")
 
 

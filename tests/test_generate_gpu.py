@@ -209,6 +209,52 @@ def test_trace_tool_whole_tail_and_batches(model_b, dtype, tmp_path):
     assert not os.path.exists(str(tmp_path / "none" / "0.f32"))
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_tool_cuts_whole_requests_itself(dtype, tmp_path):
+    """bin/trace_run --trace FILE --mode whole|tail32|batched on a model it makes itself from a
+    configuration and a seed (random:CONFIG.json:SEED): every mode gives each request's logits at
+    every position, equal to the plain implementation's on the weights the tool wrote."""
+    from agave_amd.weights import Checkpoint
+    cfg = P.tiny_config("A")
+    cfg_path = str(tmp_path / "cfg.json")
+    with open(cfg_path, "w") as f:
+        json.dump(cfg, f)
+    v = cfg["vocab_size"]
+    lens = (50, 70, 5, 41)
+    reqs = [{"id": f"r{i}", "tokens": U.random_tokens(n, v, 500 + i), "prompt": p, "batch": i // 3}
+            for i, (n, p) in enumerate(zip(lens, (20, 64, 1, 41)))]
+    trace = str(tmp_path / "trace.jsonl")
+    with open(trace, "w") as f:
+        for r in reqs:
+            f.write(json.dumps(r) + "\n")
+    refs = None
+    for mode in ("whole", "tail32", "batched"):
+        out = str(tmp_path / mode)
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", f"random:{cfg_path}:5",
+                               "--dtype", dtype, "--out", out, "--trace", trace, "--mode", mode],
+                              capture_output=True, text=True, timeout=600)
+        assert proc.returncode == 0, proc.stderr[-3000:]
+        if refs is None:
+            ck = Checkpoint(os.path.join(out, "model"))
+            w = {n: ck.read(n).double() for n in ck.names()}
+            refs = [U.plain_logits(cfg, w, r["tokens"]) for r in reqs]
+        index = json.load(open(os.path.join(out, "index.json")))
+        assert index["mode"] == mode and sorted(index["requests"]) == [r["id"] for r in reqs]
+        steps = [int(l.split()[1]) for l in proc.stdout.splitlines() if l.startswith("done ")]
+        assert steps == list(range(len(steps)))
+        # whole: a step a request; tail32: one and its tail each; batched: two batches, the longest request sets the steps
+        assert len(steps) == {"whole": 4, "tail32": sum(1 + min(32, n - 1) for n in lens),
+                              "batched": (1 + max(50 - 20, 70 - 64, 5 - 1)) + 1}[mode]
+        for r, ref in zip(reqs, refs):
+            meta = index["requests"][r["id"]]
+            got = torch.from_numpy(np.fromfile(os.path.join(out, meta["file"]), dtype="<f4").reshape(meta["positions"], meta["vocab"])).double()
+            assert got.shape == ref.shape
+            if dtype == "float32":
+                assert float((got - ref).abs().max()) < 3e-5, (mode, r["id"])
+            else:
+                assert float(((got - ref).abs().max(-1).values / ref.abs().max(-1).values).max()) < 0.04, (mode, r["id"])
+
+
 def test_steps_launched_ahead_give_the_tokens_of_steps_run_one_by_one(model_b):
     """launch_step with tokens carried on the device (also for a shrinking subset of the rows, in
     another order) against step_sample fed from the host."""

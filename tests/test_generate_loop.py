@@ -227,8 +227,16 @@ def test_a_cancelled_call_returns_what_it_has_and_loses_no_slot(backend_cls):
                 self.flag = True                      # as if another thread had called cancel() during this step
             return out
 
+    # a request to cancel that arrives before the call's first step ends it there, and is used up by it
+    be = Cancellable(10 ** 9, max_slots=2, max_context=64)
+    be.flag = True
+    res = generate(be, [[10], [20], [30]], SamplingParams(max_tokens=5), eos_ids=[])
+    assert [r.finish_reason for r in res] == ["cancelled"] * 3 and all(r.tokens == [] for r in res)
+    assert be.steps == [] and sorted(be.free) == [0, 1] and be.cleared == 1 and not be.flag
+    res = generate(be, [[10]], SamplingParams(max_tokens=2), eos_ids=[])
+    assert res[0].finish_reason == "length" and be.cleared == 1           # nothing to clear in a call that ran through
+
     be = Cancellable(4, max_slots=2, max_context=64)
-    be.flag = True                                    # left over from an earlier call: does not count
     res = generate(be, [[10], [20], [30]], [SamplingParams(max_tokens=2), SamplingParams(max_tokens=30),
                                             SamplingParams(max_tokens=30)], eos_ids=[])
     assert be.cleared == 1
@@ -253,3 +261,45 @@ def test_log_probabilities_go_to_the_requests_that_ask():
     res = generate(be, [[10], [20]], [SamplingParams(max_tokens=3, logprobs=True), SamplingParams(max_tokens=3)], eos_ids=[13])
     assert res[0].tokens == [11, 12] and res[0].finish_reason == "stop"            # 13 stops it and is not emitted
     assert res[0].logprobs == [-1.2, -1.3] and res[1].logprobs == [] and res[1].tokens == [21, 22, 23]
+
+
+def test_replay_cuts_requests_into_the_steps_of_each_mode():
+    """The step records that bin/trace_run makes from whole requests: every position is fed once,
+    in order, and its logits are found where the plan says; batches end their requests as their
+    tokens run out and never hold more than the plan's count of tokens."""
+    from agave_amd.engine.replay import plan_steps, tokens_held
+    reqs = [{"id": "a", "tokens": list(range(100, 140)), "prompt": 10, "batch": 0},
+            {"id": "b", "tokens": list(range(200, 203)), "prompt": 3, "batch": 0},
+            {"id": "c", "tokens": list(range(300, 370)), "batch": 1}]
+    for mode in ("whole", "tail32", "batched"):
+        records, where = plan_steps(mode, reqs)
+        fed = {r["id"]: [] for r in reqs}
+        live, ended = set(), set()
+        for i, rec in enumerate(records):
+            assert rec["step"] == i
+            sizes = {len(e["tokens"]) for e in rec["entries"]}
+            starts = [e["id"] not in live for e in rec["entries"]]
+            assert all(starts) or (not any(starts) and sizes == {1})      # all start, or all go on by one token
+            row = 0
+            for e in rec["entries"]:
+                assert e["id"] not in ended and e["want"] == list(range(len(e["tokens"])))
+                for k, t in enumerate(e["tokens"]):
+                    assert where[e["id"]][len(fed[e["id"]])] == (i, row + k)
+                    fed[e["id"]].append(t)
+                row += len(e["tokens"])
+                live.add(e["id"])
+            for rid in rec["end"]:
+                live.discard(rid)
+                ended.add(rid)
+        assert fed == {r["id"]: r["tokens"] for r in reqs} and not live
+        if mode == "whole":
+            assert [len(r["entries"]) for r in records] == [1, 1, 1] and tokens_held(records) == 128
+        if mode == "tail32":
+            assert len(records) == (1 + 32) + (1 + 2) + (1 + 32)
+        if mode == "batched":
+            assert [e["id"] for e in records[0]["entries"]] == ["a", "b"] and records[0]["end"] == ["b"]
+            assert len(records) == (1 + 30) + (1 + 32) and tokens_held(records) == 128
+    with pytest.raises(ValueError, match="unknown mode"):
+        plan_steps("sideways", reqs)
+    with pytest.raises(ValueError, match="must differ"):
+        plan_steps("whole", [reqs[0], reqs[0]])

@@ -87,6 +87,70 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     check_tensors({"a": (1,)}, [TensorNeed("a", (1,))])
 
 
+def _wrapped(which, prefix, seed=0):
+    """A tiny configuration as the language model of a folder that holds more than it: the
+    text keys inside ``text_config``, the decoder's tensors under ``prefix``."""
+    inner = P.tiny_config(which)
+    raw = {"architectures": ["Gemma3ForConditionalGeneration"], "model_type": "gemma3",
+           "text_config": {k: v for k, v in inner.items() if k != "architectures"},
+           "vision_config": {"hidden_size": 8}}
+    w = {prefix + k[len("model."):] if k.startswith("model.") else k: v
+         for k, v in P.random_weights(inner, seed).items()}
+    w["vision_tower.vision_model.encoder.layers.0.mlp.fc1.weight"] = torch.zeros(3, 2)
+    w["multi_modal_projector.mm_input_projection_weight"] = torch.zeros(2, 2)
+    return inner, raw, w
+
+
+@pytest.mark.parametrize("prefix", ["language_model.model.", "model.language_model."])
+def test_a_folder_that_holds_more_than_the_decoder_loads(tmp_path, prefix, capfd):
+    """The reference finds a tensor by its name under "model.language_model.", "language_model.model."
+    or "model." (src/format/safetensors.zig:333-349, 517-521) and never looks at the others, and
+    "gemma3" is one of the model types of this architecture (src/arch.zig:22-23): a vision tower
+    and a projector beside the decoder are passed over, and counted; a stray name under the
+    decoder's own prefix is still an error."""
+    from safetensors.torch import save_file
+    inner, raw, w = _wrapped("A", prefix)
+    arch = find_architecture(raw)
+    cfg = arch.parse(raw)
+    assert cfg == arch.parse(inner)
+    spec = arch.spec(cfg, w.keys())
+    assert spec.embed_weight == prefix + "embed_tokens.weight" and spec.tensor_scope == (prefix, "lm_head.")
+    src = DictWeightSource(w, tensor_needs(spec), scope=spec.tensor_scope)
+    assert sorted(src.passed_over) == ["multi_modal_projector.mm_input_projection_weight",
+                                      "vision_tower.vision_model.encoder.layers.0.mlp.fc1.weight"]
+    assert "2 tensors that are not the model's were passed over" in capfd.readouterr().err
+    save_file({k: v.bfloat16().contiguous() for k, v in w.items()}, str(tmp_path / "model.safetensors"))
+    assert len(WeightSource(Checkpoint(str(tmp_path)), tensor_needs(spec), spec.tensor_scope).passed_over) == 2
+    # without a scope every name counts, as for a model that owns its whole folder
+    with pytest.raises(WeightError) as ei:
+        DictWeightSource(w, tensor_needs(spec))
+    assert len(ei.value.unexpected) == 2
+    # inside the scope nothing is passed over
+    w[prefix + "layers.9.extra.weight"] = torch.zeros(1)
+    w["lm_head.bias"] = torch.zeros(1)
+    del w[prefix + "norm.weight"]
+    with pytest.raises(WeightError) as ei:
+        DictWeightSource(w, tensor_needs(spec), scope=spec.tensor_scope)
+    assert ei.value.unexpected == sorted(["lm_head.bias", prefix + "layers.9.extra.weight"])
+    assert ei.value.missing == [prefix + "norm.weight"]
+
+
+def test_a_plain_text_folder_owns_every_name_under_its_prefix():
+    """With the "model." prefix a foreign tower would sit under another top-level name; anything
+    under "model." that no part asked for stays an error."""
+    raw, needs = _needs("A")
+    arch = find_architecture(raw)
+    w = P.random_weights(raw, 0)
+    spec = arch.spec(arch.parse(raw), w.keys())
+    assert spec.tensor_scope == ("model.", "lm_head.")
+    w["model.vision_tower.x"] = torch.zeros(1)
+    with pytest.raises(WeightError, match="unexpected"):
+        DictWeightSource(w, needs, scope=spec.tensor_scope)
+    del w["model.vision_tower.x"]
+    w["vision_tower.x"] = torch.zeros(1)
+    assert DictWeightSource(w, needs, scope=spec.tensor_scope).passed_over == ["vision_tower.x"]
+
+
 def test_element_types_are_checked_in_the_same_error(tmp_path):
     """A matrix must be stored as BF16, F16 or F32 (what the reference's loader takes as floats,
     src/format/safetensors.zig:1605-1616); integers, doubles and booleans in its place are listed by

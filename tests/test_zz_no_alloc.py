@@ -52,6 +52,7 @@ class Case:
         self.table, self.base = table.to(DEV), _i32([0] * len(lens))
         k = torch.randn(sum(lens), nkv * hd, generator=g).bfloat16().to(DEV)
         v = torch.randn(sum(lens), nkv * hd, generator=g).bfloat16().to(DEV)
+        self.k, self.v = k, v
         seq_all = _i32([b for b, L in enumerate(lens) for _ in range(L)])
         pos_all = _i32([i for L in lens for i in range(L)])
         kernels.qk_norm_rope_kv(None, k, v, None, None, None, 0.0, 0.0, None, 1.0, seq_all, pos_all, self.kp, self.vp,
@@ -63,9 +64,29 @@ class Case:
         self.span = max((L + 63) // 64 for L in lens)
 
     def plan(self):
+        """The engine's own plan for these sizes (the kernel for this head size shares half pages
+        among the splits and looks at the number of splits only)."""
         from agave_amd.ops import attention_mfma
         chunks = -(-(self.nh // self.nkv) // 16)
-        return attention_mfma.split_plan(self.span, len(self.lens) * self.nkv * chunks)
+        return attention_mfma.split_plan(self.span, len(self.lens) * self.nkv * chunks, self.hd)
+
+    def scale(self):
+        return 0.3 * (16 / self.hd) ** 0.5
+
+    def plain(self):
+        """softmax(q k^T * scale) v per sequence and head in float64, from the rows as they were given."""
+        G, outs, at = self.nh // self.nkv, [], 0
+        for b, L in enumerate(self.lens):
+            k = self.k[at:at + L].double().cpu().view(L, self.nkv, self.hd)
+            v = self.v[at:at + L].double().cpu().view(L, self.nkv, self.hd)
+            q = self.q[b].double().cpu().view(self.nh, self.hd)
+            rows = []
+            for h in range(self.nh):
+                w = torch.softmax(k[:, h // G] @ q[h] * self.scale(), 0)
+                rows.append(w @ v[:, h // G])
+            outs.append(torch.cat(rows))
+            at += L
+        return torch.stack(outs)
 
     def run(self, lib, noalloc: bool, splits=None, per=None):
         n = len(self.lens)
@@ -75,7 +96,7 @@ class Case:
         stream = torch.cuda.current_stream().cuda_stream
         tail = (self.kp.data_ptr(), self.vp.data_ptr(), self.table.data_ptr(), self.width, self.base.data_ptr(),
                 self.n_pages, self.tok_seq.data_ptr(), self.tok_pos.data_ptr(), n, self.nh, self.nkv, self.hd,
-                0.3 * (16 / self.hd) ** 0.5, 0, splits, per, 1, 0, stream)
+                self.scale(), 0, splits, per, 1, 0, stream)
         if noalloc:
             rc = lib.agave_attn_decode_mfma_noalloc(self.q.data_ptr(), self.q.stride(0), out.data_ptr(), out.stride(0), *tail)
         else:
@@ -98,6 +119,8 @@ def test_two_calls_in_a_row_equal_the_entry_point_with_caller_buffers():
         rc, ref = case.run(lib, noalloc=False)
         assert rc == 0, lib.agave_last_error()
         refs.append(ref)
+        # the entry point it is compared with is itself right at these split counts
+        assert torch.allclose(ref.double().cpu(), case.plain(), atol=2e-2, rtol=2e-2)
     # the two calls follow each other on one stream with nothing between them
     rc1, out1 = big.run(lib, noalloc=True)
     rc2, out2 = small.run(lib, noalloc=True)
@@ -110,6 +133,12 @@ def test_two_calls_in_a_row_equal_the_entry_point_with_caller_buffers():
     rc3, out3 = big.run(lib, noalloc=True)
     torch.cuda.synchronize()
     assert rc3 == 0 and torch.equal(out3, refs[0])
+    # a batch of one at the engine's twelve splits
+    single = Case([1500], 8, 4, 256, seed=5)
+    assert single.plan()[0] == 12
+    rc, out = single.run(lib, noalloc=True)
+    torch.cuda.synchronize()
+    assert rc == 0 and torch.allclose(out.double().cpu(), single.plain(), atol=2e-2, rtol=2e-2)
     # one share a sequence: nothing of the array is used
     rc, whole = small.run(lib, noalloc=True, splits=1, per=small.span)
     torch.cuda.synchronize()
