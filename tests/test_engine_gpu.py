@@ -432,8 +432,9 @@ def test_wide_batches_at_a_published_size(tmp_path, n_seqs):
     eng = Engine.from_folder(folder, dtype="bfloat16", max_slots=n_seqs, max_context=128)
     reqs = [U.random_tokens(30 + i % 7, cfg["vocab_size"], 40 + i) for i in range(n_seqs)]
     outs = U.run_batched(eng, reqs, [14 + i % 5 for i in range(n_seqs)])
+    wide = {k: v.double() for k, v in weights.items()}        # (widened once: every request is checked)
     for i in range(n_seqs):
-        close("bfloat16")(outs[i], U.plain_logits(cfg, weights, reqs[i]), f"request {i} of {n_seqs}")
+        close("bfloat16")(outs[i], U.plain_logits(cfg, wide, reqs[i]), f"request {i} of {n_seqs}")
 
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
