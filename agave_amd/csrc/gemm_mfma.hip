@@ -1123,6 +1123,8 @@ static int dispatch_tiled(const void* X, long ldx, const void* Wp, void* Y, long
 // round two thirds full, where they gained 2 %).  Shorter prompts gain as much: down at 1,024 tokens takes 59 us
 // in three slices of 80 tiles instead of 81 us in 160 tiles of 128 x 128 (a prefill of 384 to
 // 1,024 tokens 2 to 5 % less).
+struct SlicePlan { int tile; int z; };      // tile: 0 256 x 256, 1 128 x 256, 2 128 x 128, 3 64 x 128 (weight rows x tokens)
+
 static int cut_tiled_slices(int M, int N, int K) {
     const long NB = (N + 15) / 16;
     const long rows16 = (NB + 15) / 16, rows8 = (NB + 7) / 8;
@@ -1149,34 +1151,115 @@ static int cut_tiled_slices(int M, int N, int K) {
     return z_best;
 }
 
+static SlicePlan plan_tiled_slices(int M, int N, int K) {
+    // Short prompts (up to 128 tiles of 64 x 128: some 400 tokens at 2,560 rows): as many slices of
+    // those tiles as fit one round of 256 workgroups, each with at least six stages.  Measured at
+    // 2,560 rows, 96 to 384 tokens: 10,240 columns take 17 to 36 us so (4 slices of 128 x 256 tiles:
+    // 34 to 40; one product: 28 to 52), 2,048 columns 7 to 11 us (one product and a kernel that adds
+    // its shares: 12 to 15).
+    {
+        const long rows4 = ((N + 15) / 16 + 3) / 4, t128 = (M + 127) / 128;
+        const long small = rows4 * t128;
+        if (small <= 128) {
+            const int n_stage = (K + 63) / 64;
+            int z = (int)(256 / small);
+            if (z > 8) z = 8;
+            while (z > 1 && n_stage / z < 6) --z;
+            if (z > 1) return SlicePlan{3, z};
+        }
+    }
+    const int z = cut_tiled_slices(M, N, K);
+    // 256 x 256 tiles where the slices of those fill the compute units in one round (down of the 4B
+    // sizes at 2,048 tokens: 240 workgroups, 112 us; as 480 of 128 x 256: 119)
+    const long NB = (N + 15) / 16;
+    const long big = (long)((NB + 15) / 16) * ((M + 255) / 256) * z;
+    return SlicePlan{(big > 192 && big <= 256) ? 0 : 1, z};
+}
+
 // How many 32-bit slices a product of M > 64 tokens is best computed in by a caller that can
 // add them up (1: as one product).
 extern "C" int agave_gemm_tiled_slices(int M, int N, int K) {
     if (M <= 64 || N <= 0 || K <= 0 || K % 8 != 0) return 1;
-    return cut_tiled_slices(M, N, K);
+    return plan_tiled_slices(M, N, K).z;
+}
+
+// The slices of a product in tiles of a given shape (0: 256 x 256, 1: 128 x 256, 2: 128 x 128,
+// 3: 64 x 128, weight rows x tokens).
+static int launch_slices(int tile, const void* X, long ldx, const void* Wp, float* Y, int M, int N, int K, int z,
+                         hipStream_t stream) {
+    const int KB = (K + 31) / 32, NB = (N + 15) / 16;
+    const long stride = (long)M * N;
+    switch (tile) {
+        case 0: return launch_tiled<4, 1, 4, 0, float, 8, 256, true>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, stride);
+        case 1: return launch_tiled<2, 2, 3, 0, float, 8, 256, false>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, stride);
+        case 2: return launch_tiled<2, 2, 3, 0, float, 8, 128, false>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, stride);
+        default: return launch_tiled<1, 2, 4, 0, float, 8, 128, false>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, stride);
+    }
+}
+
+static int check_slices_args(const char* who, const void* X, long ldx, int M, int N, int K) {
+    AGAVE_CHECK(M > 64 && N > 0 && K > 0, "%s: bad sizes M=%d N=%d K=%d", who, M, N, K);
+    AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
+                "%s: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", who, K, ldx);
+    AGAVE_CHECK(ldx >= K && ldx < (1L << 22), "%s: bad row stride %ld", who, ldx);
+    return 0;
 }
 
 // Y: 32-bit [z][M][N], z = agave_gemm_tiled_slices(M, N, K) > 1; slice s gets the sums over the
 // s-th run of columns of X W^T.
 extern "C" int agave_gemm_tiled_in_slices(const void* X, long ldx, const void* Wp, float* Y, int M, int N, int K,
                                           int z, hipStream_t stream) {
-    AGAVE_CHECK(M > 64 && N > 0 && K > 0, "gemm_tiled_in_slices: bad sizes M=%d N=%d K=%d", M, N, K);
-    AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
-                "gemm_tiled_in_slices: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
-    AGAVE_CHECK(ldx >= K && ldx < (1L << 22), "gemm_tiled_in_slices: bad row stride %ld", ldx);
-    const int planned = cut_tiled_slices(M, N, K);
-    AGAVE_CHECK(z > 1 && z == planned, "gemm_tiled_in_slices: %d slices asked for, %d planned", z, planned);
-    const int KB = (K + 31) / 32, NB = (N + 15) / 16;
-    // 256 x 256 tiles where the slices of those fill the compute units in one round (down of the 4B
-    // sizes at 2,048 tokens: 240 workgroups, 112 us; as 480 of 128 x 256: 119)
-    const long big = (long)((NB + 15) / 16) * ((M + 255) / 256) * z;
-    int rc;
-    if (big > 192 && big <= 256)
-        rc = launch_tiled<4, 1, 4, 0, float, 8, 256, true>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, (long)M * N);
-    else
-        rc = launch_tiled<2, 2, 3, 0, float, 8, 256, false>(X, ldx, Wp, Y, N, M, N, K, KB, NB, stream, z, (long)M * N);
-    if (rc != 0) return rc;
+    if (check_slices_args("gemm_tiled_in_slices", X, ldx, M, N, K)) return -1;
+    const SlicePlan plan = plan_tiled_slices(M, N, K);
+    AGAVE_CHECK(z > 1 && z == plan.z, "gemm_tiled_in_slices: %d slices asked for, %d planned", z, plan.z);
+    if (launch_slices(plan.tile, X, ldx, Wp, Y, M, N, K, z, stream) != 0) return -1;
     AGAVE_LAUNCH_CHECK("gemm_tiled_in_slices");
+    return 0;
+}
+
+// The same with the tile shape and the number of slices given by the caller (tile 0: 256 x 256,
+// 1: 128 x 256, 2: 128 x 128, 3: 64 x 128): for tests of every shape and for measurements.  z = 1
+// leaves the whole product in the one slice.
+extern "C" int agave_gemm_tiled_in_slices_as(const void* X, long ldx, const void* Wp, float* Y, int M, int N, int K,
+                                             int tile, int z, hipStream_t stream) {
+    if (check_slices_args("gemm_tiled_in_slices_as", X, ldx, M, N, K)) return -1;
+    const int n_stage = tile == 0 ? (K + 31) / 32 : (K + 63) / 64;
+    AGAVE_CHECK(tile >= 0 && tile <= 3 && z >= 1 && z <= 16 && z <= n_stage, "gemm_tiled_in_slices_as: tile %d in %d slices of %d stages",
+                tile, z, n_stage);
+    if (launch_slices(tile, X, ldx, Wp, Y, M, N, K, z, stream) != 0) return -1;
+    AGAVE_LAUNCH_CHECK("gemm_tiled_in_slices_as");
+    return 0;
+}
+
+// One product in tiles of a shape the caller names (0: 256 x 256, 1: 128 x 256, 2: 128 x 128,
+// 3: 64 x 128), whatever agave_gemm_tiled would choose: for tests of every shape and for measurements.
+template <int EPI, typename TC>
+static int launch_tile_shape(int tile, const void* X, long ldx, const void* Wp, void* Y, long ldy, int M, int N, int K,
+                             int KB, int NB, hipStream_t stream) {
+    switch (tile) {
+        case 0: return launch_tiled<4, 1, 4, EPI, TC, 8, 256, true>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 1: return launch_tiled<2, 2, 3, EPI, TC, 8, 256, false>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        case 2: return launch_tiled<2, 2, 3, EPI, TC, 8, 128, false>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+        default: return launch_tiled<1, 2, 4, EPI, TC, 8, 128, false>(X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    }
+}
+
+extern "C" int agave_gemm_tiled_as(const void* X, long ldx, const void* Wp, int dt_y, void* Y, long ldy, int M, int N,
+                                   int K, int epilogue, int tile, hipStream_t stream) {
+    AGAVE_CHECK(M > 0 && N > 0 && K > 0 && tile >= 0 && tile <= 3, "gemm_tiled_as: bad sizes M=%d N=%d K=%d or tile %d", M, N, K, tile);
+    AGAVE_CHECK(K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)X % 16) == 0,
+                "gemm_tiled_as: X must be 16-byte aligned with K and its row stride multiples of 8 (K=%d ldx=%ld)", K, ldx);
+    AGAVE_CHECK(ldx >= K && ldy >= N && ldx < (1L << 22), "gemm_tiled_as: bad row strides");
+    AGAVE_CHECK((epilogue == 0 && (dt_y == AGAVE_BF16 || dt_y == AGAVE_F32)) || (epilogue == 1 && dt_y == AGAVE_BF16),
+                "gemm_tiled_as: epilogue %d with output dtype %d", epilogue, dt_y);
+    const int KB = (K + 31) / 32;
+    const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
+    int rc;
+    if (epilogue == 1) rc = launch_tile_shape<1, bf16>(tile, X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    else if (dt_y == AGAVE_BF16) rc = launch_tile_shape<0, bf16>(tile, X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    else rc = launch_tile_shape<0, float>(tile, X, ldx, Wp, Y, ldy, M, N, K, KB, NB, stream);
+    if (rc != 0) return rc;
+    AGAVE_LAUNCH_CHECK("gemm_tiled_as");
     return 0;
 }
 

@@ -14,7 +14,7 @@ import torch
 
 from ..cache import GroupKey, StateNeed
 from ..config.spec import ModelSpec
-from ..ops import kernels
+from ..ops import gemm_mfma, kernels
 from ..parts import BuildEnv, Linear, add_pending_and_norm, lookup, part_tensors
 from ..weights.loader import TensorNeed
 
@@ -95,7 +95,6 @@ class Model:
         if self.embed_table is not None:
             kernels.embed_scale(step.tokens, self.embed_table, self.spec.embed_scale, h)
         else:
-            from ..ops import gemm_mfma
             gemm_mfma.embed_scale_packed(step.tokens, self.head.packed, self.spec.embed_scale, h, self.spec.vocab_size)
         pending = None
         for entry in self.spec.order:

@@ -5,7 +5,7 @@ from typing import Optional
 
 import torch
 
-from . import kernels
+from . import attention_mfma, kernels
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
@@ -15,7 +15,6 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
     step's own keys and values).  Pages in the matrix cores' tile order go to the MFMA kernels,
     pages stored row by row to the plain kernel."""
     if packed:
-        from . import attention_mfma
         attention_mfma.attention(q, out, k_pages, v_pages, table, base, step, n_heads, n_kv, head_dim, scale, window)
         return
     kernels.attn_plain(q, out, k_pages, v_pages, table, base, step.tok_seq, step.tok_pos,
@@ -32,7 +31,6 @@ def qk_attention(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.T
     ``q_rot``) and the attention kernel after it.  ``partials_ok``: see
     :func:`agave_amd.ops.attention_mfma.decode_fused`; returns the partial results or None."""
     if packed and step.is_decode:
-        from . import attention_mfma
         if head_dim in attention_mfma.FUSED_HEAD_DIMS:
             return attention_mfma.decode_fused(q, k, v, out, q_gain, k_gain, eps_q, eps_k, inv_freq, pos_scale, k_pages,
                                                v_pages, table, base, step, n_heads, n_kv, head_dim, scale, window,

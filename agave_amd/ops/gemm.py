@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import torch
 
-from . import kernels
+from . import gemm_mfma, kernels
 
 
 def linear(x: torch.Tensor, lin, out: torch.Tensor) -> None:
@@ -13,7 +13,6 @@ def linear(x: torch.Tensor, lin, out: torch.Tensor) -> None:
     if out.shape != (x.shape[0], lin.out_features):
         raise ValueError(f"{lin.name}: output is {tuple(out.shape)}, needs {(x.shape[0], lin.out_features)}")
     if getattr(lin, "packed", None) is not None:
-        from . import gemm_mfma
         if gemm_mfma.try_linear(x, lin, out):
             return
         raise ValueError(f"{lin.name}: the matrix-core product needs a 16-byte aligned bfloat16 input whose row "

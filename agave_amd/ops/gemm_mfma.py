@@ -16,6 +16,8 @@ kernels.register_signatures("gemm_mfma", {
     "agave_gemm_tiled_slices": [_I, _I, _I],
     "agave_gemm_tiled_in_slices": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
     "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P, _L, _P],
+    "agave_gemm_tiled_as": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _I, _P],
+    "agave_gemm_tiled_in_slices_as": [_P, _L, _P, _P, _I, _I, _I, _I, _I, _P],
     "agave_oproj_combine_heads_per_run": [_I, _I, _I, _I],
     "agave_gemm_oproj_combine": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P],
 })
@@ -80,7 +82,7 @@ def tiled_slices_for(m: int, n_out: int, k: int) -> int:
     got = _slices.get(key)
     if got is None:
         got = 1
-        if m > SKINNY_MAX_M and m * n_out * 4 * 4 <= TILED_SLICES_MAX_BYTES:
+        if m > SKINNY_MAX_M and m * n_out * 4 * 8 <= TILED_SLICES_MAX_BYTES:       # (at most eight slices)
             got = int(kernels.lib("gemm_mfma").agave_gemm_tiled_slices(m, n_out, k))
         _slices[key] = got
     return got
@@ -103,6 +105,37 @@ def tiled_slices(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out
         raise ValueError("packed product: the packed weight does not fit these sizes")
     library.call(kernels.lib("gemm_mfma"), "agave_gemm_tiled_in_slices", x.data_ptr(), x.stride(0), packed.data_ptr(),
                  out.data_ptr(), m, n_out, k, out.shape[0], kernels.stream())
+
+
+TILE_SHAPES = ((256, 256), (128, 256), (128, 128), (64, 128))       # weight rows x tokens a workgroup
+
+
+def tiled_as(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, tile: int, epilogue: int = 0) -> None:
+    """:func:`product` in tiles of ``TILE_SHAPES[tile]`` whatever the library would choose (tests of
+    every tile shape, measurements)."""
+    if not (x.is_cuda and packed.is_cuda and out.is_cuda) or not _x_ok(x):
+        raise ValueError("packed product: bfloat16 GPU rows, 16-byte aligned, K and the row stride multiples of 8")
+    m, k = x.shape
+    if out.dim() != 2 or out.shape != (m, n_out) or out.stride(1) != 1:
+        raise ValueError(f"packed product: out must be [{m}, {n_out}] with contiguous rows")
+    nb = (n_out + 7) // 8 if epilogue else (n_out + 15) // 16
+    if packed.numel() != nb * ((k + 31) // 32) * 512:
+        raise ValueError("packed product: the packed weight does not fit these sizes")
+    library.call(kernels.lib("gemm_mfma"), "agave_gemm_tiled_as", x.data_ptr(), x.stride(0), packed.data_ptr(),
+                 kernels.dt(out), out.data_ptr(), out.stride(0), m, n_out, k, epilogue, tile, kernels.stream())
+
+
+def tiled_slices_as(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, tile: int) -> None:
+    """:func:`tiled_slices` with the tile shape and the number of slices (``out.shape[0]``) given."""
+    if not (x.is_cuda and packed.is_cuda and out.is_cuda) or not _x_ok(x):
+        raise ValueError("packed product: bfloat16 GPU rows, 16-byte aligned, K and the row stride multiples of 8")
+    m, k = x.shape
+    if out.dtype != torch.float32 or out.dim() != 3 or out.shape[1:] != (m, n_out) or not out.is_contiguous():
+        raise ValueError(f"partial sums must be a contiguous float32 [slices, {m}, {n_out}] tensor")
+    if packed.numel() != ((n_out + 15) // 16) * ((k + 31) // 32) * 512:
+        raise ValueError("packed product: the packed weight does not fit these sizes")
+    library.call(kernels.lib("gemm_mfma"), "agave_gemm_tiled_in_slices_as", x.data_ptr(), x.stride(0), packed.data_ptr(),
+                 out.data_ptr(), m, n_out, k, tile, out.shape[0], kernels.stream())
 
 
 def skinny_slices(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int) -> None:

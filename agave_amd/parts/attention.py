@@ -30,6 +30,7 @@ class Attention:
         self.env = env
         self.qd = spec.n_heads * spec.head_dim
         self.kvd = spec.n_kv_heads * spec.head_dim
+        self._qkv_bounds = (0, self.qd, self.qd + self.kvd, self.qd + 2 * self.kvd)
         # q, k and v in one product: rows of the three matrices stacked
         self.qkv = Linear([weights.get(spec.q_proj), weights.get(spec.k_proj), weights.get(spec.v_proj)], env, "qkv")
         self.o = Linear([weights.get(spec.o_proj)], env, "attn_o")
@@ -60,7 +61,7 @@ class Attention:
         table, base = step.tables[step.cache.group_of_memory[memory]]
         fused = getattr(self.position, "fused_rotation", None)
         qkv = self.qkv.forward(x, tag="qkv")
-        q, k, v = qkv[:, :self.qd], qkv[:, self.qd:self.qd + self.kvd], qkv[:, self.qd + self.kvd:]
+        q, k, v = ws.columns(qkv, self._qkv_bounds)
         if not writes:
             k = v = None            # a run that reads another run's cache appends nothing
         q_out = ws.get("q_rot", n, self.qd, x.dtype)

@@ -80,12 +80,28 @@ class Workspace:
             buf = torch.empty((cap, cols), dtype=dtype, device=self.device)
             self._buffers[key] = buf
             self.generation += 1
-            for k in [k for k in self._views if k[:3] == key]:
-                del self._views[k]                           # views of the buffer that gave way
+            self._views.clear()                              # views of the buffer that gave way (and what was made of them)
         if len(self._views) > 4096:
             self._views.clear()
         view = self._views[vkey] = buf[:rows]
         return view
+
+    def get3(self, name: str, slices: int, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
+        """``slices`` buffers of [rows, cols] behind each other, as one [slices, rows, cols] tensor."""
+        flat = self.get(name, slices * rows, cols, dtype)
+        key = (name, cols, dtype, slices * rows, slices)
+        view = self._views.get(key)
+        if view is None or view.data_ptr() != flat.data_ptr():
+            view = self._views[key] = flat.view(slices, rows, cols)
+        return view
+
+    def columns(self, t: torch.Tensor, bounds) -> tuple:
+        """``t[:, bounds[i]:bounds[i + 1]]`` for every i, made once per tensor kept here and bounds."""
+        key = ("columns", t.data_ptr(), t.shape[0], t.stride(0), bounds)
+        got = self._views.get(key)
+        if got is None:
+            got = self._views[key] = tuple(t[:, lo:hi] for lo, hi in zip(bounds[:-1], bounds[1:]))
+        return got
 
     def reserve(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> None:
         self.get(name, rows, cols, dtype)

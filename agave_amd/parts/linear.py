@@ -13,7 +13,7 @@ from typing import List, Optional, Sequence
 
 import torch
 
-from ..ops import kernels
+from ..ops import gemm, gemm_mfma, kernels, library
 from .base import BuildEnv
 
 
@@ -44,7 +44,6 @@ class Linear:
         self.name = name
         self.packed = None          # the weight in the matrix cores' tile layout (bfloat16 engines)
         if pack and env.dtype == torch.bfloat16 and self.weight.dtype == torch.bfloat16 and self.in_features % 8 == 0:
-            from ..ops import gemm_mfma
             self.packed = gemm_mfma.pack_weight(self.weight, interleave_ff=interleave_ff)
             self.weight = None      # only the packed copy is kept
         elif env.dtype == torch.bfloat16 and self.weight.dtype == torch.float32:
@@ -59,19 +58,16 @@ class Linear:
         with few rows of W and many columns is then shared out along the columns."""
         n = x.shape[0]
         if slices_ok and out is None and self.packed is not None and not self.interleave_ff:
-            from ..ops import gemm_mfma, library
             many = n > gemm_mfma.SKINNY_MAX_M
             slices = (gemm_mfma.tiled_slices_for if many else gemm_mfma.slices_for)(n, self.out_features, self.in_features)
             if slices > 1 and gemm_mfma._x_ok(x):
-                out = self.env.workspace.get((tag or self.name) + "_slices", slices * n, self.out_features,
-                                             torch.float32).view(slices, n, self.out_features)
+                out = self.env.workspace.get3((tag or self.name) + "_slices", slices, n, self.out_features, torch.float32)
                 library.profile.label = self.name
                 (gemm_mfma.tiled_slices if many else gemm_mfma.skinny_slices)(x, self.packed, out, self.out_features)
                 library.profile.label = None
                 return out
         if out is None:
             out = self.env.workspace.get(tag or self.name, n, self.out_features, out_dtype or x.dtype)
-        from ..ops import gemm, library
         if self.interleave_ff:
             raise RuntimeError(f"{self.name}: a weight packed for GeGLU only serves forward_geglu")
         library.profile.label = self.name
@@ -84,17 +80,14 @@ class Linear:
         ``n`` tokens in ``splits`` splits (the kernel library has the last word on the sizes)."""
         if self.packed is None or self.interleave_ff or self.in_features != n_heads * head_dim:
             return False
-        from ..ops import gemm_mfma
         return gemm_mfma.partials_runs(n, n_heads, head_dim, splits) > 0
 
     def forward_partials(self, part_o: torch.Tensor, part_ml: torch.Tensor, tag: Optional[str] = None) -> torch.Tensor:
         """The product of the attention rows that the splits' partial results stand for: they are
         merged inside the product's kernel.  Returns float32 slices [runs, n, out] that add up."""
-        from ..ops import gemm_mfma, library
         n, nh, splits, hd = part_o.shape
         runs = gemm_mfma.partials_runs(n, nh, hd, splits)
-        out = self.env.workspace.get((tag or self.name) + "_runs", runs * n, self.out_features,
-                                     torch.float32).view(runs, n, self.out_features)
+        out = self.env.workspace.get3((tag or self.name) + "_runs", runs, n, self.out_features, torch.float32)
         library.profile.label = self.name
         gemm_mfma.product_of_partials(part_o, part_ml, self.packed, out, self.out_features)
         library.profile.label = None
@@ -104,7 +97,6 @@ class Linear:
         """out = gelu_tanh(gate x) * (up x) in one kernel, if the weight was packed for it."""
         if not self.interleave_ff:
             return False
-        from ..ops import gemm_mfma, library
         library.profile.label = self.name
         gemm_mfma.product(x, self.packed, out, self.interleave_ff, epilogue=1)
         library.profile.label = None

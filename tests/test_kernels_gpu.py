@@ -800,7 +800,12 @@ def test_gemm_tiled(G, m, n, k, out_dtype):
     (1024, 2560, 10240, 3),     # a shorter prompt: 80 tiles of 128 x 256 in three slices
     (768, 2560, 10240, 4),      # 60 tiles in four
     (1024, 2560, 2048, 1),      # 80 tiles, but too few columns for a slice
-    (300, 200, 4096, 1)])       # next to no tiles: one product
+    (300, 200, 4096, 8),        # next to no tiles of 64 x 128 (12): as many slices of those as leave eight stages each
+    (256, 2560, 10240, 3),      # a short prompt: 80 tiles of 64 x 128 in three slices, one round of workgroups
+    (384, 2560, 10240, 2),      # 120 tiles in two
+    (130, 2560, 2048, 3),       # few columns: the slices keep six stages each (32 stages: five slices; 80 tiles: three)
+    (100, 2560, 2048, 5),       # 40 tiles of 32 stages: five slices
+    (200, 640, 320, 1)])        # five stages in all: one product
 def test_gemm_tiled_in_slices(G, m, n, k, slices):
     """A product of many tokens whose tiles fill the compute units badly comes as 32-bit slices
     that add up to it, for a reader that adds them."""
@@ -818,6 +823,24 @@ def test_gemm_tiled_in_slices(G, m, n, k, slices):
     got = out.double().sum(0)
     assert float((got - ref).abs().max()) <= 2e-5 * float(ref.abs().max()) * math.sqrt(k / 64)
     assert float(out[0].abs().max()) > 0 and float(out[z - 1].abs().max()) > 0
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("m,n,k,z", [(300, 520, 1024, 1), (70, 200, 4096, 5), (513, 1000, 1544, 3), (256, 2560, 2048, 8)])
+def test_gemm_tiled_every_tile_shape_in_slices(G, tile, m, n, k, z):
+    """Each tile shape alone (256 x 256, 128 x 256, 128 x 128, 64 x 128), as one product and in
+    slices, whatever the library's own choice for these sizes would be."""
+    g = torch.Generator().manual_seed(m + n + k + tile)
+    x = torch.randn(m, k, generator=g).bfloat16()
+    w = (torch.randn(n, k, generator=g) * 0.1).bfloat16()
+    packed = G.pack_weight(w.to(DEV))
+    ref = x.double() @ w.double().T
+    out = torch.full((z, m, n), float("nan"), dtype=torch.float32, device=DEV)
+    G.tiled_slices_as(x.to(DEV), packed, out, n, tile)
+    assert float((out.double().sum(0).cpu() - ref).abs().max()) <= 2e-5 * float(ref.abs().max()) * math.sqrt(k / 64)
+    whole = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    G.tiled_as(x.to(DEV), packed, whole, n, tile)
+    assert float((whole.double().cpu() - ref).abs().max()) <= 6e-3 * float(ref.abs().max())
 
 
 @pytest.mark.parametrize("m,ff,k", [(70, 192, 64), (513, 1000, 96), (256, 20, 40), (1024, 5120, 1000), (2048, 10236, 64),
