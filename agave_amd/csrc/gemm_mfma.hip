@@ -1135,6 +1135,10 @@ static int cut_tiled_slices(int M, int N, int K) {
     // or 240 compute units): only with long runs of columns a slice (down, not o, whose 2,048
     // columns in two slices were no faster)
     const int min_stages = t >= 160 ? 16 : 32;
+    // (4,096 columns in two slices of 128 x 256 tiles lose to the one product at 256 and 384 tokens:
+    // 3,840 rows 29.8 us against 26.1, 5,376 rows 30.4 and 32.0 against 27.2 and 27.6; the fewer
+    // compute units a product keeps busy, the faster each of them runs)
+    if (t < 160 && K < 8192) return 1;
     auto rounds = [](long g) { return (double)((g + 255) / 256); };
     const double slice_cost = 0.07 * (10240.0 / K) * ((double)t / 160.0);
     const int n_stage = (K + 63) / 64;

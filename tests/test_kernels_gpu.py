@@ -805,6 +805,8 @@ def test_gemm_tiled(G, m, n, k, out_dtype):
     (384, 2560, 10240, 2),      # 120 tiles in two
     (130, 2560, 2048, 3),       # few columns: the slices keep six stages each (32 stages: five slices; 80 tiles: three)
     (100, 2560, 2048, 5),       # 40 tiles of 32 stages: five slices
+    (256, 3840, 4096, 2),       # 120 tiles of 64 x 128 in two slices
+    (384, 3840, 4096, 1),       # more tokens: 4,096 columns in slices of 128 x 256 tiles lose to the one product
     (200, 640, 320, 1)])        # five stages in all: one product
 def test_gemm_tiled_in_slices(G, m, n, k, slices):
     """A product of many tokens whose tiles fill the compute units badly comes as 32-bit slices
