@@ -324,32 +324,54 @@ def test_a_folder_that_holds_more_than_the_decoder(tmp_path, dtype, prefix):
     close(dtype)(U.run_tail(eng, toks, 20), ref, "wrapped folder, tail")
 
 
-@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "float32"), ("B", "bfloat16")])
+def _fast_head_config(head_dim, n_heads, n_kv, window, pattern):
+    """A narrow model whose heads take the kernels for head sizes 64, 128 and 256."""
+    cfg = dict(P.tiny_config("A"), vocab_size=640, hidden_size=128, num_hidden_layers=3, num_attention_heads=n_heads,
+               num_key_value_heads=n_kv, head_dim=head_dim, query_pre_attn_scalar=head_dim, intermediate_size=320,
+               sliding_window=window, sliding_window_pattern=pattern, rope_theta=1e6, rope_local_base_freq=1e4,
+               rope_scaling={"rope_type": "linear", "factor": 4.0}, rms_norm_eps=1e-6, max_position_embeddings=4096)
+    cfg.pop("layer_types", None)
+    return cfg
+
+
+@pytest.mark.parametrize("which,dtype", [("A", "float32"), ("C", "float32"), ("B", "bfloat16"),
+                                         ("heads of 64 in groups of 4", "bfloat16"), ("heads of 256", "bfloat16"),
+                                         ("heads of 128", "float32")])
 def test_random_schedules_of_ragged_steps(tmp_path, which, dtype):
-    """Forty steps whose make-up is drawn at random: some sequences bring many tokens and others one
-    in the same step, sequences start and end at any time, slots and pages are used again, and pieces
-    end anywhere relative to page edges and the window.  Every logit row is checked."""
+    """Steps whose make-up is drawn at random: some sequences bring many tokens and others one in
+    the same step, sequences start and end at any time, slots and pages are used again, and pieces
+    end anywhere relative to page edges and the window.  Every logit row is checked.  The tiny
+    configurations run forty steps of up to four sequences of up to 190 tokens; the ones with
+    heads of 64, 128 and 256 (the kernels that the published sizes take: prompts by items, decode
+    steps with the keys shared among workgroups, the output product that merges their shares)
+    sixty steps of up to six sequences of up to 600 tokens, half of them decode steps."""
     import random
     from agave_amd.engine import Engine
-    cfg = P.tiny_config(which)
-    weights = P.random_weights(cfg, 3)
+    fast = {"heads of 64 in groups of 4": (64, 8, 2, 64, 2), "heads of 256": (256, 2, 1, 130, 3),
+            "heads of 128": (128, 4, 2, 100, 2)}.get(which)
+    cfg = _fast_head_config(*fast) if fast else P.tiny_config(which)
+    weights = {k: v.double() for k, v in P.random_weights(cfg, 3).items()}
     folder = U.write_model(str(tmp_path / "m"), cfg, weights)
-    eng = Engine.from_folder(folder, dtype=dtype, max_slots=4, max_context=200)
+    most, context, lengths, pieces, steps = (6, 640, [1, 2, 63, 64, 65, 100, 130, 190, 257, 400, 600],
+                                             [1, 3, 31, 64, 70, 129, 300], 60) if fast else \
+                                            (4, 200, [1, 2, 63, 64, 65, 100, 130, 190], [1, 3, 31, 64, 70], 40)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=most, max_context=context)
     rnd = random.Random(17)
     live = {}                       # slot -> [tokens, reference logits, fed so far]
     started = 0
-    for it in range(40):
-        while len(live) < 4 and (started < 3 or rnd.random() < 0.5):
-            n = rnd.choice([1, 2, 63, 64, 65, 100, 130, 190])
+    for it in range(steps):
+        while len(live) < most and (started < 3 or not live or rnd.random() < 0.5):
+            n = rnd.choice(lengths)
             toks = U.random_tokens(n, cfg["vocab_size"], 1000 + started)
             live[eng.alloc_slot()] = [toks, U.plain_logits(cfg, weights, toks), 0]
             started += 1
         chosen = [s for s in live if rnd.random() < 0.8] or list(live)[:1]
+        decode_only = bool(fast) and rnd.random() < 0.5
         chunks = []
         for s in chosen:
             toks, _, fed = live[s]
             room = len(toks) - fed
-            k = 1 if rnd.random() < 0.4 else rnd.choice([1, 3, 31, 64, 70])
+            k = 1 if (decode_only or rnd.random() < 0.4) else rnd.choice(pieces)
             chunks.append(toks[fed:fed + min(k, room)])
         logits = eng.step(chosen, chunks, "all").float().cpu()
         o = 0
