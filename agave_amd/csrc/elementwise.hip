@@ -429,33 +429,54 @@ __device__ __forceinline__ float gelu_tanh(float x) {
     return 0.5f * x * (1.0f + tanhf(c * (x + 0.044715f * x * x * x)));
 }
 
+// The gate's activation, by number (the feed-forward part knows the names): 0 gelu, tanh form;
+// 1 silu, x / (1 + exp(-x)); 2 gelu with the error function; 3 relu.  Another one is another case
+// here; only the tanh form also ends the matrix-core products (gemm_mfma.hip).
+#define AGAVE_GATE_ACTS 4
+__device__ __forceinline__ float gate_act(float x, int act) {
+    switch (act) {
+        case 0: return gelu_tanh(x);
+        case 1: return x / (1.0f + expf(-x));
+        case 2: return 0.5f * x * (1.0f + erff(x * 0.7071067811865476f));
+        default: return x > 0.f ? x : 0.f;
+    }
+}
+
 template <typename T>
-__global__ void geglu_kernel(const T* __restrict__ gate, long ldg, const T* __restrict__ up, long ldu,
-                             T* __restrict__ out, long ldo, long total, int ff) {
+__global__ void gated_act_kernel(const T* __restrict__ gate, long ldg, const T* __restrict__ up, long ldu,
+                                 T* __restrict__ out, long ldo, long total, int ff, int act) {
     for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
         const long r = idx / ff;
         const int c = (int)(idx % ff);
         const float g = ld(gate + r * ldg + c), u = ld(up + r * ldu + c);
-        st(out + r * ldo + c, gelu_tanh(g) * u);
+        st(out + r * ldo + c, gate_act(g, act) * u);
     }
 }
 
-extern "C" int agave_geglu(int dtype, const void* gate, long ldg, const void* up, long ldu, void* out, long ldo,
-                           int n_rows, int ff, hipStream_t stream) {
-    AGAVE_CHECK(n_rows >= 0 && ff > 0, "geglu: bad sizes rows=%d ff=%d", n_rows, ff);
-    AGAVE_CHECK(ldg >= ff && ldu >= ff && ldo >= ff, "geglu: a row stride is below %d", ff);
+// out = act(gate) * up, row by row
+extern "C" int agave_gated_act(int dtype, int act, const void* gate, long ldg, const void* up, long ldu, void* out,
+                               long ldo, int n_rows, int ff, hipStream_t stream) {
+    AGAVE_CHECK(n_rows >= 0 && ff > 0, "gated_act: bad sizes rows=%d ff=%d", n_rows, ff);
+    AGAVE_CHECK(act >= 0 && act < AGAVE_GATE_ACTS, "gated_act: unknown activation %d", act);
+    AGAVE_CHECK(ldg >= ff && ldu >= ff && ldo >= ff, "gated_act: a row stride is below %d", ff);
     if (n_rows == 0) return 0;
     const long total = (long)n_rows * ff;
     long blocks = (total + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     if (dtype == AGAVE_F32)
-        geglu_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)gate, ldg, (const float*)up, ldu, (float*)out, ldo, total, ff);
+        gated_act_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)gate, ldg, (const float*)up, ldu, (float*)out, ldo, total, ff, act);
     else if (dtype == AGAVE_BF16)
-        geglu_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)gate, ldg, (const bf16*)up, ldu, (bf16*)out, ldo, total, ff);
+        gated_act_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((const bf16*)gate, ldg, (const bf16*)up, ldu, (bf16*)out, ldo, total, ff, act);
     else
-        AGAVE_CHECK(false, "geglu: unknown dtype %d", dtype);
-    AGAVE_LAUNCH_CHECK("geglu");
+        AGAVE_CHECK(false, "gated_act: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("gated_act");
     return 0;
+}
+
+// (the tanh form of gelu under its older name)
+extern "C" int agave_geglu(int dtype, const void* gate, long ldg, const void* up, long ldu, void* out, long ldo,
+                           int n_rows, int ff, hipStream_t stream) {
+    return agave_gated_act(dtype, 0, gate, ldg, up, ldu, out, ldo, n_rows, ff, stream);
 }
 
 // ------------------------------------------------------------------ rows of the residual stream, as they are

@@ -25,6 +25,7 @@ _SIGNATURES = {
         "agave_qk_norm_rope_kv": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F,
                                   _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
+        "agave_gated_act": [_I, _I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
         "agave_cast": [_I, _P, _I, _P, _L, _P],
         "agave_gather_rows": [_I, _P, _P, _P, _L, _I, _I, _P],
     },
@@ -228,14 +229,28 @@ def _check_table(table: torch.Tensor, base: torch.Tensor, tok_seq: Optional[torc
     return table.shape[1]
 
 
-def geglu(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor) -> None:
-    """out = gelu_tanh(gate) * up, row by row."""
+# The activations of a gated feed-forward that the elementwise kernel knows, by the number it knows them by.
+GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1, "gelu": 2, "relu": 3}
+
+
+def gated_act(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, activation: str = "gelu_tanh") -> None:
+    """out = act(gate) * up, row by row; ``activation`` is one of ``GATE_ACTIVATIONS``."""
     _dev(gate, up, out)
+    try:
+        act = GATE_ACTIVATIONS[activation]
+    except KeyError:
+        raise ValueError(f"gated_act: unknown activation {activation!r}; known: {sorted(GATE_ACTIVATIONS)}") from None
     ldg, ldu, ldo = _rows(gate, "gate"), _rows(up, "up"), _rows(out, "out")
     if gate.shape != up.shape or gate.shape != out.shape or not (gate.dtype == up.dtype == out.dtype):
-        raise ValueError("geglu: gate, up and out must agree in shape and dtype")
+        raise ValueError("gated_act: gate, up and out must agree in shape and dtype")
     n, ff = gate.shape
-    library.call(lib("elementwise"), "agave_geglu", dt(gate), ptr(gate), ldg, ptr(up), ldu, ptr(out), ldo, n, ff, stream())
+    library.call(lib("elementwise"), "agave_gated_act", dt(gate), act, ptr(gate), ldg, ptr(up), ldu, ptr(out), ldo, n, ff,
+                 stream())
+
+
+def geglu(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor) -> None:
+    """out = gelu_tanh(gate) * up, row by row."""
+    gated_act(gate, up, out, "gelu_tanh")
 
 
 def gather_rows(h: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor) -> None:

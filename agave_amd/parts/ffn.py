@@ -3,6 +3,11 @@
 Reference: ``src/models/gemma3.zig:830-880`` (gate and up products, ``geluMul``, down
 product); the activation is the tanh form of GELU
 (``src/backend/kernels/cpu/activation.zig:69-113``).  Gate and up are one stacked product.
+
+The activation is the spec's (``GatedFfnSpec.activation``, one of
+``agave_amd.ops.kernels.GATE_ACTIVATIONS``).  With the tanh form of GELU and weights on the matrix
+cores the product ends in the activation itself; with any other the stacked product is followed
+by the elementwise kernel, which takes the activation as a parameter.
 """
 from __future__ import annotations
 
@@ -16,18 +21,20 @@ from ..weights.loader import TensorNeed
 from .base import BuildEnv, register
 from .linear import Linear
 
-_ACTIVATIONS = ("gelu_tanh",)
+FUSED_ACTIVATION = "gelu_tanh"          # the one that the matrix-core products end in
 
 
 class GatedFfn:
     def __init__(self, spec: GatedFfnSpec, weights, env: BuildEnv):
-        if spec.activation not in _ACTIVATIONS:
-            raise ValueError(f"gated feed-forward: unsupported activation {spec.activation!r}; known: {_ACTIVATIONS}")
+        if spec.activation not in kernels.GATE_ACTIVATIONS:
+            raise ValueError(f"gated feed-forward: unsupported activation {spec.activation!r}; "
+                             f"known: {sorted(kernels.GATE_ACTIVATIONS)}")
         self.spec = spec
         self.env = env
-        # [gate; up] stacked; on the matrix cores their rows are interleaved so that the product ends in GeGLU
+        # [gate; up] stacked; on the matrix cores their rows are interleaved so that the product ends in
+        # GeGLU (the tanh form only: another activation takes the plain stack and the elementwise kernel)
         self.gate_up = Linear([weights.get(spec.gate_proj), weights.get(spec.up_proj)], env, "gate_up",
-                              interleave_ff=spec.intermediate)
+                              interleave_ff=spec.intermediate if spec.activation == FUSED_ACTIVATION else 0)
         self.down = Linear([weights.get(spec.down_proj)], env, "ffn_down")
 
     @staticmethod
@@ -42,7 +49,7 @@ class GatedFfn:
         act = self.env.workspace.get("ffn_act", n, ff, x.dtype)
         if not self.gate_up.forward_geglu(x, act):
             gu = self.gate_up.forward(x, tag="gate_up")
-            kernels.geglu(gu[:, :ff], gu[:, ff:], act)
+            kernels.gated_act(gu[:, :ff], gu[:, ff:], act, self.spec.activation)
         return self.down.forward(act, tag="ffn_down", slices_ok=True)    # the block adds it to the residual stream
 
 

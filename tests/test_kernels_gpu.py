@@ -171,6 +171,25 @@ def test_geglu(K, dtype):
     assert torch.isfinite(o).all() and float(o[0, 1]) == 100.0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("activation", ["gelu_tanh", "silu", "gelu", "relu"])
+def test_gated_act_takes_the_activation_as_a_parameter(K, dtype, activation):
+    """out = act(gate) * up for every activation the kernel knows, against the library's functions
+    in 64-bit; large arguments of either sign stay finite."""
+    n, ff = 7, 301
+    gu = (torch.randn(n, 2 * ff, generator=torch.Generator().manual_seed(5)) * 3).to(dtype)
+    gu[0, :4] = torch.tensor([-90.0, 90.0, -30.0, 30.0]).to(dtype)
+    out = torch.full((n, ff), float("nan"), dtype=dtype, device=DEV)
+    K.gated_act(gu[:, :ff].to(DEV), gu[:, ff:].to(DEV), out, activation)
+    g, u = gu[:, :ff].double(), gu[:, ff:].double()
+    act = {"gelu_tanh": P.gelu_tanh, "silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu,
+           "relu": torch.relu}[activation]
+    assert torch.isfinite(out.float()).all()
+    assert torch.allclose(out.cpu().double(), act(g) * u, **_tol(dtype))
+    with pytest.raises(ValueError, match="unknown activation"):
+        K.gated_act(gu[:, :ff].to(DEV), gu[:, ff:].to(DEV), out, "swish_of_tomorrow")
+
+
 @pytest.mark.parametrize("n", [128, 1152, 6912])
 def test_gelu_golden(K, n):
     x, want = _g(f"gelu_n{n}_x"), _g(f"gelu_n{n}_out")

@@ -233,6 +233,31 @@ def test_gated_ffn_part(dtype, hidden, inter, rows):
     check(y, P.geglu(x, t["f.g"], t["f.u"], t["f.d"]), dtype, "feed-forward")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("activation", ["silu", "gelu", "relu"])
+@pytest.mark.parametrize("rows", [6, 150])
+def test_gated_ffn_part_with_another_activation(dtype, activation, rows):
+    """The activation is the spec's: with another one than the tanh form of GELU the stacked
+    gate/up product keeps its rows in order and the elementwise kernel applies the activation,
+    for a handful of tokens (skinny product) and for a prompt's worth (tiled product)."""
+    from agave_amd.config.spec import GatedFfnSpec
+    from agave_amd.parts import GatedFfn
+    hidden, inter = 96, 200
+    spec = GatedFfnSpec(kind="gated_dense", hidden=hidden, intermediate=inter, activation=activation,
+                        gate_proj="f.g", up_proj="f.u", down_proj="f.d")
+    t = {"f.g": rnd((inter, hidden), 70, 0.1), "f.u": rnd((inter, hidden), 71, 0.1), "f.d": rnd((hidden, inter), 72, 0.1)}
+    b = Bench(dtype)
+    part = GatedFfn(spec, weights_of(t, GatedFfn.tensor_needs(spec), dtype), b.env)
+    assert not part.gate_up.interleave_ff
+    x = rnd((rows, hidden), 73, 2.0)
+    y = part.forward(x.to(b.dtype).to(DEV), None)
+    y = y.sum(0) if y.dim() == 3 else y
+    act = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "relu": torch.relu}[activation]
+    xd = x.to(b.dtype).double()
+    ref = (act(xd @ t["f.g"].double().T) * (xd @ t["f.u"].double().T)) @ t["f.d"].double().T
+    check(y, ref, dtype, f"feed-forward with {activation}")
+
+
 def test_gated_ffn_at_a_prompts_length_comes_in_slices_that_the_residual_kernel_adds():
     """The benchmark model's feed-forward at 2,048 tokens: the down product's tiles would leave
     many compute units idle, so it comes as 32-bit slices; summed, and added to the residual
