@@ -37,6 +37,11 @@ class Attention:
         self.q_norm = lookup("norm", spec.q_norm.kind)(spec.q_norm, weights, env) if spec.q_norm else None
         self.k_norm = lookup("norm", spec.k_norm.kind)(spec.k_norm, weights, env) if spec.k_norm else None
         self.position = lookup("position", spec.position.kind)(spec.position, env)
+        # the per-head norms are computed inside the q/k kernel, which knows the RMS kind (a gain and an eps)
+        for name, part in (("q_norm", self.q_norm), ("k_norm", self.k_norm)):
+            if part is not None and not (hasattr(part, "gain") and hasattr(part, "eps")):
+                raise ValueError(f"attention: {name} of kind {getattr(spec, name).kind!r} has no gain and eps; the q/k "
+                                 f"kernel computes the per-head norm itself and takes those of an RMS norm")
 
     @staticmethod
     def tensor_needs(spec: AttentionSpec) -> List[TensorNeed]:

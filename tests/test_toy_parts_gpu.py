@@ -449,3 +449,22 @@ def test_a_norm_of_another_form_and_a_model_without_a_final_norm(tmp_path, dtype
     reqs = [U.random_tokens(n, VOCAB, 20 + i) for i, n in enumerate((40, 9, 70))]
     for i, (r, o) in enumerate(zip(reqs, U.run_batched(eng, reqs, (30, 9, 2)))):
         close(o, plain_centred_norm_model(w, r, final), dtype, f"request {i} of a batch")
+
+
+def test_a_head_norm_that_the_q_k_kernel_cannot_compute_is_refused_by_name():
+    """The per-head norm of queries and keys is computed inside the q/k kernel, which knows the
+    RMS kind (a gain and an eps): a norm part of another form in that place is refused when the
+    mixer is built, with a message that names it, instead of failing at the first step."""
+    from agave_amd.config.spec import AttentionSpec, NormSpec, PositionSpec
+    from agave_amd.parts import BuildEnv, Workspace, lookup
+    from agave_amd.weights.loader import DictWeightSource
+    define_centred_norm_model()
+    spec = AttentionSpec(kind="attention", hidden=HIDDEN, n_heads=HEADS, n_kv_heads=KV, head_dim=HD, scale=0.25,
+                         window=None, position=PositionSpec("rope", HD, THETA, 1.0),
+                         q_norm=NormSpec("toy_centred", HD, EPS, "qn"), k_norm=NormSpec("rmsnorm", HD, EPS, "kn"),
+                         q_proj="q", k_proj="k", v_proj="v", o_proj="o")
+    cls = lookup("mixer", "attention")
+    w = {n.name: torch.zeros(n.shape) for n in cls.tensor_needs(spec)}
+    env = BuildEnv(torch.float32, torch.device("cuda:0"), Workspace(torch.device("cuda:0")))
+    with pytest.raises(ValueError, match="q_norm of kind 'toy_centred'"):
+        cls(spec, DictWeightSource(w, cls.tensor_needs(spec)), env)
