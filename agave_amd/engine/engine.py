@@ -24,7 +24,7 @@ from ..config import find_architecture, read_config_json
 from ..config.spec import ModelSpec
 from ..parts import BuildEnv, Workspace
 from ..weights import Checkpoint, DictWeightSource, RandomWeightSource, WeightSource
-from .graphs import DecodeGraphs, span_bucket
+from .graphs import PROMPT_GRAPH_PAD, PROMPT_GRAPH_TOKENS, DecodeGraphs, span_bucket
 from .model import Model, tensor_needs
 from .step import Step, StepPlanner, Want, resolve_want, split_pieces
 
@@ -114,6 +114,11 @@ class Engine:
         self.prefill_chunk = 0          # > 0: prompts enter in pieces of at most this many tokens (at most max_piece)
         self.use_graphs = os.environ.get("AGAVE_AMD_NO_GRAPHS", "") not in ("1", "true", "yes")
         self.graphs = DecodeGraphs(self)
+        # prompts are recorded only if every mixer and feed-forward says that its multi-token steps can be
+        # (no host-side work that depends on the tokens, nothing that waits for the GPU)
+        self._prompt_graphs_ok = all(getattr(b.mixer, "prompt_steps_can_be_recorded", False) and
+                                     (b.ffn is None or getattr(b.ffn, "prompt_steps_can_be_recorded", False))
+                                     for b in self.model.blocks)
         self._decode_widths = [g.table_width(self.max_context, 1) for g in self.cache.groups]
 
     # ------------------------------------------------------------------ construction
@@ -238,14 +243,21 @@ class Engine:
 
     def _run_one(self, slots, tokens, want, carry=None, floats=None):
         """Plan, run and commit one step of the model; (logits, step)."""
+        # a short prompt of one sequence that wants its last row: padded to a few rows' multiple, so that it
+        # can be replayed as a graph (the host needs longer to launch such a step than the GPU to run it)
+        as_prompt_graph = (self.use_graphs and self._prompt_graphs_ok and carry is None and len(slots) == 1
+                           and len(tokens) == 1 and 2 <= len(tokens[0]) <= PROMPT_GRAPH_TOKENS
+                           and isinstance(want, str) and want == "last")
         step = self.planner.plan(slots, tokens, want, decode_widths=self._decode_widths if self.use_graphs else None,
-                                 carry=carry, floats=floats)
+                                 carry=carry, floats=floats, pad_to=PROMPT_GRAPH_PAD if as_prompt_graph else 0)
         if carry is not None:
             from ..ops import sampling as sample_ops
             sample_ops.gather_tokens(self._sampled_all(), step.carry_dev, step.tokens)
         if self.use_graphs and step.is_decode and step.n_want == step.n_tokens:
             step.fixed_span = span_bucket(step.page_span(None))
             logits = self.graphs.run(step)
+        elif as_prompt_graph and step.n_tokens <= PROMPT_GRAPH_TOKENS:
+            logits = self.graphs.run_prompt(step)
         else:
             logits = self.model.forward(step)
         self.planner.commit(step)

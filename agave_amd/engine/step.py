@@ -39,7 +39,7 @@ class Step:
     slots: List[int]
     pos0: List[int]                 # length of each sequence before the step
     n_new: List[int]                # tokens each sequence brings
-    cu: List[int]                   # prefix sums of n_new (host)
+    cu: List[int]                   # prefix sums of the rows each sequence has in the step (host): n_new, and n_pad behind the last
     max_new: int
     max_len: int                    # longest sequence after the step
     tokens: torch.Tensor            # int32 [N] (device)
@@ -57,6 +57,7 @@ class Step:
     tables_start_at_reach: bool = False  # decode: column 0 of every table row is the first page the token reaches
     carry_dev: Optional[torch.Tensor] = None    # int32 [B]: rows of the previous step's sample that these tokens are
     floats_dev: Optional[torch.Tensor] = None   # float32 payload that travelled with the step (sampling parameters)
+    n_pad: int = 0                               # rows behind the last sequence's tokens that belong to no request (see plan)
 
     def page_span(self, window: Optional[int]) -> int:
         """Most pages any sequence's last token of this step reaches back over."""
@@ -157,12 +158,21 @@ class StepPlanner:
 
     def plan(self, slots: Sequence[int], tokens: Sequence[Sequence[int]], want: Want = "last",
              decode_widths: Optional[List[int]] = None, carry: Optional[Sequence[int]] = None,
-             floats: Optional[np.ndarray] = None) -> Step:
+             floats: Optional[np.ndarray] = None, pad_to: int = 0) -> Step:
         """``decode_widths``: table widths to use if this turns out to be a decode step (one token per
         sequence), so that all decode steps of a batch size have the same layout on the device.
         ``carry``: one index per sequence into what the previous step sampled (the tokens given
         are placeholders then); ``floats``: float32 values that travel in the same upload.  Both
-        lie behind everything else, so they do not move what a recorded graph reads."""
+        lie behind everything else, so they do not move what a recorded graph reads.
+        ``pad_to`` (a step of one sequence; a divisor of the page's length): rows are added behind
+        the sequence's tokens until it ends at a multiple of ``pad_to``, so that every step that
+        ends in the same stretch has the same shape and can be replayed as one recorded graph.
+        The added rows carry token 0 at the positions that follow and run through the model like
+        the others (``cu`` counts them, ``n_new`` and the wanted rows do not, ``n_pad`` says how
+        many they are); they belong to no request: the sequence's length stays the real one,
+        attention never looks at a later position, and the keys and values that the rows leave in
+        the unused places of the sequence's last page are
+        overwritten by the tokens that come to stand there before anything reads them."""
         if len(slots) != len(tokens) or len(slots) == 0:
             raise StepError("a step needs as many token lists as slots, and at least one")
         n_new = [len(t) for t in tokens]
@@ -175,11 +185,21 @@ class StepPlanner:
         wanted = resolve_want(want, n_new)
         pos0, plans = self.cache.plan_step(list(slots), n_new)
 
-        b, n = len(slots), int(flat.size)
+        b, n_real = len(slots), int(flat.size)
         cu = [0]
         for x in n_new:
             cu.append(cu[-1] + x)
         want_rows = [cu[i] + x for i, w in enumerate(wanted) for x in w]
+        n_pad = 0
+        if pad_to:
+            if b != 1 or PAGE % pad_to:
+                raise StepError("only a step of one sequence is padded, and only within its last page")
+            n_pad = (-(pos0[0] + n_new[0])) % pad_to
+        n = n_real + n_pad
+        rows_of = list(n_new)
+        rows_of[-1] += n_pad                 # the added rows follow the last sequence's tokens and positions
+        cu = list(cu)
+        cu[-1] += n_pad                      # to the kernels they are rows of that sequence like the others
         widths = []
         fixed = decode_widths if (decode_widths is not None and max(n_new) == 1) else self.fixed_width
         for gi, p in enumerate(plans):
@@ -203,9 +223,9 @@ class StepPlanner:
             off += count
             return span
 
-        s_tok = put(flat, n)
-        s_seq = put(np.repeat(np.arange(b, dtype=np.int32), n_new), n)
-        s_pos = put(np.concatenate([np.arange(p, p + k, dtype=np.int32) for p, k in zip(pos0, n_new)]), n)
+        s_tok = put(np.concatenate([flat, np.zeros(n_pad, dtype=np.int64)]) if n_pad else flat, n)
+        s_seq = put(np.repeat(np.arange(b, dtype=np.int32), rows_of), n)
+        s_pos = put(np.concatenate([np.arange(p, p + k, dtype=np.int32) for p, k in zip(pos0, rows_of)]), n)
         s_slots = put(np.asarray(slots, dtype=np.int32), b)
         s_pos0 = put(np.asarray(pos0, dtype=np.int32), b)
         s_cu = put(np.asarray(cu, dtype=np.int32), b + 1)
@@ -239,7 +259,7 @@ class StepPlanner:
             bases_host=[list(p.base) for p in plans], cache=self.cache,
             workspace=self.workspace, tables_start_at_reach=(max(n_new) == 1),
             carry_dev=view(s_carry) if s_carry is not None else None,
-            floats_dev=view(s_floats).view(torch.float32) if s_floats is not None else None)
+            floats_dev=view(s_floats).view(torch.float32) if s_floats is not None else None, n_pad=n_pad)
 
     def commit(self, step: Step) -> None:
         self.cache.commit_step(step.slots, step.n_new)

@@ -121,14 +121,19 @@ def prefill_by_items(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, 
     import numpy as np
     lib = kernels.lib("attention_mfma")
     hw = int(lib.agave_attn_prefill_items_hw(n_heads, n_kv))
-    waves = 8 if step.max_new > 32 else 4          # eight waves once a sequence brings enough tokens for them
+    # (the rows that pad a step to a fixed multiple are rows of its sequence like the others: every
+    # step of that shape then has the same plan, whatever its real length)
+    n_pad = getattr(step, "n_pad", 0)
+    n_rows = list(step.n_new)
+    n_rows[-1] += n_pad
+    waves = 8 if max(n_rows) > 32 else 4           # eight waves once a sequence brings enough tokens for them
     blk_len = (waves // hw) * 16
     chunks = -(-(n_heads // n_kv) // hw)
     cache = step.__dict__.setdefault("_prefill_items", {})
     key = (window, blk_len, n_kv * chunks, n_heads, head_dim)
     plan = cache.get(key)
     if plan is None:
-        items, tok_pieces, max_pieces, max_item_pages = plan_prefill_items(step.pos0, step.n_new, window, blk_len,
+        items, tok_pieces, max_pieces, max_item_pages = plan_prefill_items(step.pos0, n_rows, window, blk_len,
                                                                            n_kv * chunks, n_heads, head_dim)
         both = torch.from_numpy(np.concatenate([items.reshape(-1), tok_pieces])).to(q.device)
         plan = cache[key] = (both[:items.size].view(-1, 6), both[items.size:], max_pieces, max_item_pages)
@@ -199,7 +204,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages
         library.call(lib, "agave_attn_prefill_mfma", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
                      k_pages.data_ptr(), v_pages.data_ptr(), table.data_ptr(), width, base.data_ptr(), n_pages,
                      step.tok_seq.data_ptr(), step.tok_pos.data_ptr(), step.cu_dev.data_ptr(), step.n_seqs,
-                     step.max_new, n, n_heads, n_kv, head_dim, scale, w, kernels.stream())
+                     step.max_new + getattr(step, "n_pad", 0), n, n_heads, n_kv, head_dim, scale, w, kernels.stream())
 
 
 def decode_fused(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], out: torch.Tensor,

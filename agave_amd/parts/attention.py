@@ -23,6 +23,8 @@ from .linear import Linear
 
 
 class Attention:
+    prompt_steps_can_be_recorded = True        # a multi-token step is the same launches whatever its tokens are
+
     def __init__(self, spec: AttentionSpec, weights, env: BuildEnv):
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("query heads must be a multiple of kv heads")

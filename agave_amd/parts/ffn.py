@@ -25,6 +25,8 @@ FUSED_ACTIVATION = "gelu_tanh"          # the one that the matrix-core products 
 
 
 class GatedFfn:
+    prompt_steps_can_be_recorded = True        # a multi-token step is the same launches whatever its tokens are
+
     def __init__(self, spec: GatedFfnSpec, weights, env: BuildEnv):
         if spec.activation not in kernels.GATE_ACTIVATIONS:
             raise ValueError(f"gated feed-forward: unsupported activation {spec.activation!r}; "

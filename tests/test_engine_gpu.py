@@ -137,6 +137,54 @@ def test_graph_replays_equal_eager_steps(tiny, dtype):
     assert len(a.graphs._graphs) >= 1
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_short_prompts_of_one_sequence_are_replayed_as_graphs(tiny, dtype):
+    """A short prompt of one sequence that wants its last row is padded until it ends at a multiple
+    of 16 positions and, from its kind's second occurrence on, recorded and replayed.  Prompts of
+    different lengths that end in the same stretch share a graph: each must give what the plain
+    implementation gives for its own length, on the eager run, on the recording and on every
+    replay, and so must the tokens decoded after it (they come to stand where the padding left
+    keys and values), also when the prompt is a continuation that starts in the middle of a page."""
+    from agave_amd.engine import Engine
+    from agave_amd.engine.graphs import PROMPT_GRAPH_PAD, PROMPT_GRAPH_TOKENS
+    assert (PROMPT_GRAPH_PAD, PROMPT_GRAPH_TOKENS) == (16, 128)      # the lengths below are chosen for these
+    which, cfg, weights, folder = tiny
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=3, max_context=256)
+    v = cfg["vocab_size"]
+    seed = 300
+    # (a long one first: it sizes the workspace, and it is too long to be recorded)
+    for lengths in ((150,), (100, 112, 97, 105), (5, 16, 2, 9), (60, 64, 49), (128, 113, 120)):
+        for n in lengths:
+            seed += 1
+            toks = U.random_tokens(n + 4, v, seed)
+            ref = U.plain_logits(cfg, weights, toks)
+            slot = eng.alloc_slot()
+            got = [eng.step([slot], [toks[:n]], "last").float().cpu().clone()]
+            for t in toks[n:]:
+                got.append(eng.step([slot], [[t]], "last").float().cpu().clone())
+            eng.free_slot(slot)
+            close(dtype)(torch.cat(got, 0), ref[n - 1:], f"prompt of {n} and four tokens after it")
+    kinds = [k for k in eng.graphs._graphs if k[0] == "prompt"]
+    assert sorted(k[1] for k in kinds) == [16, 64, 112, 128], kinds
+
+    # continuations: 40 tokens, then some more that end between 81 and 96 (a step that starts at 40 and is
+    # padded to 56 rows), three times so that it is run eagerly, recorded and replayed
+    for rep, more in enumerate((50, 56, 41)):
+        toks = U.random_tokens(40 + more + 3, v, 400 + rep)
+        ref = U.plain_logits(cfg, weights, toks)
+        slot = eng.alloc_slot()
+        got = [eng.step([slot], [toks[:40]], "last").float().cpu().clone(),
+               eng.step([slot], [toks[40:40 + more]], "last").float().cpu().clone()]
+        for t in toks[40 + more:]:
+            got.append(eng.step([slot], [[t]], "last").float().cpu().clone())
+        eng.free_slot(slot)
+        want = torch.cat([ref[39:40], ref[40 + more - 1:]], 0)
+        close(dtype)(torch.cat(got, 0), want, f"40 tokens, then {more} more")
+    assert any(k[0] == "prompt" and k[1:3] == (56, 40) for k in eng.graphs._graphs)
+    for g in eng.cache.groups:
+        assert g.pool.n_free == g.pool.n_pages
+
+
 def test_long_decoding(engine_of):
     """A short prompt, then many tokens one by one: over page edges, past the window's reach (the
     window groups give pages back while the sequence grows) and through many graph replays."""

@@ -281,6 +281,7 @@ def test_toy_model_is_built_and_stepped(toy, dtype):
     assert set(eng.cache.state) == {0, 3}                       # the decay mixer's two runs, a state each
     assert sorted(eng.cache.group_of_memory) == [1, 2]          # the two attention memories; layer 3 has none
     assert len(eng.cache.groups) == 2                           # a window group and a group of all keys
+    assert not eng._prompt_graphs_ok                            # a mixer that does not say so is never recorded over a prompt
 
     toks = U.random_tokens(100, VOCAB, 1)
     ref = plain_toy(w, toks)
