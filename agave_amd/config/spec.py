@@ -53,6 +53,10 @@ class AttentionSpec(MixerSpec):
     k_proj: str = ""
     v_proj: str = ""
     o_proj: str = ""
+    q_bias: str = ""               # names of the projections' bias vectors; "": none
+    k_bias: str = ""
+    v_bias: str = ""
+    o_bias: str = ""
 
 
 @dataclass(frozen=True)
@@ -68,6 +72,9 @@ class GatedFfnSpec(FeedForwardSpec):
     gate_proj: str = ""
     up_proj: str = ""
     down_proj: str = ""
+    gate_bias: str = ""            # names of the products' bias vectors; "": none
+    up_bias: str = ""
+    down_bias: str = ""
 
 
 @dataclass(frozen=True)
@@ -116,6 +123,10 @@ class ModelSpec:
     # part asked for is an error under one of them and is passed over elsewhere (a vision
     # tower beside a text decoder).  None: every name in the checkpoint is the model's.
     tensor_scope: Optional[Tuple[str, ...]] = None
+    # what is done to the logits after the output product: multiplied by ``logit_scale``, then
+    # soft-capped to +-``logit_softcap`` (cap * tanh(x / cap)) if that is above zero
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0
     extra: Dict[str, object] = field(default_factory=dict)
 
     def default_order(self) -> List[RunEntry]:

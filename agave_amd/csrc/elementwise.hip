@@ -479,6 +479,56 @@ extern "C" int agave_geglu(int dtype, const void* gate, long ldg, const void* up
     return agave_gated_act(dtype, 0, gate, ldg, up, ldu, out, ldo, n_rows, ff, stream);
 }
 
+// ------------------------------------------------------------------ a product's bias
+// y[r][c] += bias[c], summed in 32-bit and rounded to y's element type once
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, long ldy, const float* __restrict__ bias, long total, int n_cols) {
+    for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
+        const long r = idx / n_cols;
+        const int c = (int)(idx % n_cols);
+        T* at = y + r * ldy + c;
+        st(at, ld(at) + bias[c]);
+    }
+}
+
+extern "C" int agave_add_bias(int dtype, void* y, long ldy, const float* bias, int n_rows, int n_cols, hipStream_t stream) {
+    AGAVE_CHECK(n_rows >= 0 && n_cols > 0 && ldy >= n_cols, "add_bias: bad sizes rows=%d cols=%d stride=%ld", n_rows, n_cols, ldy);
+    AGAVE_CHECK(y != nullptr && bias != nullptr, "add_bias: null tensor");
+    if (n_rows == 0) return 0;
+    const long total = (long)n_rows * n_cols;
+    long blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    if (dtype == AGAVE_F32)
+        add_bias_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)y, ldy, bias, total, n_cols);
+    else if (dtype == AGAVE_BF16)
+        add_bias_kernel<bf16><<<(int)blocks, 256, 0, stream>>>((bf16*)y, ldy, bias, total, n_cols);
+    else
+        AGAVE_CHECK(false, "add_bias: unknown dtype %d", dtype);
+    AGAVE_LAUNCH_CHECK("add_bias");
+    return 0;
+}
+
+// ------------------------------------------------------------------ logits: a factor, and a soft cap
+// x <- cap * tanh(scale * x / cap) if cap > 0, scale * x otherwise (32-bit logits, in place)
+__global__ void scale_cap_kernel(float* __restrict__ x, long n, float scale, float cap) {
+    const float inv = cap > 0.f ? 1.0f / cap : 0.f;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const float v = x[i] * scale;
+        x[i] = cap > 0.f ? cap * tanhf(v * inv) : v;
+    }
+}
+
+extern "C" int agave_scale_cap(float* x, long n, float scale, float cap, hipStream_t stream) {
+    AGAVE_CHECK(n >= 0 && cap >= 0.f, "scale_cap: bad arguments n=%ld cap=%g", n, (double)cap);
+    AGAVE_CHECK(x != nullptr || n == 0, "scale_cap: null tensor");
+    if (n == 0) return 0;
+    long blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    scale_cap_kernel<<<(int)blocks, 256, 0, stream>>>(x, n, scale, cap);
+    AGAVE_LAUNCH_CHECK("scale_cap");
+    return 0;
+}
+
 // ------------------------------------------------------------------ rows of the residual stream, as they are
 // out[i] = h[rows[i]] (rows null: h[i]) in out's element type: what a model without a final norm
 // hands to its output matrix.

@@ -105,4 +105,6 @@ class Model:
         add_pending_and_norm(h, pending, self.final_norm, x, rows=step.want_rows)   # no final norm: the rows as they are
         logits = ws.get("logits", step.n_want, self.spec.vocab_size, torch.float32)
         self.head.forward(x, out=logits)
+        if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:
+            kernels.scale_cap(logits, self.spec.logit_scale, self.spec.logit_softcap)
         return logits

@@ -27,6 +27,8 @@ _SIGNATURES = {
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
         "agave_gated_act": [_I, _I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
         "agave_cast": [_I, _P, _I, _P, _L, _P],
+        "agave_add_bias": [_I, _P, _L, _P, _I, _I, _P],
+        "agave_scale_cap": [_P, _L, _F, _F, _P],
         "agave_gather_rows": [_I, _P, _P, _P, _L, _I, _I, _P],
     },
     "gemm": {
@@ -251,6 +253,25 @@ def gated_act(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor, activatio
 def geglu(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor) -> None:
     """out = gelu_tanh(gate) * up, row by row."""
     gated_act(gate, up, out, "gelu_tanh")
+
+
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
+    """y[r] += bias for every row of y (float32 or bfloat16, rows contiguous); the bias is float32."""
+    _dev(y, bias)
+    ldy = _rows(y, "y")
+    _f32vec(bias, "bias", y.shape[1])
+    library.call(lib("elementwise"), "agave_add_bias", dt(y), ptr(y), ldy, ptr(bias), y.shape[0], y.shape[1], stream())
+
+
+def scale_cap(logits: torch.Tensor, scale: float = 1.0, cap: float = 0.0) -> None:
+    """logits <- cap * tanh(scale * logits / cap) if ``cap`` > 0, scale * logits otherwise, in place
+    (soft-capping as ``src/models/gemma4.zig:2365-2385`` states it)."""
+    _dev(logits)
+    if logits.dtype != torch.float32 or not logits.is_contiguous():
+        raise ValueError("scale_cap: logits must be a contiguous float32 tensor")
+    if cap < 0:
+        raise ValueError("scale_cap: a cap cannot be negative")
+    library.call(lib("elementwise"), "agave_scale_cap", ptr(logits), logits.numel(), float(scale), float(cap), stream())
 
 
 def gather_rows(h: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor) -> None:

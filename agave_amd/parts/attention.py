@@ -33,9 +33,13 @@ class Attention:
         self.qd = spec.n_heads * spec.head_dim
         self.kvd = spec.n_kv_heads * spec.head_dim
         self._qkv_bounds = (0, self.qd, self.qd + self.kvd, self.qd + 2 * self.kvd)
+        def bias(name):
+            return weights.get(name) if name else None
+
         # q, k and v in one product: rows of the three matrices stacked
-        self.qkv = Linear([weights.get(spec.q_proj), weights.get(spec.k_proj), weights.get(spec.v_proj)], env, "qkv")
-        self.o = Linear([weights.get(spec.o_proj)], env, "attn_o")
+        self.qkv = Linear([weights.get(spec.q_proj), weights.get(spec.k_proj), weights.get(spec.v_proj)], env, "qkv",
+                          biases=[bias(spec.q_bias), bias(spec.k_bias), bias(spec.v_bias)])
+        self.o = Linear([weights.get(spec.o_proj)], env, "attn_o", biases=[bias(spec.o_bias)])
         self.q_norm = lookup("norm", spec.q_norm.kind)(spec.q_norm, weights, env) if spec.q_norm else None
         self.k_norm = lookup("norm", spec.k_norm.kind)(spec.k_norm, weights, env) if spec.k_norm else None
         self.position = lookup("position", spec.position.kind)(spec.position, env)
@@ -50,6 +54,9 @@ class Attention:
         qd, kvd = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim
         needs = [TensorNeed(spec.q_proj, (qd, spec.hidden)), TensorNeed(spec.k_proj, (kvd, spec.hidden)),
                  TensorNeed(spec.v_proj, (kvd, spec.hidden)), TensorNeed(spec.o_proj, (spec.hidden, qd))]
+        for name, size in ((spec.q_bias, qd), (spec.k_bias, kvd), (spec.v_bias, kvd), (spec.o_bias, spec.hidden)):
+            if name:
+                needs.append(TensorNeed(name, (size,)))
         for n in (spec.q_norm, spec.k_norm):
             if n is not None:
                 needs += lookup("norm", n.kind).tensor_needs(n)

@@ -35,15 +35,26 @@ class GatedFfn:
         self.env = env
         # [gate; up] stacked; on the matrix cores their rows are interleaved so that the product ends in
         # GeGLU (the tanh form only: another activation takes the plain stack and the elementwise kernel)
+        # (nor with a bias on gate or up: the fused product has no place for one)
+        def bias(name):
+            return weights.get(name) if name else None
+
+        fused = spec.activation == FUSED_ACTIVATION and not (spec.gate_bias or spec.up_bias)
         self.gate_up = Linear([weights.get(spec.gate_proj), weights.get(spec.up_proj)], env, "gate_up",
-                              interleave_ff=spec.intermediate if spec.activation == FUSED_ACTIVATION else 0)
-        self.down = Linear([weights.get(spec.down_proj)], env, "ffn_down")
+                              interleave_ff=spec.intermediate if fused else 0,
+                              biases=[bias(spec.gate_bias), bias(spec.up_bias)])
+        self.down = Linear([weights.get(spec.down_proj)], env, "ffn_down", biases=[bias(spec.down_bias)])
 
     @staticmethod
     def tensor_needs(spec: GatedFfnSpec) -> List[TensorNeed]:
-        return [TensorNeed(spec.gate_proj, (spec.intermediate, spec.hidden)),
-                TensorNeed(spec.up_proj, (spec.intermediate, spec.hidden)),
-                TensorNeed(spec.down_proj, (spec.hidden, spec.intermediate))]
+        needs = [TensorNeed(spec.gate_proj, (spec.intermediate, spec.hidden)),
+                 TensorNeed(spec.up_proj, (spec.intermediate, spec.hidden)),
+                 TensorNeed(spec.down_proj, (spec.hidden, spec.intermediate))]
+        for name, size in ((spec.gate_bias, spec.intermediate), (spec.up_bias, spec.intermediate),
+                           (spec.down_bias, spec.hidden)):
+            if name:
+                needs.append(TensorNeed(name, (size,)))
+        return needs
 
     def forward(self, x: torch.Tensor, step) -> torch.Tensor:
         ff = self.spec.intermediate

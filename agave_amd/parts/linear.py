@@ -19,10 +19,12 @@ from .base import BuildEnv
 
 class Linear:
     def __init__(self, weights: Sequence[torch.Tensor], env: BuildEnv, name: str = "linear", pack: bool = True,
-                 interleave_ff: int = 0):
+                 interleave_ff: int = 0, biases: Optional[Sequence[Optional[torch.Tensor]]] = None):
         """``weights``: one or more [out_i, in] matrices that are stacked along ``out``.
         ``interleave_ff``: the stack is [gate; up] of that many rows each; if the weight is packed
-        its rows are interleaved for the product that ends in GeGLU (see ``forward_geglu``)."""
+        its rows are interleaved for the product that ends in GeGLU (see ``forward_geglu``).
+        ``biases``: one vector [out_i] or None per matrix; y = W x + b then (the sum is made in
+        32-bit by a kernel of its own after the product: a model without biases pays nothing)."""
         ws = []
         for w in weights:
             if w.dim() != 2:
@@ -49,6 +51,20 @@ class Linear:
         elif env.dtype == torch.bfloat16 and self.weight.dtype == torch.float32:
             env.kept_32bit.append(name)
         self.interleave_ff = interleave_ff if self.packed is not None else 0
+        self.bias: Optional[torch.Tensor] = None
+        if biases is not None and any(b is not None for b in biases):
+            if len(biases) != len(ws):
+                raise ValueError(f"{name}: {len(biases)} biases for {len(ws)} matrices")
+            if interleave_ff:
+                raise ValueError(f"{name}: a product that ends in GeGLU takes no bias")
+            pieces = []
+            for w, b in zip(ws, biases):
+                if b is None:
+                    b = torch.zeros(w.shape[0])
+                if tuple(b.shape) != (w.shape[0],):
+                    raise ValueError(f"{name}: a bias of shape {tuple(b.shape)} for a matrix of {w.shape[0]} rows")
+                pieces.append(b.to(device=env.device, dtype=torch.float32))
+            self.bias = torch.cat(pieces).contiguous()
 
     def forward(self, x: torch.Tensor, out: Optional[torch.Tensor] = None,
                 out_dtype: Optional[torch.dtype] = None, tag: Optional[str] = None,
@@ -64,6 +80,8 @@ class Linear:
                 out = self.env.workspace.get3((tag or self.name) + "_slices", slices, n, self.out_features, torch.float32)
                 library.profile.label = self.name
                 (gemm_mfma.tiled_slices if many else gemm_mfma.skinny_slices)(x, self.packed, out, self.out_features)
+                if self.bias is not None:
+                    kernels.add_bias(out[0], self.bias)
                 library.profile.label = None
                 return out
         if out is None:
@@ -72,6 +90,8 @@ class Linear:
             raise RuntimeError(f"{self.name}: a weight packed for GeGLU only serves forward_geglu")
         library.profile.label = self.name
         gemm.linear(x, self, out)
+        if self.bias is not None:
+            kernels.add_bias(out, self.bias)
         library.profile.label = None
         return out
 
@@ -90,6 +110,8 @@ class Linear:
         out = self.env.workspace.get3((tag or self.name) + "_runs", runs, n, self.out_features, torch.float32)
         library.profile.label = self.name
         gemm_mfma.product_of_partials(part_o, part_ml, self.packed, out, self.out_features)
+        if self.bias is not None:
+            kernels.add_bias(out[0], self.bias)
         library.profile.label = None
         return out
 

@@ -190,6 +190,38 @@ def test_gated_act_takes_the_activation_as_a_parameter(K, dtype, activation):
         K.gated_act(gu[:, :ff].to(DEV), gu[:, ff:].to(DEV), out, "swish_of_tomorrow")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_bias_to_rows_of_a_wider_matrix(K, dtype):
+    """y[r] += bias, summed in 32-bit and rounded once; the columns beside the rows' stretch stay."""
+    n, cols = 9, 203
+    g = torch.Generator().manual_seed(6)
+    wide = torch.randn(n, cols + 13, generator=g).to(dtype).to(DEV)
+    before = wide.clone()
+    bias = torch.randn(cols, generator=g).to(DEV)
+    K.add_bias(wide[:, 5:5 + cols], bias)
+    want = (before[:, 5:5 + cols].float() + bias).to(dtype)
+    assert torch.equal(wide[:, 5:5 + cols], want)
+    assert torch.equal(wide[:, :5], before[:, :5]) and torch.equal(wide[:, 5 + cols:], before[:, 5 + cols:])
+    with pytest.raises(TypeError):
+        K.add_bias(wide[:, 5:5 + cols], bias[:-1])
+
+
+@pytest.mark.parametrize("scale,cap", [(1.0, 30.0), (2.5, 4.0), (0.125, 0.0)])
+def test_scale_and_soft_cap_of_logits(K, scale, cap):
+    """x <- cap tanh(scale x / cap), or scale x without a cap; huge logits end at the cap, not at NaN."""
+    x = torch.randn(5, 1001, generator=torch.Generator().manual_seed(7)) * 6
+    x[0, :3] = torch.tensor([1e6, -1e6, 0.0])
+    y = x.to(DEV)
+    K.scale_cap(y, scale, cap)
+    want = x.double() * scale
+    if cap > 0:
+        want = cap * torch.tanh(want / cap)
+    assert torch.isfinite(y).all()
+    assert torch.allclose(y.cpu().double(), want, atol=2e-6 * max(cap, 1.0), rtol=2e-6)
+    with pytest.raises(ValueError):
+        K.scale_cap(y, 1.0, -1.0)
+
+
 @pytest.mark.parametrize("n", [128, 1152, 6912])
 def test_gelu_golden(K, n):
     x, want = _g(f"gelu_n{n}_x"), _g(f"gelu_n{n}_out")

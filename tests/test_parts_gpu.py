@@ -258,6 +258,57 @@ def test_gated_ffn_part_with_another_activation(dtype, activation, rows):
     check(y, ref, dtype, f"feed-forward with {activation}")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,out_f,in_f,slices_ok", [(5, 96, 200, False), (8, 2560, 10240, True), (256, 3840, 4096, True),
+                                                     (150, 130, 72, True)])
+def test_linear_with_a_bias_on_every_path(dtype, rows, out_f, in_f, slices_ok):
+    """y = W x + b with two stacked matrices of which one has a bias: as one tensor and as 32-bit
+    slices that add up (few rows of a long product, and a prompt's worth of rows), the bias
+    being added once, not once a slice."""
+    from agave_amd.parts import Linear
+    b = Bench(dtype)
+    top = out_f // 3
+    w0, w1 = rnd((top, in_f), 80, 0.05), rnd((out_f - top, in_f), 81, 0.05)
+    bias1 = rnd((out_f - top,), 82, 2.0)
+    tdt = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+    lin = Linear([w0.to(tdt), w1.to(tdt)], b.env, "biased", biases=[None, bias1.to(tdt)])
+    assert lin.bias.dtype == torch.float32 and float(lin.bias[:top].abs().max()) == 0.0
+    x = rnd((rows, in_f), 83, 1.0)
+    y = lin.forward(x.to(b.dtype).to(DEV), slices_ok=slices_ok)
+    if dtype == "bfloat16" and (rows, out_f, in_f) in ((8, 2560, 10240), (256, 3840, 4096)):
+        assert y.dim() == 3 and y.shape[0] > 1, "this shape was chosen because it comes in slices"
+    y = y.sum(0) if y.dim() == 3 else y
+    ref = x @ torch.cat([w0, w1]).T + torch.cat([torch.zeros(top, dtype=torch.float64), bias1])
+    check(y, ref, dtype, "linear with a bias")
+    with pytest.raises(ValueError, match="bias of shape"):
+        Linear([w0.to(tdt)], b.env, "wrong", biases=[bias1.to(tdt)[:top + 1]])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gated_ffn_part_with_biases(dtype):
+    """Biases on gate, up and down: the gate/up product then keeps its rows in order (the product
+    that ends in the activation has no place for a bias) and the elementwise kernel follows."""
+    from agave_amd.config.spec import GatedFfnSpec
+    from agave_amd.parts import GatedFfn
+    hidden, inter = 96, 200
+    spec = GatedFfnSpec(kind="gated_dense", hidden=hidden, intermediate=inter, activation="gelu_tanh",
+                        gate_proj="f.g", up_proj="f.u", down_proj="f.d", gate_bias="f.gb", up_bias="f.ub", down_bias="f.db")
+    t = {"f.g": rnd((inter, hidden), 70, 0.1), "f.u": rnd((inter, hidden), 71, 0.1), "f.d": rnd((hidden, inter), 72, 0.1),
+         "f.gb": rnd((inter,), 74, 1.0), "f.ub": rnd((inter,), 75, 1.0), "f.db": rnd((hidden,), 76, 1.0)}
+    b = Bench(dtype)
+    needs = GatedFfn.tensor_needs(spec)
+    assert {n.name for n in needs} == set(t)
+    part = GatedFfn(spec, weights_of(t, needs, dtype), b.env)
+    assert not part.gate_up.interleave_ff
+    for rows in (6, 150):
+        x = rnd((rows, hidden), 73, 2.0)
+        y = part.forward(x.to(b.dtype).to(DEV), None)
+        y = y.sum(0) if y.dim() == 3 else y
+        xd = x.to(b.dtype).double()
+        ref = (P.gelu_tanh(xd @ t["f.g"].T + t["f.gb"]) * (xd @ t["f.u"].T + t["f.ub"])) @ t["f.d"].T + t["f.db"]
+        check(y, ref, dtype, f"feed-forward with biases, {rows} rows")
+
+
 def test_gated_ffn_at_a_prompts_length_comes_in_slices_that_the_residual_kernel_adds():
     """The benchmark model's feed-forward at 2,048 tokens: the down product's tiles would leave
     many compute units idle, so it comes as 32-bit slices; summed, and added to the residual

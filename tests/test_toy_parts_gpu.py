@@ -469,3 +469,128 @@ def test_a_head_norm_that_the_q_k_kernel_cannot_compute_is_refused_by_name():
     env = BuildEnv(torch.float32, torch.device("cuda:0"), Workspace(torch.device("cuda:0")))
     with pytest.raises(ValueError, match="q_norm of kind 'toy_centred'"):
         cls(spec, DictWeightSource(w, cls.tensor_needs(spec)), env)
+
+
+# ---------------------------------------------------------------- biases on every product, logits scaled and capped
+BIAS_INTER, BIAS_WINDOW, LOGIT_SCALE, LOGIT_CAP = 144, 24, 3.0, 2.5
+
+
+def define_biased_model():
+    """The built-in attention and gated feed-forward with a bias on each of their products (and on
+    some only), SiLU and the tanh form of GELU as gates, and logits that are multiplied by a factor
+    and soft-capped: all of it is the specs' data, no part is defined here."""
+    from agave_amd.config import register_architecture
+    from agave_amd.config.registry import Architecture
+    from agave_amd.config.spec import AttentionSpec, GatedFfnSpec, LayerSpec, ModelSpec, NormSpec, PositionSpec, RunEntry
+
+    def rms(name):
+        return NormSpec("rmsnorm", HIDDEN, EPS, name, True)
+
+    def attention(prefix, window, biases):
+        names = {f"{p}_bias": prefix + p + "b" for p in biases}
+        return AttentionSpec(kind="attention", hidden=HIDDEN, n_heads=HEADS, n_kv_heads=KV, head_dim=HD,
+                             scale=1.0 / math.sqrt(HD), window=window, position=PositionSpec("rope", HD, THETA, 1.0),
+                             q_proj=prefix + "q", k_proj=prefix + "k", v_proj=prefix + "v", o_proj=prefix + "o", **names)
+
+    def dense(prefix, activation, biases):
+        names = {f"{p}_bias": prefix + p[0] + "b" for p in biases}
+        return GatedFfnSpec(kind="gated_dense", hidden=HIDDEN, intermediate=BIAS_INTER, activation=activation,
+                            gate_proj=prefix + "g", up_proj=prefix + "u", down_proj=prefix + "d", **names)
+
+    def spec_of(cfg, names=None):
+        layers = [
+            LayerSpec("prenorm", attention("l0.", None, ("q", "k", "v", "o")), dense("l0.", "silu", ("gate", "up", "down")),
+                      pre_mixer_norm=rms("l0.n0"), pre_ffn_norm=rms("l0.n2")),
+            LayerSpec("prenorm", attention("l1.", BIAS_WINDOW, ("v",)), dense("l1.", "gelu_tanh", ("down",)),
+                      pre_mixer_norm=rms("l1.n0"), pre_ffn_norm=rms("l1.n2")),
+            LayerSpec("prenorm", attention("l2.", None, ("q", "o")), dense("l2.", "gelu_tanh", ("up",)),
+                      pre_mixer_norm=rms("l2.n0"), pre_ffn_norm=rms("l2.n2")),
+        ]
+        return ModelSpec(architecture="ToyBiasForCausalLM", vocab_size=VOCAB, hidden=HIDDEN, embed_weight="emb",
+                         embed_scale=1.0, layers=layers, order=[RunEntry(i, i) for i in range(3)], final_norm=rms("final"),
+                         head_weight=None, max_context=cfg["max_position_embeddings"], eos_token_ids=(),
+                         logit_scale=cfg["logit_scale"], logit_softcap=cfg["logit_softcap"])
+
+    register_architecture(Architecture("ToyBiasForCausalLM", ("toy_bias",), lambda raw: dict(raw), spec_of))
+    return spec_of
+
+
+def plain_biased_model(w, tokens, scale, cap) -> torch.Tensor:
+    W = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    ang = P.rope_angles(torch.arange(T, dtype=torch.float64), HD, THETA, 1.0)
+
+    def b(name):
+        return W[name] if name in W else 0.0
+
+    def rms(x, name):
+        return P.rms_norm(x, W[name], EPS)
+
+    def attn(pre, x, window):
+        q = P.apply_rope((x @ W[pre + "q"].T + b(pre + "qb")).view(T, HEADS, HD), ang)
+        k = P.apply_rope((x @ W[pre + "k"].T + b(pre + "kb")).view(T, KV, HD), ang)
+        v = (x @ W[pre + "v"].T + b(pre + "vb")).view(T, KV, HD)
+        return P.attention_core(q, k, v, 1.0 / math.sqrt(HD), window).reshape(T, -1) @ W[pre + "o"].T + b(pre + "ob")
+
+    def ffn(pre, x, act):
+        gate, up = x @ W[pre + "g"].T + b(pre + "gb"), x @ W[pre + "u"].T + b(pre + "ub")
+        gate = gate * torch.sigmoid(gate) if act == "silu" else P.gelu_tanh(gate)
+        return (gate * up) @ W[pre + "d"].T + b(pre + "db")
+
+    h = W["emb"][torch.tensor(tokens)]
+    for pre, window, act in (("l0.", None, "silu"), ("l1.", BIAS_WINDOW, "gelu_tanh"), ("l2.", None, "gelu_tanh")):
+        h = h + attn(pre, rms(h, pre + "n0"), window)
+        h = h + ffn(pre, rms(h, pre + "n2"), act)
+    logits = rms(h, "final") @ W["emb"].T * scale
+    return cap * torch.tanh(logits / cap) if cap > 0 else logits
+
+
+@pytest.mark.parametrize("scale,cap", [(LOGIT_SCALE, LOGIT_CAP), (0.5, 0.0)])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_biases_on_the_products_and_logits_scaled_and_capped(tmp_path, dtype, scale, cap):
+    """Biases are named by the specs of the attention and of the feed-forward, the logits' factor and
+    cap by the model's: a model that has them is stated in data alone.  The biases are drawn as
+    large as the products they are added to, and the cap lies inside the logits' range, so that
+    leaving one out, or capping before scaling, moves the logits far beyond rounding."""
+    from safetensors.torch import save_file
+    from agave_amd.engine import Engine
+    from agave_amd.engine.model import tensor_needs
+    cfg = {"architectures": ["ToyBiasForCausalLM"], "model_type": "toy_bias", "max_position_embeddings": 256,
+           "logit_scale": scale, "logit_softcap": cap}
+    spec = define_biased_model()(cfg)
+    g = torch.Generator().manual_seed(12)
+    w = {}
+    for need in tensor_needs(spec):
+        std = 0.1 if len(need.shape) > 1 else (1.0 if need.name.endswith("b") else 0.3)
+        w[need.name] = (torch.randn(need.shape, generator=g) * std).bfloat16().float()
+    assert sum(1 for k in w if k.endswith("b") and k != "emb") == 4 + 3 + 1 + 1 + 2 + 1
+    folder = str(tmp_path)
+    save_file({k: v.bfloat16().contiguous() for k, v in w.items()}, os.path.join(folder, "model.safetensors"))
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    eng = Engine.from_folder(folder, dtype=dtype, max_slots=3, max_context=192)
+    toks = U.random_tokens(100, VOCAB, 3)
+    ref = plain_biased_model(w, toks, scale, cap)
+    if cap > 0:
+        assert float(ref.abs().max()) > 0.9 * cap and float((ref.abs() < 0.5 * cap).float().mean()) > 0.2, \
+            "the cap must bend some logits and leave others"
+    # (each bias matters: without it the plain model's logits move by far more than the tolerance)
+    for name in [k for k in w if k.endswith("b") and k != "emb"]:
+        without = dict(w)
+        without[name] = torch.zeros_like(w[name])
+        moved = float((plain_biased_model(without, toks, scale, cap) - ref).abs().max())
+        assert moved > 0.02 * float(ref.abs().max()), f"{name} would not be missed ({moved:.3e})"     # (the 32-bit run sees 3e-5)
+    close(U.run_whole(eng, toks), ref, dtype, "whole")
+    close(U.run_tail(eng, toks, 32), ref, dtype, "last 32 one by one")
+    reqs = [U.random_tokens(n, VOCAB, 30 + i) for i, n in enumerate((40, 9, 70))]
+    for i, (r, o) in enumerate(zip(reqs, U.run_batched(eng, reqs, (30, 9, 2)))):
+        close(o, plain_biased_model(w, r, scale, cap), dtype, f"request {i} of a batch")
+    # sampling sees the capped logits: greedy generation agrees with the plain model's own loop
+    if dtype == "float32":
+        from agave_amd.sampling import SamplingParams
+        prompt = U.random_tokens(11, VOCAB, 40)
+        res = eng.generate([prompt], SamplingParams(temperature=0.0, max_tokens=5))[0]
+        seq = list(prompt)
+        for _ in range(5):
+            seq.append(P.argmax_first(plain_biased_model(w, seq, scale, cap)[-1]))
+        assert list(res.tokens) == seq[len(prompt):]
