@@ -45,11 +45,12 @@ template <typename T>
 __global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
                                      long part_stride, const float* __restrict__ post_gain, float post_eps,
                                      T* __restrict__ out, long ldo, const float* __restrict__ pre_gain,
-                                     float pre_eps, const int* __restrict__ rows, int e) {
+                                     float pre_eps, const int* __restrict__ rows, int e, const float* __restrict__ h_src) {
     __shared__ float red[16];
     const int i = blockIdx.x;
     const int r = rows ? rows[i] : i;
     float* hr = h + (size_t)r * e;
+    const float* hs = h_src ? h_src + (size_t)r * e : hr;        // where the row is read (it is always written to h)
     float ss_h = 0.f;
     if (branch) {
         const T* br = branch + (size_t)r * ldb;
@@ -73,13 +74,14 @@ __global__ void residual_norm_kernel(float* __restrict__ h, const T* __restrict_
         }
         for (int c = threadIdx.x; c < e; c += blockDim.x) {
             const float y = post_gain ? at(c) * inv * post_gain[c] : at(c);
-            const float hv = hr[c] + y;
+            const float hv = hs[c] + y;
             hr[c] = hv;
             ss_h += hv * hv;
         }
-    } else if (out) {
+    } else if (out || h_src) {
         for (int c = threadIdx.x; c < e; c += blockDim.x) {
-            const float hv = hr[c];
+            const float hv = hs[c];
+            if (h_src) hr[c] = hv;
             ss_h += hv * hv;
         }
     }
@@ -123,11 +125,13 @@ template <typename T, int VPT, int PB>          // PB: slices asked for at a tim
 __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __restrict__ branch, long ldb, int n_parts,
                                           long part_stride, const float* __restrict__ post_gain, float post_eps,
                                           T* __restrict__ out, long ldo, const float* __restrict__ pre_gain,
-                                          float pre_eps, const int* __restrict__ rows, int e) {
+                                          float pre_eps, const int* __restrict__ rows, int e,
+                                          const float* __restrict__ h_src) {
     __shared__ float red[16];
     const int i = blockIdx.x;
     const int r = rows ? rows[i] : i;
     float* hr = h + (size_t)r * e;
+    const float* hs = h_src ? h_src + (size_t)r * e : hr;        // where the row is read (it is always written to h)
     const float4 z = float4{0.f, 0.f, 0.f, 0.f};
     float4 hv[VPT], bv[VPT], g1[VPT], g2[VPT], pv[PB][VPT];
     int col[VPT];
@@ -142,7 +146,7 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
         col[v] = in[v] ? c : 0;
         g1[v] = *reinterpret_cast<const float4*>(g1p + col[v]);
         g2[v] = *reinterpret_cast<const float4*>(g2p + col[v]);
-        hv[v] = *reinterpret_cast<const float4*>(hr + col[v]);
+        hv[v] = *reinterpret_cast<const float4*>(hs + col[v]);
         bv[v] = z;
     }
     if (branch && n_parts == 0) {
@@ -196,6 +200,10 @@ __global__ void residual_norm_fast_kernel(float* __restrict__ h, const T* __rest
             }
             if (in[v]) *reinterpret_cast<float4*>(hr + col[v]) = hv[v];
         }
+    } else if (h_src) {
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+            if (in[v]) *reinterpret_cast<float4*>(hr + col[v]) = hv[v];
     }
     if (out) {
         float ss = 0.f;
@@ -217,8 +225,9 @@ template <typename T>
 static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, int n_parts, long part_stride,
                                       const float* post_gain, float post_eps,
                                       void* out, long ldo, const float* pre_gain, float pre_eps, const int* rows,
-                                      int n_rows, int e, hipStream_t stream) {
+                                      int n_rows, int e, const float* h_src, hipStream_t stream) {
     const size_t align = sizeof(T) * 4;
+    if ((uintptr_t)h_src % 16 != 0) return false;
     if (e % 4 != 0 || e > 16384 || (branch && (ldb % 4 != 0 || (uintptr_t)branch % (n_parts ? 16 : align) != 0)) ||
         (n_parts && part_stride % 4 != 0) ||
         (out && (ldo % 4 != 0 || (uintptr_t)out % align != 0)) || (uintptr_t)h % 16 != 0 ||
@@ -240,11 +249,11 @@ static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, in
     if (n_parts > 4 && V == 1)                                                                                        \
         residual_norm_fast_kernel<T, V, 8><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts,        \
                                                                            part_stride, post_gain, post_eps, (T*)out, \
-                                                                           ldo, pre_gain, pre_eps, rows, e);          \
+                                                                           ldo, pre_gain, pre_eps, rows, e, h_src);   \
     else                                                                                                              \
     residual_norm_fast_kernel<T, V, 4><<<n_rows, threads, 0, stream>>>(h, (const T*)branch, ldb, n_parts, part_stride,  \
                                                                     post_gain, post_eps,                             \
-                                                                    (T*)out, ldo, pre_gain, pre_eps, rows, e)
+                                                                    (T*)out, ldo, pre_gain, pre_eps, rows, e, h_src)
     if (vpt <= 1) RN_FAST(1);
     else if (vpt <= 2) RN_FAST(2);
     else RN_FAST(4);
@@ -254,11 +263,15 @@ static bool launch_residual_norm_fast(float* h, const void* branch, long ldb, in
 
 // n_parts > 0: branch points at that many 32-bit slices [n_rows][ldb], part_stride elements apart,
 // whose sum is the branch (whatever dtype says, which then names out's type alone).
+// h_src: the rows are read there instead of from h (and written to h as ever): the residual stream
+// as a kernel left it that could not write it in place.
 extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long ldb, int n_parts, long part_stride,
                                    const float* post_gain, float post_eps, void* out, long ldo, const float* pre_gain,
-                                   float pre_eps, const int* rows, int n_rows, int e, hipStream_t stream) {
+                                   float pre_eps, const int* rows, int n_rows, int e, const float* h_src,
+                                   hipStream_t stream) {
     AGAVE_CHECK(n_rows >= 0 && e > 0, "residual_norm: bad sizes rows=%d e=%d", n_rows, e);
     AGAVE_CHECK(h != nullptr, "residual_norm: residual stream is null");
+    AGAVE_CHECK(!(h_src && rows), "residual_norm: rows are gathered from the residual stream itself, not from another source");
     AGAVE_CHECK(!out || pre_gain, "residual_norm: output without its gain");
     AGAVE_CHECK(!branch || ldb >= e, "residual_norm: branch row stride %ld < %d", ldb, e);
     AGAVE_CHECK(!out || ldo >= e, "residual_norm: output row stride %ld < %d", ldo, e);
@@ -267,18 +280,18 @@ extern "C" int agave_residual_norm(int dtype, float* h, const void* branch, long
     if (n_rows == 0 || (!branch && !out)) return 0;
     const int threads = e >= 2048 ? 512 : (e >= 512 ? 256 : 64);
     if (dtype == AGAVE_F32 && launch_residual_norm_fast<float>(h, branch, ldb, n_parts, part_stride, post_gain, post_eps,
-                                                              out, ldo, pre_gain, pre_eps, rows, n_rows, e, stream)) {
+                                                              out, ldo, pre_gain, pre_eps, rows, n_rows, e, h_src, stream)) {
     } else if (dtype == AGAVE_BF16 && launch_residual_norm_fast<bf16>(h, branch, ldb, n_parts, part_stride, post_gain,
                                                                      post_eps, out, ldo, pre_gain, pre_eps, rows, n_rows,
-                                                                     e, stream)) {
+                                                                     e, h_src, stream)) {
     } else if (dtype == AGAVE_F32)
         residual_norm_kernel<float><<<n_rows, threads, 0, stream>>>(h, (const float*)branch, ldb, n_parts, part_stride,
                                                                     post_gain, post_eps,
-                                                                    (float*)out, ldo, pre_gain, pre_eps, rows, e);
+                                                                    (float*)out, ldo, pre_gain, pre_eps, rows, e, h_src);
     else if (dtype == AGAVE_BF16)
         residual_norm_kernel<bf16><<<n_rows, threads, 0, stream>>>(h, (const bf16*)branch, ldb, n_parts, part_stride,
                                                                    post_gain, post_eps,
-                                                                   (bf16*)out, ldo, pre_gain, pre_eps, rows, e);
+                                                                   (bf16*)out, ldo, pre_gain, pre_eps, rows, e, h_src);
     else
         AGAVE_CHECK(false, "residual_norm: unknown dtype %d", dtype);
     AGAVE_LAUNCH_CHECK("residual_norm");

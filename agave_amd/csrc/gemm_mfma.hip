@@ -399,6 +399,295 @@ static int dispatch_skinny(const void* X, long ldx, const void* Wp, void* Y, lon
     return 0;
 }
 
+// ------------------------------------------------------------------ one token: the product makes its normalised row itself
+// A decode step of one sequence is bound by its kernels' starts and ends (some 4.6 us for the
+// norm between two products, which moves a few kilobytes).  Here the product that reads the
+// normalised row makes it: h' = h + post(branch), x = pre(h') (two RMS norms, the first one
+// optional), for one token.  Every workgroup computes all of x while its first tiles of W are on
+// their way from memory and keeps it in LDS; workgroup 0 also writes h' to `h_out`, which must not
+// be the memory that the others still read (`h_in`).
+//
+// What the row is made of is some four times its bytes, read by every workgroup: with one
+// workgroup a row block (1280 for gate and up at 4B sizes) that would be as much again as the
+// weights.  So there are at most 256 workgroups, one a compute unit, and each takes several row
+// blocks one after another: row block b, b + G, b + 2G, ... of G workgroups, so that at any moment
+// the workgroups read neighbouring tiles.  The eight waves share a row block's columns in chunks
+// of two k-steps, three chunks in flight a wave, across the row blocks' boundaries; a wave's sums
+// for a row block go to LDS when it moves on to the next, and meet there at the end.
+struct RowNorm {
+    const float* h_in;          // [K]
+    float* h_out;               // [K], or null without a branch (h' is h then)
+    const void* branch;         // [K] in bfloat16 or 32-bit, or 32-bit slices; null: none
+    int branch_f32;
+    int n_parts;                // 32-bit slices that add up to the branch (0: one tensor)
+    long part_stride;
+    const float* post_gain;     // null: the branch is added as it is
+    float post_eps;
+    const float* pre_gain;
+    float pre_eps;
+};
+#define ROW_NORM_MAX_K 6144
+#define ROW_NORM_WGS 256
+#define ROW_NORM_MAX_SEQ 16        // row blocks a workgroup takes at most (their sums wait in LDS)
+#define ROW_NORM_MAX_LDS (ROW_NORM_MAX_SEQ * 8 * 1024 + ROW_NORM_MAX_K * 2)     // the sums and the row: 140 KB of the 160
+
+// NV: pieces of four columns a thread holds of the row (512 threads: K <= 2048 NV); PB: slices of
+// the branch asked for ahead of the tiles (the others follow one after another).
+template <int EPI, int NV, int PB>
+__global__ __launch_bounds__(512) void gemm_row_normed_kernel(RowNorm nz, const uint4* __restrict__ Wp,
+                                                             bf16* __restrict__ Y, int N, int K, int KB, int NB) {
+    // (three chunks of two k-steps in flight a wave: 6 KB; with 12 or 16 KB a step of the 4B sizes
+    // was 3 to 4 % slower, with 2 KB 7 %)
+    constexpr int NW = 8, NT = NW * 64, KS = 2, S = 3;
+    extern __shared__ __attribute__((aligned(16))) unsigned char rown_smem[];
+    const int G = gridDim.x;
+    const int n_seq = (NB - (int)blockIdx.x + G - 1) / G;              // row blocks of this workgroup (at least one)
+    float* red = reinterpret_cast<float*>(rown_smem);                   // [n_seq][NW][256] sums of the waves
+    bf16* xfull = reinterpret_cast<bf16*>(red + (size_t)((NB + G - 1) / G) * NW * 256);   // [K]
+    __shared__ float rs[16];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int j = lane & 15, g = lane >> 4;
+    const int n_chunks = (KB + KS - 1) / KS;
+    const int items = n_seq * n_chunks;                                // (row block, chunk), row block by row block
+    const int n_iter = (items + NW - 1) / NW;
+
+    // everything the row is made of is asked for before the first tile of W: a wave's loads come
+    // back in the order they left, and behind the tiles the few kilobytes from the cache would
+    // wait for the tiles from memory
+    float4 n_part[PB][NV], n_h[NV], n_g1[NV], n_g2[NV];
+    uint2 n_b16[NV];
+    const bool has_branch = nz.branch != nullptr;                       // (uniform, like all of nz)
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        const int c = (v * NT + (int)threadIdx.x) * 4;
+        const int cc = c < K ? c : 0;                  // (a lane past the row's end reads its start and uses nothing of it)
+        n_h[v] = *reinterpret_cast<const float4*>(nz.h_in + cc);
+        n_g2[v] = *reinterpret_cast<const float4*>(nz.pre_gain + cc);
+        n_g1[v] = *reinterpret_cast<const float4*>((nz.post_gain != nullptr ? nz.post_gain : nz.pre_gain) + cc);
+        if (has_branch && nz.branch_f32) {
+            const float* bp = reinterpret_cast<const float*>(nz.branch) + cc;
+            const int last = nz.n_parts > 0 ? nz.n_parts - 1 : 0;
+#pragma unroll
+            for (int u = 0; u < PB; ++u)              // (a slice that is not there: the last one again, not added)
+                n_part[u][v] = *reinterpret_cast<const float4*>(bp + (size_t)(u < last ? u : last) * nz.part_stride);
+        } else if (has_branch) {
+            n_b16[v] = *reinterpret_cast<const uint2*>(reinterpret_cast<const bf16*>(nz.branch) + cc);
+        }
+    }
+
+    frag16 wreg[S][KS];
+#define RN_LOAD(ST, IT)                                                                          \
+    {                                                                                            \
+        int i_ = (IT) * NW + wave;                    /* items are dealt to the waves in turn */  \
+        i_ = i_ < items ? i_ : items - 1;             /* past the end: the last one again, not used */ \
+        const int sq_ = i_ / n_chunks, ch_ = i_ - sq_ * n_chunks;                                \
+        const int nb_ = (int)blockIdx.x + G * sq_;                                               \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                      \
+            const int kb = ch_ * KS + ks;                                                        \
+            wreg[ST][ks].u = Wp[w_tile(nb_, kb < KB ? kb : KB - 1, NB, KB) * 64 + lane];         \
+        }                                                                                        \
+    }
+#pragma unroll
+    for (int st = 0; st < S; ++st) RN_LOAD(st, st)
+
+    // the row, while the tiles travel
+    {
+        const bool writer = blockIdx.x == 0 && nz.h_out != nullptr;
+        const int n_sl = nz.n_parts > 0 ? nz.n_parts : 1;
+        float ss = 0.f;
+        float4 bsum[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int c = (v * NT + (int)threadIdx.x) * 4;
+            float4 b = float4{0.f, 0.f, 0.f, 0.f};
+            if (has_branch && c < K) {
+                if (nz.branch_f32) {
+#pragma unroll
+                    for (int u = 0; u < PB; ++u)
+                        if (u < n_sl) {
+                            b.x += n_part[u][v].x; b.y += n_part[u][v].y; b.z += n_part[u][v].z; b.w += n_part[u][v].w;
+                        }
+                    for (int p = PB; p < n_sl; ++p) {      // more slices than were asked for ahead: one after another
+                        const float4 q = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(nz.branch) + c +
+                                                                          (size_t)p * nz.part_stride);
+                        b.x += q.x; b.y += q.y; b.z += q.z; b.w += q.w;
+                    }
+                } else {
+                    const uint2 u2 = n_b16[v];
+                    b = float4{__builtin_bit_cast(float, u2.x << 16), __builtin_bit_cast(float, u2.x & 0xffff0000u),
+                               __builtin_bit_cast(float, u2.y << 16), __builtin_bit_cast(float, u2.y & 0xffff0000u)};
+                }
+            }
+            bsum[v] = b;
+            ss += b.x * b.x + b.y * b.y + b.z * b.z + b.w * b.w;
+        }
+        float inv1 = 1.0f;
+        if (has_branch && nz.post_gain != nullptr) inv1 = 1.0f / sqrtf(block_sum(ss, rs) / (float)K + nz.post_eps);
+        ss = 0.f;
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {                     // h' = h + post(branch)
+            const int c = (v * NT + (int)threadIdx.x) * 4;
+            float4 h4 = float4{0.f, 0.f, 0.f, 0.f};
+            if (c < K) {
+                h4 = n_h[v];
+                if (has_branch) {
+                    const float4 b = bsum[v];
+                    if (nz.post_gain != nullptr) {
+                        h4.x += b.x * inv1 * n_g1[v].x; h4.y += b.y * inv1 * n_g1[v].y;
+                        h4.z += b.z * inv1 * n_g1[v].z; h4.w += b.w * inv1 * n_g1[v].w;
+                    } else {
+                        h4.x += b.x; h4.y += b.y; h4.z += b.z; h4.w += b.w;
+                    }
+                    if (writer) *reinterpret_cast<float4*>(nz.h_out + c) = h4;
+                }
+            }
+            n_h[v] = h4;
+            ss += h4.x * h4.x + h4.y * h4.y + h4.z * h4.z + h4.w * h4.w;
+        }
+        // x = pre(h'), rounded to bfloat16 once, as the norm kernel rounds it
+        const float inv2 = 1.0f / sqrtf(block_sum(ss, rs) / (float)K + nz.pre_eps);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            const int c = (v * NT + (int)threadIdx.x) * 4;
+            if (c < K)
+                store4<bf16>(xfull + c, float4{n_h[v].x * inv2 * n_g2[v].x, n_h[v].y * inv2 * n_g2[v].y,
+                                              n_h[v].z * inv2 * n_g2[v].z, n_h[v].w * inv2 * n_g2[v].w});
+        }
+        // a wave that gets no chunk of some row block leaves zeros there
+        for (int i = threadIdx.x; i < n_seq * NW * 64; i += NT)
+            reinterpret_cast<f32x4_t*>(red)[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+    }
+
+    f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    int cur = -1;                                       // the row block (in this workgroup's order) that acc belongs to
+    // only lanes 0..15 of a group hold a token's column of the tile; the token is row 0: the others multiply zeros
+#define RN_USE(ST, IT)                                                                           \
+    if ((IT) * NW + wave < items) {                                                              \
+        const int i_ = (IT) * NW + wave;                                                         \
+        const int sq_ = i_ / n_chunks, ch_ = i_ - sq_ * n_chunks;                                \
+        if (sq_ != cur) {                                                                        \
+            if (cur >= 0) *reinterpret_cast<f32x4_t*>(red + ((size_t)(cur * NW + wave) * 64 + lane) * 4) = acc; \
+            acc = f32x4_t{0.f, 0.f, 0.f, 0.f};                                                   \
+            cur = sq_;                                                                           \
+        }                                                                                        \
+        _Pragma("unroll") for (int ks = 0; ks < KS; ++ks) {                                      \
+            const int k_ = (ch_ * KS + ks) * 32 + g * 8;                                         \
+            frag16 xb;                                                                           \
+            xb.u = (j == 0 && k_ < K) ? *reinterpret_cast<const uint4*>(xfull + k_) : uint4{0, 0, 0, 0}; \
+            acc = mfma_16x16x32(wreg[ST][ks], xb, acc);                                          \
+        }                                                                                        \
+    }
+    // (a load past the last item asks for the last one again and is not used: loads without a
+    // condition around them let a wait name the ones it needs and leave the younger ones in flight)
+    for (int it = 0; it < n_iter; it += S) {
+#pragma unroll
+        for (int st = 0; st < S; ++st) {
+            RN_USE(st, it + st)
+            RN_LOAD(st, it + st + S)
+        }
+    }
+#undef RN_LOAD
+#undef RN_USE
+    if (cur >= 0) *reinterpret_cast<f32x4_t*>(red + ((size_t)(cur * NW + wave) * 64 + lane) * 4) = acc;
+    __syncthreads();
+
+    // the waves' sums meet; the token's outputs are in the lanes with j == 0
+    for (int sq = wave; sq < n_seq; sq += NW) {
+        f32x4_t s = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w = 0; w < NW; ++w) s += *reinterpret_cast<const f32x4_t*>(red + ((size_t)(sq * NW + w) * 64 + lane) * 4);
+        const int nb = (int)blockIdx.x + G * sq;
+        if (j != 0 || nb >= NB) continue;
+        if (EPI == 0) {
+            const int n = nb * 16 + g * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (n + e < N) st(Y + n + e, s[e]);
+        } else {
+            const int n = nb * 8 + g * 2;                 // N counts output columns (ff)
+            if (n < N) st(Y + n, gelu_tanh_f(s[0]) * s[2]);
+            if (n + 1 < N) st(Y + n + 1, gelu_tanh_f(s[1]) * s[3]);
+        }
+    }
+}
+
+template <int EPI, int NV, int PB>
+static int launch_row_normed(const RowNorm& nz, const void* Wp, void* Y, int N, int K, int KB, int NB, int wgs, size_t lds,
+                             hipStream_t stream) {
+    static bool raised = false;                 // (once per process: the sums of many row blocks need more than the default 64 KB)
+    if (lds > 64 * 1024 && !raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_row_normed_kernel<EPI, NV, PB>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, ROW_NORM_MAX_LDS);
+        AGAVE_CHECK(e == hipSuccess, "gemm_row_normed: cannot raise the LDS allowance: %s", hipGetErrorString(e));
+        raised = true;
+    }
+    gemm_row_normed_kernel<EPI, NV, PB><<<wgs, 512, lds, stream>>>(nz, (const uint4*)Wp, (bf16*)Y, N, K, KB, NB);
+    return 0;
+}
+
+// Whether agave_gemm_row_normed takes a product of these sizes (N counts rows of W, or ff with the
+// GeGLU epilogue): one token.
+extern "C" int agave_gemm_row_normed_ok(int M, int N, int K, int epilogue) {
+    if (!(M == 1 && N > 0 && K > 0 && K % 8 == 0 && K <= ROW_NORM_MAX_K)) return 0;
+    const long NB = epilogue == 0 ? ((long)N + 15) / 16 : ((long)N + 7) / 8;
+    return NB <= (long)ROW_NORM_WGS * ROW_NORM_MAX_SEQ ? 1 : 0;
+}
+
+// Y = pre(h_in + post(branch)) W^T in bfloat16 for one token, the residual row h_in + post(branch)
+// going to h_out (see RowNorm).  branch null: Y = pre(h_in) W^T, nothing else is written.
+extern "C" int agave_gemm_row_normed(const float* h_in, float* h_out, const void* branch, int branch_f32, int n_parts,
+                                     long part_stride, const float* post_gain, float post_eps, const float* pre_gain,
+                                     float pre_eps, const void* Wp, void* Y, int N, int K, int epilogue,
+                                     hipStream_t stream) {
+    AGAVE_CHECK(epilogue == 0 || epilogue == 1, "gemm_row_normed: unknown epilogue %d", epilogue);
+    AGAVE_CHECK(agave_gemm_row_normed_ok(1, N, K, epilogue),
+                "gemm_row_normed: sizes N=%d K=%d (K <= %d, K %% 8 == 0, at most %d row blocks)", N, K, ROW_NORM_MAX_K,
+                ROW_NORM_WGS * ROW_NORM_MAX_SEQ);
+    AGAVE_CHECK(h_in != nullptr && pre_gain != nullptr && Wp != nullptr && Y != nullptr, "gemm_row_normed: null tensor");
+    AGAVE_CHECK(((uintptr_t)h_in % 16) == 0 && ((uintptr_t)pre_gain % 16) == 0 && ((uintptr_t)post_gain % 16) == 0,
+                "gemm_row_normed: the residual row and the gains must be 16-byte aligned");
+    if (branch != nullptr) {
+        AGAVE_CHECK(h_out != nullptr && h_out != h_in && ((uintptr_t)h_out % 16) == 0,
+                    "gemm_row_normed: the sum needs 16-byte aligned memory of its own (other workgroups still read h_in)");
+        AGAVE_CHECK(((uintptr_t)branch % (branch_f32 ? 16 : 8)) == 0, "gemm_row_normed: the branch must be aligned");
+        AGAVE_CHECK(n_parts >= 0 && n_parts <= 64 && (n_parts == 0 || (branch_f32 && part_stride % 4 == 0 && part_stride >= K)),
+                    "gemm_row_normed: %d slices (32-bit, a multiple of four elements apart)", n_parts);
+    }
+    const int KB = (K + 31) / 32;
+    const int NB = epilogue == 0 ? (N + 15) / 16 : (N + 7) / 8;
+    RowNorm nz;
+    nz.h_in = h_in;
+    nz.h_out = branch != nullptr ? h_out : nullptr;
+    nz.branch = branch;
+    nz.branch_f32 = branch_f32;
+    nz.n_parts = n_parts;
+    nz.part_stride = part_stride;
+    nz.post_gain = post_gain;
+    nz.post_eps = post_eps;
+    nz.pre_gain = pre_gain;
+    nz.pre_eps = pre_eps;
+    const int wgs = NB < ROW_NORM_WGS ? NB : ROW_NORM_WGS;
+    const int max_seq = (NB + wgs - 1) / wgs;
+    const size_t lds = (size_t)max_seq * 8 * 256 * sizeof(float) + (size_t)K * sizeof(bf16);
+    const bool many = branch != nullptr && branch_f32 && n_parts > 2;       // slices: eight are asked for ahead
+    int rc;
+#define RN_CASE(EPI_)                                                                                             \
+    if (K <= 4096 && !many) rc = launch_row_normed<EPI_, 2, 2>(nz, Wp, Y, N, K, KB, NB, wgs, lds, stream);          \
+    else if (K <= 4096) rc = launch_row_normed<EPI_, 2, 8>(nz, Wp, Y, N, K, KB, NB, wgs, lds, stream);              \
+    else if (!many) rc = launch_row_normed<EPI_, 3, 2>(nz, Wp, Y, N, K, KB, NB, wgs, lds, stream);                  \
+    else rc = launch_row_normed<EPI_, 3, 8>(nz, Wp, Y, N, K, KB, NB, wgs, lds, stream)
+    if (epilogue == 1) {
+        RN_CASE(1);
+    } else {
+        RN_CASE(0);
+    }
+#undef RN_CASE
+    if (rc != 0) return rc;
+    AGAVE_LAUNCH_CHECK("gemm_row_normed");
+    return 0;
+}
+
 // How many 32-bit slices a product of M <= 64 tokens is best computed in by a caller that can add
 // them up (1: as one product).
 extern "C" int agave_gemm_skinny_slices(int M, int N, int K) {

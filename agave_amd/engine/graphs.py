@@ -97,12 +97,14 @@ class DecodeGraphs:
             self._seen.pop(old, None)            # should its kind of step come back, it starts over
             self._plans.pop(old, None)
             self.evicted += 1
-        stamp = self._valid_stamp()
+        stamp, made = self._valid_stamp(), eng.workspace.allocations
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             logits = eng.model.forward(step)
-        if self._valid_stamp() != stamp:
-            # the workspace grew while recording: do not keep the graph, run the step eagerly
+        if self._valid_stamp() != stamp or eng.workspace.allocations != made:
+            # the workspace made or replaced a buffer while recording: do not keep the graph, run the
+            # step eagerly (the kind's next step is recorded with every buffer in place)
+            self._seen[key] = 1
             return eng.model.forward(step)
         self._graphs[key] = (graph, logits)
         self._stamp = stamp

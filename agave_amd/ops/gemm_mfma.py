@@ -13,6 +13,8 @@ kernels.register_signatures("gemm_mfma", {
     "agave_embed_scale_packed": [_P, _P, _F, _P, _I, _I, _I, _P],
     "agave_gemm_skinny": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _I, _P],
     "agave_gemm_skinny_slices": [_I, _I, _I],
+    "agave_gemm_row_normed_ok": [_I, _I, _I, _I],
+    "agave_gemm_row_normed": [_P, _P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _P, _I, _I, _I, _P],
     "agave_gemm_tiled_slices": [_I, _I, _I],
     "agave_gemm_tiled_in_slices": [_P, _L, _P, _P, _I, _I, _I, _I, _P],
     "agave_gemm_tiled": [_P, _L, _P, _I, _P, _L, _I, _I, _I, _I, _P, _L, _P],
@@ -57,6 +59,61 @@ def product(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int
 def skinny(x: torch.Tensor, packed: torch.Tensor, out: torch.Tensor, n_out: int, epilogue: int = 0) -> None:
     """out[M, n_out] = x[M, K] @ W^T (epilogue 0) or gelu_tanh(gate) * up (epilogue 1) for M <= 64."""
     _launch("agave_gemm_skinny", x, packed, out, n_out, epilogue)
+
+
+_normed_ok = {}
+
+
+def normed_ok(m: int, n_out: int, k: int, epilogue: int = 0) -> bool:
+    """Whether :func:`row_normed` takes a product of these sizes (the kernel library decides)."""
+    key = (m, n_out, k, epilogue)
+    got = _normed_ok.get(key)
+    if got is None:
+        got = _normed_ok[key] = bool(kernels.lib("gemm_mfma").agave_gemm_row_normed_ok(m, n_out, k, epilogue))
+    return got
+
+
+def row_normed(h_in: torch.Tensor, h_out: Optional[torch.Tensor], branch: Optional[torch.Tensor],
+                  post_gain: Optional[torch.Tensor], post_eps: float, pre_gain: torch.Tensor, pre_eps: float,
+                  packed: torch.Tensor, out: torch.Tensor, n_out: int, epilogue: int = 0) -> None:
+    """out = rmsnorm(h') * pre_gain @ W^T (or its GeGLU) with h' = h_in + post(branch), for one row:
+    the product's workgroups make the normalised row themselves, and h' goes to ``h_out``, which
+    must be other memory than ``h_in``.  ``branch``: [1, K] in bfloat16 or float32, or float32
+    slices [slices, 1, K] that add up to it, or None (then h' is h_in and nothing but ``out`` is
+    written); ``post_gain`` None: the branch is added as it is."""
+    for t in (h_in, h_out, branch, post_gain, pre_gain, packed, out):
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("agave_amd kernels run on the GPU only; got a CPU tensor")
+    if h_in.dtype != torch.float32 or h_in.dim() != 2 or not h_in.is_contiguous():
+        raise ValueError("row_normed: the residual row must be a contiguous float32 [1, K] tensor")
+    m, k = h_in.shape
+    if not normed_ok(m, n_out, k, epilogue):
+        raise ValueError(f"row_normed: no kernel for {m} rows, {n_out} outputs and {k} columns")
+    if out.dtype != torch.bfloat16 or out.dim() != 2 or out.shape != (m, n_out) or out.stride(1) != 1:
+        raise ValueError(f"row_normed: out must be bfloat16 [{m}, {n_out}] with contiguous rows")
+    if branch is not None and branch.dim() == 2 and branch.stride(0) < k:
+        raise ValueError("row_normed: the branch's row is too short")
+    nb = (n_out + 7) // 8 if epilogue else (n_out + 15) // 16
+    if packed.numel() != nb * ((k + 31) // 32) * 512:
+        raise ValueError("row_normed: the packed weight does not fit these sizes")
+    for g, what in ((pre_gain, "pre_gain"), (post_gain, "post_gain")):
+        if g is not None and (g.dtype != torch.float32 or not g.is_contiguous() or g.numel() != k):
+            raise TypeError(f"row_normed: {what} must hold {k} contiguous float32 values")
+    n_parts = part_stride = 0
+    if branch is not None:
+        if h_out is None or h_out.dtype != torch.float32 or h_out.shape != h_in.shape or not h_out.is_contiguous() \
+                or h_out.data_ptr() == h_in.data_ptr():
+            raise ValueError("row_normed: the sum needs a float32 tensor of its own, shaped like the residual row")
+        if branch.dim() == 3:
+            if branch.dtype != torch.float32 or branch.shape[1:] != (m, k) or not branch.is_contiguous():
+                raise ValueError(f"row_normed: slices must be a contiguous float32 [slices, {m}, {k}] tensor")
+            n_parts, part_stride = branch.shape[0], m * k
+        elif branch.dtype not in (torch.float32, torch.bfloat16) or branch.shape != (m, k) or branch.stride(1) != 1:
+            raise ValueError(f"row_normed: the branch must be [{m}, {k}] in float32 or bfloat16 with contiguous rows")
+    library.call(kernels.lib("gemm_mfma"), "agave_gemm_row_normed", h_in.data_ptr(), kernels.ptr(h_out), kernels.ptr(branch),
+                 1 if (branch is not None and branch.dtype == torch.float32) else 0, n_parts, part_stride,
+                 kernels.ptr(post_gain), post_eps, pre_gain.data_ptr(), pre_eps, packed.data_ptr(), out.data_ptr(),
+                 n_out, k, epilogue, kernels.stream())
 
 
 _slices = {}

@@ -21,7 +21,7 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 _SIGNATURES = {
     "elementwise": {
         "agave_embed_scale": [_I, _P, _P, _F, _P, _I, _I, _I, _P],
-        "agave_residual_norm": [_I, _P, _P, _L, _I, _L, _P, _F, _P, _L, _P, _F, _P, _I, _I, _P],
+        "agave_residual_norm": [_I, _P, _P, _L, _I, _L, _P, _F, _P, _L, _P, _F, _P, _I, _I, _P, _P],
         "agave_qk_norm_rope_kv": [_I, _P, _L, _P, _L, _P, _L, _P, _L, _P, _P, _F, _F, _P, _I, _F,
                                   _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
         "agave_geglu": [_I, _P, _L, _P, _L, _P, _L, _I, _I, _P],
@@ -130,19 +130,27 @@ def embed_scale(tokens: torch.Tensor, table: torch.Tensor, scale: float, out: to
 
 def residual_norm(h: torch.Tensor, branch: Optional[torch.Tensor], post_gain: Optional[torch.Tensor],
                   post_eps: float, out: Optional[torch.Tensor], pre_gain: Optional[torch.Tensor],
-                  pre_eps: float, rows: Optional[torch.Tensor] = None) -> None:
+                  pre_eps: float, rows: Optional[torch.Tensor] = None, src: Optional[torch.Tensor] = None) -> None:
     """If ``branch``: h += rmsnorm(branch) * post_gain.  If ``out``: out = rmsnorm(h) * pre_gain.
     ``rows`` (int32) picks the rows of ``h`` that ``out`` is computed for.  A three-dimensional
     float32 ``branch`` [slices, rows, hidden] stands for the sum of its slices (a product that was
-    shared out along its columns)."""
-    _dev(h, branch, post_gain, out, pre_gain, rows)
+    shared out along its columns).  ``src``: the residual rows are read from this tensor and
+    written to ``h`` (a kernel that could not update the stream in place left it there)."""
+    _dev(h, branch, post_gain, out, pre_gain, rows, src)
     if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
         raise ValueError("residual stream must be a contiguous float32 [rows, hidden] tensor")
     n_h, e = h.shape
     n = n_h if rows is None else rows.numel()
     _i32(rows, "rows")
+    if src is not None:
+        if src.dtype != torch.float32 or src.shape != h.shape or not src.is_contiguous() or src.data_ptr() == h.data_ptr():
+            raise ValueError("the source of the residual rows must be another contiguous float32 tensor of h's shape")
+        if rows is not None:
+            raise ValueError("rows are gathered from the residual stream itself, not from another source")
     act = branch if branch is not None else out
     if act is None:
+        if src is not None:
+            h.copy_(src)
         return
     ldb = ldo = n_parts = part_stride = 0
     if branch is not None and branch.dim() == 3:
@@ -165,7 +173,7 @@ def residual_norm(h: torch.Tensor, branch: Optional[torch.Tensor], post_gain: Op
         if branch is not None and n_parts == 0 and branch.dtype != out.dtype:
             raise TypeError("branch and out must have the same dtype")
     library.call(lib("elementwise"), "agave_residual_norm", dt(act), ptr(h), ptr(branch), ldb, n_parts, part_stride,
-                 ptr(post_gain), post_eps, ptr(out), ldo, ptr(pre_gain), pre_eps, ptr(rows), n, e, stream())
+                 ptr(post_gain), post_eps, ptr(out), ldo, ptr(pre_gain), pre_eps, ptr(rows), n, e, ptr(src), stream())
 
 
 def qk_norm_rope_kv(q: Optional[torch.Tensor], k: Optional[torch.Tensor], v: Optional[torch.Tensor],

@@ -24,6 +24,7 @@ from .linear import Linear
 
 class Attention:
     prompt_steps_can_be_recorded = True        # a multi-token step is the same launches whatever its tokens are
+    takes_rows_to_be_normed = True             # its first product may make the normalised rows itself (NormedRows)
 
     def __init__(self, spec: AttentionSpec, weights, env: BuildEnv):
         if spec.n_heads % spec.n_kv_heads:

@@ -56,14 +56,17 @@ class BuildEnv:
 
 class Workspace:
     """Named device buffers that are reused from step to step, so a step allocates nothing
-    once its sizes have been seen.  ``generation`` changes whenever a buffer had to grow,
-    which tells a captured graph that its addresses are stale."""
+    once its sizes have been seen.  ``generation`` changes whenever a buffer had to grow (the
+    smaller one it replaces is freed), which tells a captured graph that its addresses are
+    stale; a buffer under a new name moves nothing and leaves the graphs alone.  ``allocations``
+    counts both: nothing may be allocated while a graph is being recorded."""
 
     def __init__(self, device: torch.device):
         self.device = device
         self._buffers: Dict[tuple, torch.Tensor] = {}
         self._views: Dict[tuple, torch.Tensor] = {}        # (name, cols, dtype, rows) -> the first rows of the buffer
         self.generation = 0
+        self.allocations = 0
 
     def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
         # (a step asks for a few hundred buffers: the views are kept, one dictionary lookup each)
@@ -77,10 +80,11 @@ class Workspace:
             cap = max(rows, 1)
             if buf is not None:
                 cap = max(cap, buf.shape[0] * 2)
+                self.generation += 1
+                self._views.clear()                          # views of the buffer that gives way (and what was made of them)
             buf = torch.empty((cap, cols), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-            self.generation += 1
-            self._views.clear()                              # views of the buffer that gave way (and what was made of them)
+            self.allocations += 1
         if len(self._views) > 4096:
             self._views.clear()
         view = self._views[vkey] = buf[:rows]
@@ -112,9 +116,11 @@ class Workspace:
         key = ("zeros:" + name, 0, dtype)
         buf = self._buffers.get(key)
         if buf is None or buf.numel() < n:
+            if buf is not None:
+                self.generation += 1
             buf = torch.zeros(max(n, 1024 if buf is None else 2 * buf.numel()), dtype=dtype, device=self.device)
             self._buffers[key] = buf
-            self.generation += 1
+            self.allocations += 1
         return buf[:n]
 
 

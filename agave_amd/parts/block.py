@@ -19,7 +19,10 @@ import torch
 from ..config.spec import LayerSpec
 from ..weights.loader import TensorNeed
 from .base import BuildEnv, lookup, register
-from .norm import Pending, add_branch, rows_as_they_are
+from .norm import NormedRows, Pending, add_branch, rows_as_they_are
+
+
+NORMED_ROWS_AS_A_PROMISE = 1        # up to this many rows a sublayer may make its normalised input itself
 
 
 def add_pending_and_norm(h: torch.Tensor, pending: Pending, norm, out: Optional[torch.Tensor],
@@ -70,6 +73,8 @@ class SandwichBlock:
 
     def forward(self, h: torch.Tensor, pending: Pending, step, memory: int, writes: bool) -> Pending:
         n = h.shape[0]
+        if n <= NORMED_ROWS_AS_A_PROMISE:
+            return self._forward_few_rows(h, pending, step, memory, writes)
         x = self.env.workspace.get("normed", n, self.hidden, self.env.dtype)
         self.pre_mixer.add_and_norm(h, pending, x)
         a = self.mixer.forward(x, step, memory, writes)
@@ -79,6 +84,24 @@ class SandwichBlock:
         self.pre_ffn.add_and_norm(h, pending, x)
         f = self.ffn.forward(x, step)
         return (f, self.post_ffn)
+
+    def _forward_few_rows(self, h: torch.Tensor, pending: Pending, step, memory: int, writes: bool) -> Pending:
+        """One row (a decode step of one sequence): a sublayer that says so is handed the normalised
+        row as a promise, so that its first product can make it in its own kernel (two kernels a
+        layer less, of seven that each cost their start and their end)."""
+        ws, dtype = self.env.workspace, self.env.dtype
+        x = NormedRows(h, pending, self.pre_mixer, ws, dtype)
+        a = self.mixer.forward(x if getattr(self.mixer, "takes_rows_to_be_normed", False) else x.rows(), step, memory, writes)
+        if not x.taken:
+            raise RuntimeError(f"{type(self.mixer).__name__} was handed rows to be normalised and never took them")
+        pending = (a, self.post_mixer, x.base)
+        if self.ffn is None:
+            return pending
+        x = NormedRows(h, pending, self.pre_ffn, ws, dtype)
+        f = self.ffn.forward(x if getattr(self.ffn, "takes_rows_to_be_normed", False) else x.rows(), step)
+        if not x.taken:
+            raise RuntimeError(f"{type(self.ffn).__name__} was handed rows to be normalised and never took them")
+        return (f, self.post_ffn, x.base)
 
 
 class PreNormBlock(SandwichBlock):

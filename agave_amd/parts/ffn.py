@@ -26,6 +26,7 @@ FUSED_ACTIVATION = "gelu_tanh"          # the one that the matrix-core products 
 
 class GatedFfn:
     prompt_steps_can_be_recorded = True        # a multi-token step is the same launches whatever its tokens are
+    takes_rows_to_be_normed = True             # its first product may make the normalised rows itself (NormedRows)
 
     def __init__(self, spec: GatedFfnSpec, weights, env: BuildEnv):
         if spec.activation not in kernels.GATE_ACTIVATIONS:

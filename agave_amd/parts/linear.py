@@ -15,6 +15,7 @@ import torch
 
 from ..ops import gemm, gemm_mfma, kernels, library
 from .base import BuildEnv
+from .norm import NormedRows
 
 
 class Linear:
@@ -72,6 +73,11 @@ class Linear:
         """``slices_ok``: the caller also takes a float32 [slices, n, out] tensor whose slices add
         up to the product (a norm that adds a branch to the residual stream does); a product
         with few rows of W and many columns is then shared out along the columns."""
+        if isinstance(x, NormedRows):
+            made = self._forward_normed(x, out, tag, 0) if not self.interleave_ff else None
+            if made is not None:
+                return made
+            x = x.rows()
         n = x.shape[0]
         if slices_ok and out is None and self.packed is not None and not self.interleave_ff:
             many = n > gemm_mfma.SKINNY_MAX_M
@@ -115,10 +121,37 @@ class Linear:
         library.profile.label = None
         return out
 
-    def forward_geglu(self, x: torch.Tensor, out: torch.Tensor) -> bool:
+    def _forward_normed(self, x: NormedRows, out: Optional[torch.Tensor], tag: Optional[str], epilogue: int):
+        """The product of rows that are still a promise, made inside the product's kernel if the
+        kernel library has one for these sizes and both norms are RMS norms; None otherwise."""
+        n, k = x.shape
+        n_out = self.interleave_ff if epilogue else self.out_features
+        if self.packed is None or x.dtype != torch.bfloat16 or k != self.in_features or (out is not None and out.dtype != torch.bfloat16):
+            return None
+        if not gemm_mfma.normed_ok(n, n_out, k, epilogue):
+            return None
+        args = x.rms_arguments()
+        if args is None:
+            return None
+        h_in, h_out, branch, post_gain, post_eps, pre_gain, pre_eps = args
+        if out is None:
+            out = self.env.workspace.get(tag or self.name, n, n_out, torch.bfloat16)
+        library.profile.label = self.name
+        gemm_mfma.row_normed(h_in, h_out, branch, post_gain, post_eps, pre_gain, pre_eps, self.packed, out, n_out, epilogue)
+        x.made_by_consumer(h_in, h_out)
+        if self.bias is not None:
+            kernels.add_bias(out, self.bias)
+        library.profile.label = None
+        return out
+
+    def forward_geglu(self, x, out: torch.Tensor) -> bool:
         """out = gelu_tanh(gate x) * (up x) in one kernel, if the weight was packed for it."""
         if not self.interleave_ff:
             return False
+        if isinstance(x, NormedRows):
+            if self._forward_normed(x, out, None, 1) is not None:
+                return True
+            x = x.rows()
         library.profile.label = self.name
         gemm_mfma.product(x, self.packed, out, self.interleave_ff, epilogue=1)
         library.profile.label = None

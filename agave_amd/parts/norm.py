@@ -24,19 +24,84 @@ from ..ops import kernels
 from ..weights.loader import TensorNeed
 from .base import BuildEnv, register
 
-Pending = Optional[Tuple[torch.Tensor, Optional[object]]]     # (branch, the norm after its sublayer | None)
+# (branch, the norm after its sublayer | None[, base]).  ``base``: the tensor that holds the residual
+# stream at this moment if that is not ``h`` (a product that made its own normalised rows summed the
+# stream up in other memory, see NormedRows); whoever adds the branch reads the rows there and
+# writes them to ``h``.
+Pending = Optional[Tuple]
+
+
+def unpack_pending(pending: Pending):
+    """(branch, post norm, base), each None where there is none."""
+    if pending is None:
+        return None, None, None
+    if len(pending) == 2:
+        return pending[0], pending[1], None
+    return pending
 
 
 def add_branch(h: torch.Tensor, pending: Pending) -> None:
     """h += post(branch) for a branch that is still to be added (post None: h += branch).  The
     branch may be 32-bit slices [slices, rows, hidden] that add up to it."""
-    if pending is None:
+    branch, post, base = unpack_pending(pending)
+    if branch is None:
+        if base is not None:
+            h.copy_(base)
         return
-    branch, post = pending
     if post is None:
-        kernels.residual_norm(h, branch, None, 0.0, None, None, 0.0)
+        kernels.residual_norm(h, branch, None, 0.0, None, None, 0.0, src=base)
     else:
+        if base is not None:
+            h.copy_(base)
         post.add_to(h, branch)
+
+
+class NormedRows:
+    """``norm(h + post(branch))`` as a promise: the rows that a sublayer is given, not yet computed.
+
+    Whoever takes them either calls :meth:`rows` (the norm's kernel runs, ``h`` holds the sum, and
+    the rows come back as a tensor), or, being a product that can make them in its own kernel,
+    takes :meth:`rms_arguments` and reports with :meth:`made_by_consumer` where it left the sum
+    (it cannot write ``h`` in place: its other workgroups still read it).  ``shape`` and ``dtype``
+    are those of the rows to be."""
+
+    def __init__(self, h: torch.Tensor, pending: Pending, norm, workspace, dtype: torch.dtype):
+        self.h, self.pending, self.norm = h, pending, norm
+        self.workspace = workspace
+        self.shape, self.dtype = h.shape, dtype
+        self.base: Optional[torch.Tensor] = None      # afterwards: where the stream is, if not in h
+        self._rows: Optional[torch.Tensor] = None
+        self.taken = False
+
+    def rows(self) -> torch.Tensor:
+        if self._rows is None:
+            if self.taken:
+                raise RuntimeError("these rows were made inside a product's kernel and exist nowhere else")
+            x = self.workspace.get("normed", self.shape[0], self.shape[1], self.dtype)
+            self.norm.add_and_norm(self.h, self.pending, x)
+            self._rows, self.taken = x, True
+        return self._rows
+
+    def rms_arguments(self):
+        """(h_in, h_out, branch, post_gain, post_eps, pre_gain, pre_eps) if nothing was computed yet and
+        both norms are RMS norms (the one on the branch may be absent), else None."""
+        if self.taken:
+            return None
+        branch, post, base = unpack_pending(self.pending)
+        if not isinstance(self.norm, RmsNorm) or (post is not None and not isinstance(post, RmsNorm)):
+            return None
+        h_in = base if base is not None else self.h
+        h_out = None
+        if branch is not None:
+            h_out = self.h if base is not None else self.workspace.get("residual_aside", self.shape[0], self.shape[1],
+                                                                       torch.float32)
+        return (h_in, h_out, branch, post.gain if (branch is not None and post is not None) else None,
+                post.eps if (branch is not None and post is not None) else 0.0, self.norm.gain, self.norm.eps)
+
+    def made_by_consumer(self, h_in: torch.Tensor, h_out: Optional[torch.Tensor]) -> None:
+        self.taken = True
+        now = h_out if h_out is not None else h_in
+        self.base = None if now is self.h or now.data_ptr() == self.h.data_ptr() else now
 
 
 def rows_as_they_are(h: torch.Tensor, pending: Pending, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
@@ -91,18 +156,20 @@ class RmsNorm(Norm):
     def add_and_norm(self, h, pending, out, rows=None) -> None:
         """One kernel adds the branch (through the RMS norm after its sublayer, if it has one) and
         computes this norm, reading and writing ``h`` once."""
-        branch, post = pending if pending is not None else (None, None)
+        branch, post, base = unpack_pending(pending)
         if branch is not None and post is not None and not isinstance(post, RmsNorm):
-            post.add_to(h, branch)              # another kind of norm after the sublayer: its own kernel
-            branch = post = None
-        if rows is not None and branch is not None:
-            add_branch(h, (branch, post))       # the fused kernel gathers rows only without a branch
-            branch = post = None
+            add_branch(h, (branch, post, base))     # another kind of norm after the sublayer: its own kernel
+            branch = post = base = None
+        if rows is not None and (branch is not None or base is not None):
+            add_branch(h, (branch, post, base))     # the fused kernel gathers rows only without a branch
+            branch = post = base = None
         if branch is None and out is None:
+            add_branch(h, (None, None, base))
             return
         kernels.residual_norm(h, branch, post.gain if (branch is not None and post) else None,
                               post.eps if (branch is not None and post) else 0.0,
-                              out, self.gain if out is not None else None, self.eps if out is not None else 0.0, rows)
+                              out, self.gain if out is not None else None, self.eps if out is not None else 0.0, rows,
+                              src=base)
 
 
 register("norm", "rmsnorm", RmsNorm)

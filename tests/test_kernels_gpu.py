@@ -71,6 +71,38 @@ def test_residual_norm(K, dtype, e):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("e", [100, 2560, 20000])
+def test_residual_norm_reads_the_stream_elsewhere(K, dtype, e):
+    """``src``: the residual rows are read from another tensor and written to h, with a branch, with
+    slices, with a norm only and with nothing else to do (both kernels: 20,000 columns are too many
+    for the one that holds a row in registers)."""
+    n = 4
+    src = torch.randn(n, e) * 3
+    br = (torch.randn(n, e) * 0.3).to(dtype)
+    parts = torch.randn(3, n, e) * 0.3
+    gp, gq = torch.randn(e) * 0.1 + 1, torch.randn(e) * 0.1 + 1
+    for branch, b_sum in ((br, br.double()), (parts, parts.double().sum(0)), (None, None)):
+        h = torch.full((n, e), 9.0, device=DEV)
+        s_dev = src.clone().to(DEV)
+        out = torch.empty(n, e, dtype=dtype, device=DEV)
+        K.residual_norm(h, branch.to(DEV) if branch is not None else None, gp.to(DEV) if branch is not None else None, 1e-5,
+                        out, gq.to(DEV), 3e-6, src=s_dev)
+        h_ref = src.double() + (P.rms_norm(b_sum, gp.double(), 1e-5, add_one=False) if b_sum is not None else 0.0)
+        assert torch.allclose(h.cpu().double(), h_ref, atol=3e-6, rtol=1e-6)
+        assert torch.allclose(out.cpu().double(), P.rms_norm(h_ref, gq.double(), 3e-6, add_one=False), **_tol(dtype))
+        assert torch.equal(s_dev.cpu(), src)
+    h = torch.full((n, e), 9.0, device=DEV)
+    K.residual_norm(h, br.to(DEV), None, 0.0, None, None, 0.0, src=src.to(DEV))         # a plain add
+    assert torch.allclose(h.cpu().double(), src.double() + br.double(), atol=1e-6)
+    K.residual_norm(h, None, None, 0.0, None, None, 0.0, src=src.to(DEV))               # nothing but the move
+    assert torch.equal(h.cpu(), src)
+    with pytest.raises(ValueError):
+        K.residual_norm(h, None, None, 0.0, None, None, 0.0, src=h)
+    with pytest.raises(ValueError):
+        K.residual_norm(h, None, None, 0.0, torch.empty(1, e, dtype=dtype, device=DEV), gq.to(DEV), 1e-6, _i32([1]), src=src.to(DEV))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("e", [72, 2560, 5000])
 def test_residual_norm_takes_a_branch_in_slices(K, dtype, e):
     """A float32 [slices, rows, hidden] branch stands for the sum of its slices: the same residual
@@ -549,6 +581,76 @@ def test_gemm_skinny_in_slices(G, m, n, k, slices):
     with pytest.raises(ValueError):
         G.skinny_slices(x.to(DEV), packed, out.bfloat16(), n)
     assert G.slices_for(8, 2560, 10240) > 1 and G.slices_for(8, 10240, 2560) == 1 and G.slices_for(65, 2560, 10240) == 1
+
+
+@pytest.mark.parametrize("m,n,k,epi", [(1, 4096, 2560, 0), (1, 10240, 2560, 1), (1, 1000, 5376, 1), (1, 53, 200, 0),
+                                       (1, 40, 72, 1), (1, 130, 3080, 0), (1, 96, 6144, 0), (1, 8192, 3840, 0),
+                                       (1, 21504, 5376, 1), (1, 4100, 4104, 0), (1, 40000, 64, 0)])
+@pytest.mark.parametrize("branch", ["none", "bf16", "f32", "slices", "slices_unnormed", "slices11"])
+def test_product_of_one_token_that_makes_its_own_normalised_row(G, m, n, k, epi, branch):
+    """out = rmsnorm(h + post(branch)) W^T (or its GeGLU) for one row, h + post(branch) going
+    to other memory: against the same written out in 64-bit, with the normalised rows rounded to
+    bfloat16 as the kernel rounds them.  The gains differ per column and the branch is large against
+    h, so that a gain or a norm left out, or applied in the wrong place, shows; memory beside the
+    outputs must stay as it was."""
+    assert G.normed_ok(m, n, k, epi)
+    g = torch.Generator().manual_seed(m * 7 + n + k + len(branch))
+    h = torch.randn(m, k, generator=g) * 2
+    pre_gain, post_gain = torch.rand(k, generator=g) + 0.5, torch.rand(k, generator=g) * 2 + 0.5
+    pre_eps, post_eps = 1e-3, 0.5
+    rows = 2 * n if epi else n
+    w = (torch.randn(rows, k, generator=g) * 0.1).bfloat16()
+    packed = G.pack_weight(w.to(DEV), interleave_ff=n if epi else 0)
+    b = b_sum = None
+    if branch == "bf16":
+        b = (torch.randn(m, k, generator=g) * 5).bfloat16()
+        b_sum = b.double()
+    elif branch == "f32":
+        b = torch.randn(m, k, generator=g) * 5
+        b_sum = b.double()
+    elif branch.startswith("slices"):
+        b = torch.randn(11 if branch == "slices11" else 5, m, k, generator=g) * 3      # (two are asked for ahead, the others follow)
+        b_sum = b.double().sum(0)
+    with_post = branch not in ("none", "slices_unnormed")
+    hd = h.double()
+    if b_sum is not None:
+        if with_post:
+            hd = hd + b_sum / torch.sqrt((b_sum * b_sum).mean(-1, keepdim=True) + post_eps) * post_gain.double()
+        else:
+            hd = hd + b_sum
+    x = (hd / torch.sqrt((hd * hd).mean(-1, keepdim=True) + pre_eps) * pre_gain.double()).bfloat16().double()
+    y = x @ w.double().T
+    ref = P.gelu_tanh(y[:, :n]) * y[:, n:] if epi else y
+
+    h_dev = h.to(DEV)
+    h_out = torch.full((m + 1, k), 7.0, device=DEV)
+    out = torch.full((m + 1, n), float("nan"), dtype=torch.bfloat16, device=DEV)
+    G.row_normed(h_dev, h_out[:m] if b is not None else None, b.to(DEV) if b is not None else None,
+                    post_gain.to(DEV) if with_post else None, post_eps, pre_gain.to(DEV), pre_eps, packed, out[:m], n, epi)
+    scale = float(ref.abs().max())
+    assert float((out[:m].cpu().double() - ref).abs().max()) <= 8e-3 * scale
+    assert torch.equal(h_dev.cpu(), h), "the rows that were read are not touched"
+    if b is not None:
+        assert float((h_out[:m].cpu().double() - hd).abs().max()) <= 2e-5 * float(hd.abs().max())
+    else:
+        assert float(h_out[:m].min()) == 7.0
+    assert float(h_out[m].min()) == 7.0 and float(h_out[m].max()) == 7.0 and bool(torch.isnan(out[m].float()).all())
+
+
+def test_product_of_one_token_refuses_what_it_cannot_do(G):
+    assert not G.normed_ok(2, 4096, 2560, 0) and not G.normed_ok(1, 4096, 6152, 0) and not G.normed_ok(1, 4096, 2564, 0)
+    assert not G.normed_ok(1, 262208, 2560, 0)            # (a workgroup would take more row blocks than its LDS holds sums for)
+    k, n = 64, 32
+    w = G.pack_weight(torch.zeros(n, k, dtype=torch.bfloat16, device=DEV))
+    h = torch.zeros(1, k, device=DEV)
+    gain = torch.ones(k, device=DEV)
+    out = torch.empty(1, n, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError, match="of its own"):
+        G.row_normed(h, h, torch.zeros(1, k, device=DEV), None, 0.0, gain, 1e-6, w, out, n)      # the sum in place
+    with pytest.raises(ValueError):
+        G.row_normed(torch.zeros(3, k, device=DEV), None, None, None, 0.0, gain, 1e-6, w, torch.empty(3, n, dtype=torch.bfloat16, device=DEV), n)
+    with pytest.raises(ValueError):
+        G.row_normed(h, None, None, None, 0.0, gain, 1e-6, w, out.float(), n)
 
 
 def test_product_of_many_shapes(G):
