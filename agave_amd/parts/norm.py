@@ -50,6 +50,8 @@ def add_branch(h: torch.Tensor, pending: Pending) -> None:
         return
     if post is None:
         kernels.residual_norm(h, branch, None, 0.0, None, None, 0.0, src=base)
+    elif isinstance(post, RmsNorm):
+        kernels.residual_norm(h, branch, post.gain, post.eps, None, None, 0.0, src=base)
     else:
         if base is not None:
             h.copy_(base)
