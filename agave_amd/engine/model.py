@@ -102,7 +102,9 @@ class Model:
         if step.n_want == 0:
             return None
         x = ws.get("final_normed", step.n_want, self.spec.hidden, self.env.dtype)
-        add_pending_and_norm(h, pending, self.final_norm, x, rows=step.want_rows)   # no final norm: the rows as they are
+        # (a decode step wants every row, in order: no gather, and the last branch is added in the norm's kernel)
+        rows = None if (step.is_decode and step.n_want == n) else step.want_rows
+        add_pending_and_norm(h, pending, self.final_norm, x, rows=rows)   # no final norm: the rows as they are
         logits = ws.get("logits", step.n_want, self.spec.vocab_size, torch.float32)
         self.head.forward(x, out=logits)
         if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0.0:
