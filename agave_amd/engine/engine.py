@@ -57,7 +57,7 @@ class Engine:
     def __init__(self, spec: ModelSpec, weights, *, dtype="bfloat16", max_slots: int = 8,
                  max_context: Optional[int] = None, cache_tokens: Optional[int] = None,
                  prefill_piece: Optional[int] = None, keep_stored_precision: bool = True, device=None,
-                 config=None):
+                 config=None, will_sample: bool = True):
         """``max_context``: longest sequence a slot may hold; None: the smaller of the model's
         context and 4096, 0: the model's whole context (the reference's ``--ctx-size``,
         ``src/main.zig:1100-1113``, ``src/models/gemma3.zig:164-166``).
@@ -70,7 +70,9 @@ class Engine:
         ``keep_stored_precision``: in a bfloat16 engine a matrix that the checkpoint stores in
         32-bit stays in 32-bit (its products then run on the plain multiply-add kernel, far from
         the matrix cores' speed; a line on standard error says how many do); False casts such
-        matrices to bfloat16 at load.  Half precision is always cast to the engine's type."""
+        matrices to bfloat16 at load.  Half precision is always cast to the engine's type.
+        ``will_sample`` False: the sampling kernels are not built with the others at construction (a
+        caller that only reads logits never needs them; they would still be built at first use)."""
         self.device = require_gpu(device)
         self.dtype = parse_dtype(dtype)
         self._cancel = threading.Event()
@@ -80,7 +82,9 @@ class Engine:
         # what this element type needs is compiled now, side by side, rather than one library
         # after the other as the first step meets them (a fresh checkout's first run)
         from ..ops import library
-        needed = ["elementwise", "gemm", "attention_plain", "sampling"]
+        needed = ["elementwise", "gemm", "attention_plain"]
+        if will_sample:                    # (a caller that only wants logits, like trace replay, builds no sampling kernels)
+            needed.append("sampling")
         if self.dtype == torch.bfloat16:
             needed += ["gemm_mfma", "attention_mfma"]
         library.ensure_built(needed)

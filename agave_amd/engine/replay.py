@@ -103,7 +103,7 @@ class Replay:
         pages = (int(max_tokens) + PAGE - 1) // PAGE
         # every live request holds at least one page, so there are never more requests than pages
         self.engine = Engine.from_folder(model_dir, dtype=dtype, max_slots=pages,
-                                         max_context=pages * PAGE, cache_tokens=pages * PAGE)
+                                         max_context=pages * PAGE, cache_tokens=pages * PAGE, will_sample=False)
         self.slot_of: Dict[str, int] = {}
 
     def run_step(self, entries: Sequence[dict], end: Sequence[str]) -> Optional[np.ndarray]:
