@@ -585,8 +585,9 @@ def test_gemm_skinny_in_slices(G, m, n, k, slices):
 
 @pytest.mark.parametrize("m,n,k,epi", [(1, 4096, 2560, 0), (1, 10240, 2560, 1), (1, 1000, 5376, 1), (1, 53, 200, 0),
                                        (1, 40, 72, 1), (1, 130, 3080, 0), (1, 96, 6144, 0), (1, 8192, 3840, 0),
-                                       (1, 21504, 5376, 1), (1, 4100, 4104, 0), (1, 40000, 64, 0)])
-@pytest.mark.parametrize("branch", ["none", "bf16", "f32", "slices", "slices_unnormed", "slices11"])
+                                       (1, 21504, 5376, 1), (1, 4100, 4104, 0), (1, 40000, 64, 0), (1, 36, 72, 1),
+                                       (1, 21, 40, 0)])
+@pytest.mark.parametrize("branch", ["none", "bf16", "f32", "slices", "slices_unnormed", "slices11", "slices2"])
 def test_product_of_one_token_that_makes_its_own_normalised_row(G, m, n, k, epi, branch):
     """out = rmsnorm(h + post(branch)) W^T (or its GeGLU) for one row, h + post(branch) going
     to other memory: against the same written out in 64-bit, with the normalised rows rounded to
@@ -609,7 +610,8 @@ def test_product_of_one_token_that_makes_its_own_normalised_row(G, m, n, k, epi,
         b = torch.randn(m, k, generator=g) * 5
         b_sum = b.double()
     elif branch.startswith("slices"):
-        b = torch.randn(11 if branch == "slices11" else 5, m, k, generator=g) * 3      # (two are asked for ahead, the others follow)
+        # (two slices are asked for ahead of the weights, or eight when there are more than two; others follow)
+        b = torch.randn({"slices11": 11, "slices2": 2}.get(branch, 5), m, k, generator=g) * 3
         b_sum = b.double().sum(0)
     with_post = branch not in ("none", "slices_unnormed")
     hd = h.double()
