@@ -5,9 +5,9 @@ from .attention import Attention
 from .block import PreNormBlock, SandwichBlock, add_pending_and_norm
 from .ffn import GatedFfn
 from .linear import Linear
-from .norm import Norm, RmsNorm, add_branch
+from .norm import Norm, NormedRows, RmsNorm, add_branch
 from .position import NoPosition, RotaryPosition
 
 __all__ = ["BuildEnv", "Workspace", "lookup", "part_tensors", "register", "registered", "Attention", "GatedFfn",
-           "Linear", "Norm", "RmsNorm", "add_branch", "RotaryPosition", "NoPosition", "SandwichBlock", "PreNormBlock",
+           "Linear", "Norm", "NormedRows", "RmsNorm", "add_branch", "RotaryPosition", "NoPosition", "SandwichBlock", "PreNormBlock",
            "add_pending_and_norm"]

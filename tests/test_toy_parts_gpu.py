@@ -43,7 +43,10 @@ def define_and_register():
         out_proj: str = ""
 
     class DecayMixer:
-        """s_t = sigmoid(d) * s_{t-1} + x_t ;  y_t = W s_t.  The state s is kept per sequence."""
+        """s_t = sigmoid(d) * s_{t-1} + x_t ;  y_t = W s_t.  The state s is kept per sequence.
+        It says that it takes the normalised rows as a promise (a step of one row hands it a
+        ``NormedRows``) and asks for the tensor itself, as a part from outside may."""
+        takes_rows_to_be_normed = True
 
         def __init__(self, spec, weights, env):
             self.a = torch.sigmoid(weights.get(spec.decay).float().to(env.device))
@@ -61,6 +64,10 @@ def define_and_register():
             return StateNeed((self.spec.hidden,), torch.float32)
 
         def forward(self, x, step, memory, writes=True):
+            from agave_amd.parts import NormedRows
+            if isinstance(x, NormedRows):
+                assert x.shape[0] == 1 and not x.taken
+                x = x.rows()
             state = step.cache.state[memory]
             xf = x.float()
             if step.is_decode:                       # device indices only: the step may be a graph replay
