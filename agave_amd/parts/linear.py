@@ -74,7 +74,8 @@ class Linear:
         up to the product (a norm that adds a branch to the residual stream does); a product
         with few rows of W and many columns is then shared out along the columns."""
         if isinstance(x, NormedRows):
-            made = self._forward_normed(x, out, tag, 0) if not self.interleave_ff else None
+            plain = not self.interleave_ff and out_dtype in (None, torch.bfloat16)
+            made = self._forward_normed(x, out, tag, 0) if plain else None
             if made is not None:
                 return made
             x = x.rows()
